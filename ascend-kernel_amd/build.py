@@ -1,0 +1,92 @@
+"""Builds the gfx950 binaries of this package, in-tree.
+
+  libmoe_gfx950.so          HIP kernels + the C ABI declared in include/moe_gfx950.h
+  cinfer_ascendc.*.so       pybind11/torch module with the reference's Python API
+
+Run as `python ascend-kernel_amd/build.py [--no-ext]`; hipcc cross-compiles for
+gfx950 without a GPU.
+"""
+from __future__ import annotations
+
+import argparse
+import os
+import subprocess
+import sys
+import sysconfig
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(HERE)
+CSRC = os.path.join(HERE, "csrc")
+LIB = os.path.join(HERE, "libmoe_gfx950.so")
+KERNEL_SOURCES = ["moe_abi.cpp", "moe_dequant.hip", "moe_gemv.hip", "moe_gemm.hip"]
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+# -packed-fp32-ops off: the compiler must not form v_pk_*_f32 from scalar float code
+HIP_FLAGS = ["-O3", "--offload-arch=gfx950", "-std=c++17", "-fPIC", "-Xclang", "-target-feature", "-Xclang",
+             "-packed-fp32-ops", "-Wall", "-Wno-unused-function"]
+
+
+def ext_path() -> str:
+    return os.path.join(HERE, "cinfer_ascendc" + sysconfig.get_config_var("EXT_SUFFIX"))
+
+
+def _run(cmd):
+    print("+", " ".join(cmd), flush=True)
+    subprocess.check_call(cmd)
+
+
+def build_kernels(jobs: int = 4) -> str:
+    objs, procs = [], []
+    os.makedirs(os.path.join(HERE, "build"), exist_ok=True)
+    for src in KERNEL_SOURCES:
+        obj = os.path.join(HERE, "build", src + ".o")
+        cmd = [HIPCC, *HIP_FLAGS, "-x", "hip", "-I", os.path.join(ROOT, "include"), "-I", CSRC, "-c",
+               os.path.join(CSRC, src), "-o", obj]
+        print("+", " ".join(cmd), flush=True)
+        procs.append((src, subprocess.Popen(cmd, stderr=subprocess.PIPE, text=True)))
+        objs.append(obj)
+        if len(procs) >= jobs:
+            _wait(procs)
+    _wait(procs)
+    _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", LIB])
+    return LIB
+
+
+def _wait(procs):
+    for src, p in procs:
+        _, err = p.communicate()
+        err = "\n".join(l for l in err.splitlines() if "packed-fp32-ops" not in l)
+        if err.strip():
+            print(err, file=sys.stderr)
+        if p.returncode:
+            raise RuntimeError(f"hipcc failed on {src}")
+    procs.clear()
+
+
+def build_extension() -> str:
+    import pybind11  # noqa: F401
+    from torch.utils import cpp_extension as ce
+
+    out = ext_path()
+    inc = [f"-I{p}" for p in ce.include_paths()] + [f"-I{sysconfig.get_paths()['include']}",
+                                                    f"-I{os.path.join(ROOT, 'include')}", "-I/opt/rocm/include"]
+    libdirs = ce.library_paths()
+    cmd = ["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1",
+           "-DTORCH_EXTENSION_NAME=cinfer_ascendc", "-D_GLIBCXX_USE_CXX11_ABI=1", *inc,
+           os.path.join(CSRC, "cinfer_ascendc.cpp"), "-o", out, f"-L{HERE}", "-lmoe_gfx950",
+           *[f"-L{d}" for d in libdirs], "-lc10", "-lc10_hip", "-ltorch_cpu", "-ltorch", "-ltorch_python",
+           "-Wl,-rpath,$ORIGIN", *[f"-Wl,-rpath,{d}" for d in libdirs]]
+    _run(cmd)
+    return out
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--no-ext", action="store_true", help="skip the torch/pybind11 module")
+    args = ap.parse_args()
+    build_kernels()
+    if not args.no_ext:
+        build_extension()
+
+
+if __name__ == "__main__":
+    main()

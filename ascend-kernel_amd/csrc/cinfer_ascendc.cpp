@@ -1,0 +1,183 @@
+// Python module `cinfer_ascendc`: same functions, keyword names and argument order as
+// the reference's pybind module (pybind.cpp:13-19), on top of the C ABI of
+// libmoe_gfx950.so.  This file is host glue only: argument checks, the current HIP
+// stream, and the translation of at::Tensor into raw pointers and sizes.
+//
+// Differences from the reference adapters (grouped_gemm/src/grouped_gemm.cpp:122-161,
+// grouped_soft_gemv/src/grouped_soft_gemv.cpp:123-155): shapes, dtypes, devices and
+// contiguity are validated before the launch; no workspace is allocated or cached;
+// computeType accepts "int8", "int4", "fp4_b32" and "bf16" besides "fp4" and "fp8";
+// dequant_fp4 is an extra entry point.  Every failure raises RuntimeError, as the
+// reference does.
+#include <c10/core/DeviceGuard.h>
+#include <c10/hip/HIPStream.h>
+#include <torch/extension.h>
+
+#include <stdexcept>
+#include <string>
+
+#include "moe_gfx950.h"
+
+namespace {
+
+[[noreturn]] void fail(const std::string& what) { throw std::runtime_error("cinfer_ascendc: " + what); }
+
+void check_status(int rc, const char* op) {
+    if (rc != MOE_OK) fail(std::string(op) + ": " + moe_strerror(rc));
+}
+
+void check_tensor(const at::Tensor& t, const char* name, at::ScalarType dtype, int64_t dim, const at::Tensor& like) {
+    if (!t.defined()) fail(std::string(name) + " is undefined");
+    if (!t.is_cuda()) fail(std::string(name) + " must be on the GPU");
+    if (t.device() != like.device()) fail(std::string(name) + " is on a different device than x");
+    if (t.scalar_type() != dtype) fail(std::string(name) + " has dtype " + c10::toString(t.scalar_type()) +
+                                       ", expected " + c10::toString(dtype));
+    if (t.dim() != dim) fail(std::string(name) + " must have " + std::to_string(dim) + " dimensions");
+    if (!t.is_contiguous()) fail(std::string(name) + " must be contiguous");
+}
+
+int parse_format(const char* computeType) {
+    const int fmt = moe_format_from_compute_type(computeType);
+    if (fmt < 0)
+        fail(std::string("Invalid compute type: ") + (computeType ? computeType : "(null)") +
+             ". Supported: \"fp4\", \"fp8\", \"int8\", \"int4\", \"fp4_b32\", \"bf16\"");
+    return fmt;
+}
+
+// Fills args from the tensors; returns the logical (K, N) through args.
+void fill_grouped(moe_grouped_args& a, const at::Tensor& x, const at::Tensor& weight, const at::Tensor& scale,
+                  const at::Tensor* offset, const at::Tensor& groupList, int fmt, const at::Tensor& output) {
+    if (!x.defined() || !x.is_cuda()) fail("x must be a GPU tensor");
+    check_tensor(x, "x", at::kBFloat16, 2, x);
+    check_tensor(output, "output", at::kBFloat16, 2, x);
+    check_tensor(groupList, "groupList", at::kLong, 1, x);
+    const int64_t M = x.size(0), K = x.size(1), G = groupList.size(0);
+    int64_t N = 0, scale_rows = 1;
+    auto want = [&](const at::Tensor& t, const char* name, std::initializer_list<int64_t> shape) {
+        if (t.sizes() != at::IntArrayRef(shape)) {
+            std::string s = std::string(name) + " has shape [";
+            for (auto d : t.sizes()) s += std::to_string(d) + ",";
+            s += "], expected [";
+            for (auto d : shape) s += std::to_string(d) + ",";
+            fail(s + "]");
+        }
+    };
+    switch (fmt) {
+        case MOE_FMT_FP4_REF:
+            // int8 [G, K, N/2] (grouped_gemm/src/grouped_gemm.cpp:134-135 re-describes it as INT4 [G, K, N])
+            check_tensor(weight, "weight", at::kChar, 3, x);
+            N = weight.size(2) * 2;
+            want(weight, "weight", {G, K, N / 2});
+            check_tensor(scale, "scale", at::kBFloat16, 3, x);
+            want(scale, "scale", {G, K / 16, N});
+            scale_rows = K / 16;
+            break;
+        case MOE_FMT_FP8_REF:
+            check_tensor(weight, "weight", at::kByte, 3, x);
+            N = weight.size(2);
+            want(weight, "weight", {G, K, N});
+            check_tensor(scale, "scale", at::kFloat, 3, x);
+            want(scale, "scale", {G, (K + 127) / 128, (N + 127) / 128});
+            break;
+        case MOE_FMT_INT8:
+            check_tensor(weight, "weight", at::kChar, 3, x);
+            N = weight.size(2);
+            want(weight, "weight", {G, K, N});
+            check_tensor(scale, "scale", at::kBFloat16, 2, x);
+            want(scale, "scale", {G, N});
+            if (!offset) fail("computeType \"int8\" needs an offset tensor");
+            check_tensor(*offset, "offset", at::kBFloat16, 2, x);
+            want(*offset, "offset", {G, N});
+            break;
+        case MOE_FMT_INT4:
+            if (weight.defined() && weight.scalar_type() == at::kChar)
+                check_tensor(weight, "weight", at::kChar, 3, x);
+            else
+                check_tensor(weight, "weight", at::kByte, 3, x);
+            N = weight.size(2) * 2;
+            want(weight, "weight", {G, K, N / 2});
+            check_tensor(scale, "scale", at::kBFloat16, 3, x);
+            scale_rows = scale.size(1);
+            want(scale, "scale", {G, scale_rows, N});
+            break;
+        case MOE_FMT_FP4_B32:
+            check_tensor(weight, "weight", at::kByte, 3, x);
+            N = weight.size(1);
+            want(weight, "weight", {G, N, K / 2});
+            check_tensor(scale, "scale", at::kBFloat16, 3, x);
+            want(scale, "scale", {G, N, K / 32});
+            break;
+        default:  // MOE_FMT_BF16
+            check_tensor(weight, "weight", at::kBFloat16, 3, x);
+            N = weight.size(1);
+            want(weight, "weight", {G, N, K});
+            break;
+    }
+    want(output, "output", {M, N});
+    a.x = x.data_ptr();
+    a.weight = weight.data_ptr();
+    a.scale = fmt == MOE_FMT_BF16 ? nullptr : scale.data_ptr();
+    a.offset = (fmt == MOE_FMT_INT8 && offset) ? offset->data_ptr() : nullptr;
+    a.group_list = groupList.data_ptr<int64_t>();
+    a.y = output.data_ptr();
+    a.M = M; a.K = K; a.N = N; a.G = G;
+    a.scale_rows = scale_rows;
+    a.format = fmt;
+    a.reserved = 0;
+}
+
+moe_stream_t current_stream(const at::Tensor& x) {
+    return static_cast<moe_stream_t>(c10::hip::getCurrentHIPStream(x.device().index()).stream());
+}
+
+// pybind.cpp:17-19
+void GroupedGemm(at::Tensor x, at::Tensor weight, at::Tensor antiquantScaleOptional,
+                 at::Tensor antiquantOffsetOptional, at::Tensor groupListOptional, const char* computeType,
+                 at::Tensor output) {
+    const int fmt = parse_format(computeType);
+    moe_grouped_args a;
+    fill_grouped(a, x, weight, antiquantScaleOptional, &antiquantOffsetOptional, groupListOptional, fmt, output);
+    c10::DeviceGuard guard(x.device());
+    check_status(moe_grouped_gemm(&a, current_stream(x)), "grouped_gemm");
+}
+
+// pybind.cpp:14-16
+void GroupedSoftGemv(at::Tensor x, at::Tensor weight, at::Tensor scale, at::Tensor groupList,
+                     const char* computeType, at::Tensor output) {
+    const int fmt = parse_format(computeType);
+    moe_grouped_args a;
+    fill_grouped(a, x, weight, scale, nullptr, groupList, fmt, output);
+    c10::DeviceGuard guard(x.device());
+    check_status(moe_grouped_gemv(&a, current_stream(x)), "grouped_soft_gemv");
+}
+
+// Extra entry point: codes uint8 [R, C/2], scale bf16 [R, C/block] -> output bf16 [R, C].
+void DequantFp4(at::Tensor weight, at::Tensor scale, at::Tensor output) {
+    if (!weight.defined() || !weight.is_cuda()) fail("weight must be a GPU tensor");
+    check_tensor(weight, "weight", at::kByte, 2, weight);
+    check_tensor(scale, "scale", at::kBFloat16, 2, weight);
+    check_tensor(output, "output", at::kBFloat16, 2, weight);
+    const int64_t R = weight.size(0), C = weight.size(1) * 2;
+    if (output.size(0) != R || output.size(1) != C) fail("output must be [rows, 2 * weight.shape[1]]");
+    if (scale.size(0) != R || scale.size(1) == 0 || C % scale.size(1)) fail("scale must be [rows, cols / block]");
+    moe_dequant_args a;
+    a.codes = weight.data_ptr();
+    a.scale = scale.data_ptr();
+    a.out = output.data_ptr();
+    a.rows = R; a.cols = C;
+    a.block = static_cast<int32_t>(C / scale.size(1));
+    a.reserved = 0;
+    c10::DeviceGuard guard(weight.device());
+    check_status(moe_dequant_fp4_bf16(&a, current_stream(weight)), "dequant_fp4");
+}
+
+}  // namespace
+
+PYBIND11_MODULE(cinfer_ascendc, m) {
+    using namespace pybind11::literals;
+    m.def("grouped_soft_gemv", &GroupedSoftGemv, "x"_a, "weight"_a, "scale"_a, "groupList"_a, "computeType"_a,
+          "output"_a, "GROUP GEMV.");
+    m.def("grouped_gemm", &GroupedGemm, "x"_a, "weight"_a, "antiquantScaleOptional"_a, "antiquantOffsetOptional"_a,
+          "groupListOptional"_a, "computeType"_a, "output"_a, "GROUP GEMM.");
+    m.def("dequant_fp4", &DequantFp4, "weight"_a, "scale"_a, "output"_a, "FP4 (e2m1) -> BF16 block dequant.");
+}

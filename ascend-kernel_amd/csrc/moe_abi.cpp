@@ -1,0 +1,129 @@
+// C ABI of libmoe_gfx950.so: argument validation (host only, usable without a GPU),
+// error strings, and the extern "C" entry points that hand over to the launchers.
+#include <cstdint>
+#include <cstring>
+
+#include "moe_internal.h"
+
+namespace {
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+inline bool fits_i32(int64_t v) { return v >= 0 && v <= 0x7fffffffLL; }
+
+// Checks shared by GEMM and GEMV.  k_mult / n_mult are what the op's kernels
+// need on top of what the container itself implies.
+int validate_grouped(const moe_grouped_args* a, int64_t k_mult, int64_t n_mult) {
+    if (!a) return MOE_ERR_NULL_POINTER;
+    if (a->format < 0 || a->format >= MOE_FMT_COUNT || a->reserved != 0) return MOE_ERR_BAD_FORMAT;
+    if (a->M < 0 || a->K <= 0 || a->N <= 0 || a->G <= 0) return MOE_ERR_BAD_SHAPE;
+    // same limit as the reference: grouped_matmul_antiquant_tiling.cpp:260-264
+    if (!fits_i32(a->M) || !fits_i32(a->K) || !fits_i32(a->N) || !fits_i32(a->G)) return MOE_ERR_TOO_LARGE;
+    if (!a->weight || !a->group_list) return MOE_ERR_NULL_POINTER;
+    if (a->M > 0 && (!a->x || !a->y)) return MOE_ERR_NULL_POINTER;
+    if (a->format != MOE_FMT_BF16 && !a->scale) return MOE_ERR_NULL_POINTER;
+    if (a->format == MOE_FMT_INT8 && !a->offset) return MOE_ERR_NULL_POINTER;
+    if (a->K % k_mult || a->N % n_mult) return MOE_ERR_BAD_ALIGNMENT;
+    switch (a->format) {
+        case MOE_FMT_FP4_REF:
+            // the byte permutation works on 64(k) x 256(n) tiles; groups of 16 along K
+            if (a->K % 64 || a->N % 256) return MOE_ERR_BAD_ALIGNMENT;
+            if (a->scale_rows * 16 != a->K) return MOE_ERR_BAD_SHAPE;
+            break;
+        case MOE_FMT_FP8_REF:
+            if (a->K % 128 || a->N % 128) return MOE_ERR_BAD_ALIGNMENT;
+            break;
+        case MOE_FMT_INT4:
+            if (a->scale_rows <= 0 || a->K % a->scale_rows) return MOE_ERR_BAD_SHAPE;
+            if ((a->K / a->scale_rows) % 32) return MOE_ERR_BAD_ALIGNMENT;
+            break;
+        case MOE_FMT_FP4_B32:
+            if (a->K % 32) return MOE_ERR_BAD_ALIGNMENT;
+            break;
+        default:
+            break;
+    }
+    if (!aligned16(a->x) || !aligned16(a->weight) || !aligned16(a->y) || !aligned16(a->scale) ||
+        !aligned16(a->offset) || (reinterpret_cast<uintptr_t>(a->group_list) & 7u))
+        return MOE_ERR_BAD_ALIGNMENT;
+    return MOE_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int moe_abi_version(void) { return MOE_GFX950_ABI_VERSION; }
+
+const char* moe_strerror(int status) {
+    switch (status) {
+        case MOE_OK: return "ok";
+        case MOE_ERR_NULL_POINTER: return "a required pointer is NULL";
+        case MOE_ERR_BAD_FORMAT: return "unknown weight format / computeType";
+        case MOE_ERR_BAD_SHAPE: return "shape not valid for this weight format";
+        case MOE_ERR_BAD_ALIGNMENT: return "size or pointer alignment not supported by the kernels";
+        case MOE_ERR_TOO_LARGE: return "M, K, N or G out of int32 range";
+        case MOE_ERR_LAUNCH: return "kernel launch failed";
+        case MOE_ERR_NO_DEVICE: return "no gfx950 device";
+        default: return "unknown moe_status";
+    }
+}
+
+int moe_format_from_compute_type(const char* s) {
+    if (!s) return MOE_ERR_BAD_FORMAT;
+    if (!std::strcmp(s, "fp4")) return MOE_FMT_FP4_REF;
+    if (!std::strcmp(s, "fp8")) return MOE_FMT_FP8_REF;
+    if (!std::strcmp(s, "int8")) return MOE_FMT_INT8;
+    if (!std::strcmp(s, "int4")) return MOE_FMT_INT4;
+    if (!std::strcmp(s, "fp4_b32")) return MOE_FMT_FP4_B32;
+    if (!std::strcmp(s, "bf16")) return MOE_FMT_BF16;
+    return MOE_ERR_BAD_FORMAT;
+}
+
+int moe_dequant_fp4_bf16_validate(const moe_dequant_args* a) {
+    if (!a) return MOE_ERR_NULL_POINTER;
+    if (a->reserved != 0 || (a->block != 16 && a->block != 32)) return MOE_ERR_BAD_FORMAT;
+    if (a->rows < 0 || a->cols < 0) return MOE_ERR_BAD_SHAPE;
+    if (a->cols % a->block) return MOE_ERR_BAD_ALIGNMENT;
+    if (a->rows > 0 && a->cols > 0 && a->rows > (INT64_MAX / 4) / a->cols) return MOE_ERR_TOO_LARGE;
+    if (a->rows * a->cols > 0 && (!a->codes || !a->scale || !a->out)) return MOE_ERR_NULL_POINTER;
+    if (!aligned16(a->codes) || !aligned16(a->out) || (reinterpret_cast<uintptr_t>(a->scale) & 1u))
+        return MOE_ERR_BAD_ALIGNMENT;
+    return MOE_OK;
+}
+
+// GEMM: the workgroup tile spans 64 k and 256 n.
+int moe_grouped_gemm_validate(const moe_grouped_args* a) { return validate_grouped(a, 64, 256); }
+
+// GEMV: N-contiguous containers are read 256 columns per wavefront step,
+// K-contiguous ones 8 k per lane.
+int moe_grouped_gemv_validate(const moe_grouped_args* a) {
+    if (a && a->format == MOE_FMT_INT8) return MOE_ERR_BAD_FORMAT;  // the GEMV op has no offset operand
+    const bool k_major = a && (a->format == MOE_FMT_BF16 || a->format == MOE_FMT_FP4_B32);
+    return validate_grouped(a, k_major ? 32 : 64, k_major ? 1 : 256);
+}
+
+size_t moe_dequant_fp4_bf16_workspace_bytes(const moe_dequant_args*) { return 0; }
+size_t moe_grouped_gemm_workspace_bytes(const moe_grouped_args*) { return 0; }
+size_t moe_grouped_gemv_workspace_bytes(const moe_grouped_args*) { return 0; }
+
+int moe_dequant_fp4_bf16(const moe_dequant_args* a, moe_stream_t stream) {
+    int rc = moe_dequant_fp4_bf16_validate(a);
+    if (rc != MOE_OK) return rc;
+    return moe::launch_dequant_fp4_bf16(a, static_cast<hipStream_t>(stream));
+}
+
+int moe_grouped_gemm(const moe_grouped_args* a, moe_stream_t stream) {
+    int rc = moe_grouped_gemm_validate(a);
+    if (rc != MOE_OK) return rc;
+    if (a->M == 0) return MOE_OK;
+    return moe::launch_grouped_gemm(a, static_cast<hipStream_t>(stream));
+}
+
+int moe_grouped_gemv(const moe_grouped_args* a, moe_stream_t stream) {
+    int rc = moe_grouped_gemv_validate(a);
+    if (rc != MOE_OK) return rc;
+    if (a->M == 0) return MOE_OK;
+    return moe::launch_grouped_gemv(a, static_cast<hipStream_t>(stream));
+}
+
+}  // extern "C"

@@ -1,0 +1,63 @@
+// FP4 (e2m1) -> BF16 block-scaled dequantization for gfx950: a pure streaming
+// kernel.  HBM bound: 0.5 B (code) + 2/block B (scale) read and 2 B written per
+// element.  Replaces phase 1 of the reference GEMM kernel (CastWeightProcess,
+// grouped_gemm/op_kernel/grouped_matmul_antiquant.h:537-662) as a stand-alone op.
+#include "moe_device.h"
+#include "moe_internal.h"
+
+namespace moe {
+
+// One thread decodes UNROLL independent dwords (8 codes each) and writes UNROLL
+// 16-byte vectors.  Consecutive lanes take consecutive dwords, so every load
+// instruction of a wavefront covers 256 contiguous bytes and every store 1 KiB.
+// The tensors are addressed flat: rows are contiguous and cols % BLOCK == 0, so
+// element e uses scale e / BLOCK.
+template <int BLOCK, int UNROLL>
+__global__ __launch_bounds__(256) void dequant_fp4_bf16_kernel(const uint32_t* __restrict__ codes,
+                                                               const uint16_t* __restrict__ scale,
+                                                               u32x4_t* __restrict__ out,
+                                                               int64_t nwords) {
+    const int64_t base = (int64_t)blockIdx.x * (256 * UNROLL) + threadIdx.x;
+    uint32_t w[UNROLL];
+    float s[UNROLL];
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+        const int64_t i = base + u * 256;
+        if (i < nwords) {
+            w[u] = __builtin_nontemporal_load(codes + i);
+            s[u] = bf16_bits_to_f32(scale[(i * 8) / BLOCK]);
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+        const int64_t i = base + u * 256;
+        if (i < nwords) {
+            u32x4_t o;
+            o[0] = e2m1_pair_scaled_bf16<0>(w[u], s[u]);
+            o[1] = e2m1_pair_scaled_bf16<1>(w[u], s[u]);
+            o[2] = e2m1_pair_scaled_bf16<2>(w[u], s[u]);
+            o[3] = e2m1_pair_scaled_bf16<3>(w[u], s[u]);
+            __builtin_nontemporal_store(o, out + i);
+        }
+    }
+}
+
+int launch_dequant_fp4_bf16(const moe_dequant_args* a, hipStream_t stream) {
+    const int64_t nwords = a->rows * a->cols / 8;
+    if (nwords == 0) return MOE_OK;
+    constexpr int UNROLL = 4;
+    const int64_t blocks = (nwords + 256 * UNROLL - 1) / (256 * UNROLL);
+    if (blocks > 0x7fffffffLL) return MOE_ERR_TOO_LARGE;
+    const uint32_t* codes = static_cast<const uint32_t*>(a->codes);
+    const uint16_t* scale = static_cast<const uint16_t*>(a->scale);
+    u32x4_t* out = static_cast<u32x4_t*>(a->out);
+    if (a->block == 32)
+        hipLaunchKernelGGL((dequant_fp4_bf16_kernel<32, UNROLL>), dim3((unsigned)blocks), dim3(256), 0, stream,
+                           codes, scale, out, nwords);
+    else
+        hipLaunchKernelGGL((dequant_fp4_bf16_kernel<16, UNROLL>), dim3((unsigned)blocks), dim3(256), 0, stream,
+                           codes, scale, out, nwords);
+    return hipGetLastError() == hipSuccess ? MOE_OK : MOE_ERR_LAUNCH;
+}
+
+}  // namespace moe

@@ -1,0 +1,623 @@
+// Grouped GEMM with weight antiquant for MoE prefill on gfx950.
+//
+//   y[rows of expert g, :] = x[rows of expert g, :] . dequant(W[g])     bf16 x bf16 -> fp32 -> bf16
+//
+// Replaces grouped_matmul_antiquant (grouped_gemm/op_kernel/grouped_matmul_antiquant.h:225-364,
+// grouped_matmul.h:147-463).  The reference decodes each weight slab to a bf16 copy in
+// global memory and then runs a bf16 matmul on it; here the packed weights go
+// HBM -> registers -> bf16 MFMA fragments directly and never touch LDS or HBM again.
+//
+// Work decomposition.  A tile is (expert, chunk of <= 192 rows, 256 columns).  The
+// tile list is derived inside the kernel from the device-resident cumulative
+// group_list (no host sync); a persistent grid walks it with an XCD-aware order so
+// that the workgroups of one XCD share the x rows of the same experts in that XCD's
+// L2.  A workgroup has 4 wavefronts; every wavefront owns 64 of the 256 columns for
+// ALL rows of the tile, so each weight element is dequantized exactly once per tile.
+// x tiles go through a double-buffered, XOR-swizzled LDS tile shared by the 4 waves.
+//
+// MFMA: v_mfma_f32_16x16x32_bf16.  Lane l = 16*q + i holds, for A, row i and
+// k = 8q..8q+7 of the 16x32 block; for B, column i and the same k; for the result,
+// column i and rows 4q..4q+3.  The contraction index may be permuted freely as long
+// as A and B agree, and so may the column <-> (MFMA, lane) assignment; each weight
+// container picks the assignment that makes its global loads wide and contiguous.
+#include "moe_device.h"
+#include "moe_internal.h"
+
+namespace moe {
+
+constexpr int GM_BN = 256;     // columns per workgroup
+constexpr int GM_MT_MAX = 12;  // 16-row blocks per tile (192 rows)
+constexpr int GM_THREADS = 256;
+
+struct GemmParams {
+    const uint16_t* x;
+    const uint8_t* w;
+    const void* scale;
+    const uint16_t* offset;
+    const int64_t* gl;
+    uint16_t* y;
+    int64_t M;
+    int K, N, G, scale_rows;
+};
+
+// Buffer resources keep the addressing compact: one 128-bit descriptor in SGPRs per
+// tensor slab, one 32-bit per-lane offset that is constant for the whole tile, and a
+// wave-uniform (scalar) offset per load.  Reads beyond the slab return 0.
+typedef __amdgpu_buffer_rsrc_t rsrc_t;
+__device__ __forceinline__ rsrc_t make_rsrc(const void* p, int64_t bytes) {
+    const uint32_t n = bytes > 0xffffffffLL ? 0xffffffffu : (uint32_t)bytes;
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, n, 0x00020000);
+}
+__device__ __forceinline__ uint32_t ldg_b32(rsrc_t r, int voff, int soff) {
+    return __builtin_amdgcn_raw_buffer_load_b32(r, voff, soff, 0);
+}
+__device__ __forceinline__ u32x2_t ldg_b64(rsrc_t r, int voff, int soff) {
+    return __builtin_amdgcn_raw_buffer_load_b64(r, voff, soff, 0);
+}
+__device__ __forceinline__ u32x4_t ldg_b128(rsrc_t r, int voff, int soff) {
+    return __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, 0);
+}
+
+// Per-lane view of one tile for the weight loaders.
+struct BCtx {
+    rsrc_t rw, rs;       // weight / scale slab of the expert
+    int vw, vs;          // per-lane byte offsets into them (constant over the tile)
+    const uint16_t* sg;  // int8: scale / offset rows of the expert
+    const uint16_t* og;
+    const float* s8;     // fp8: scale blocks of the expert
+    int K, N, n0, gs;    // gs = k per scale group (int4)
+    int i, q, w;         // lane & 15, lane >> 4, wavefront (scalar)
+};
+
+template <int FMT>
+struct BTraits;
+
+// ------------------------------------------------------------------ int4, [K, N/2]
+// Lane (i, q) of wavefront w loads, for each of its 8 k rows, the dword holding the
+// 8 columns 128(w>>1) + 8i + [0,8); wavefronts 2p and 2p+1 read the same dwords and
+// use nibbles 0-3 and 4-7.  MFMA t gets nibble 4(w&1) + t.
+template <>
+struct BTraits<MOE_FMT_INT4> {
+    static constexpr int BK = 64, NS = 2;
+    struct Raw {
+        uint32_t r[2][8];
+        u32x2_t sc[2];
+    };
+    __device__ static __forceinline__ int a_chunk(int s, int q) { return 4 * s + q; }
+    __device__ static __forceinline__ int col(const BCtx& c, int t) {
+        return 128 * (c.w >> 1) + 8 * c.i + 4 * (c.w & 1) + t;
+    }
+    __device__ static __forceinline__ void init(BCtx& c) {
+        c.vw = 8 * c.q * (c.N >> 1) + 64 * (c.w >> 1) + 4 * c.i;
+        c.vs = col(c, 0) * 2;
+    }
+    __device__ static __forceinline__ void load(Raw& raw, const BCtx& c, int k0) {
+        const int nb = c.N >> 1;
+#pragma unroll
+        for (int s = 0; s < 2; ++s) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) raw.r[s][j] = ldg_b32(c.rw, c.vw, (k0 + 32 * s + j) * nb + (c.n0 >> 1));
+            // a 32-k sub-step never straddles a scale group (group % 32 == 0)
+            raw.sc[s] = ldg_b64(c.rs, c.vs, (((k0 + 32 * s) / c.gs) * c.N + c.n0) * 2);
+        }
+    }
+    __device__ static __forceinline__ void frags(const Raw& raw, const BCtx& c, int s, u32x4_t out[4]) {
+        const int sh = 16 * (c.w & 1);
+        const float sc[4] = {bf16_lo(raw.sc[s][0]), bf16_hi(raw.sc[s][0]), bf16_lo(raw.sc[s][1]),
+                             bf16_hi(raw.sc[s][1])};
+#pragma unroll
+        for (int j = 0; j < 8; j += 2) {
+            const uint32_t a = raw.r[s][j] >> sh, b = raw.r[s][j + 1] >> sh;
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                const float fa = (float)((int)((a >> (4 * t)) & 15u) - 8) * sc[t];
+                const float fb = (float)((int)((b >> (4 * t)) & 15u) - 8) * sc[t];
+                out[t][j >> 1] = pack_bf16_rne(fa, fb);
+            }
+        }
+    }
+};
+
+// ---------------------------------------------- reference "fp4": pre-shuffled [K, N/2]
+// Inside tile (a = k/64, 256-column block) destination row R = j<<5 | i'<<3 | p holds
+// k = 64a + 16i' + 8j + [0,8) for columns 32p + [0,32); bytes 32q' + 4r + [0,4) of
+// that row are the 8 columns 32p + 8q' + [0,8) at k offset r.  So the 8 k rows a lane
+// needs for its 8-column group are 32 contiguous bytes.
+template <>
+struct BTraits<MOE_FMT_FP4_REF> {
+    static constexpr int BK = 64, NS = 2;
+    struct Raw {
+        u32x4_t r[2][2];
+        u32x2_t sc[2];
+    };
+    __device__ static __forceinline__ int a_chunk(int s, int q) { return 4 * s + q; }
+    __device__ static __forceinline__ int col(const BCtx& c, int t) {
+        return 128 * (c.w >> 1) + 8 * c.i + 4 * (c.w & 1) + t;
+    }
+    __device__ static __forceinline__ void init(BCtx& c) {
+        const int c8 = 16 * (c.w >> 1) + c.i, p = c8 >> 2, qq = c8 & 3;
+        // row of sub-step 0; sub-step s adds 16 rows (i' = 2s + (q >> 1))
+        const int R0 = ((c.q & 1) << 5) | ((c.q >> 1) << 3) | p;
+        c.vw = R0 * (c.N >> 1) + 32 * qq;
+        c.vs = ((c.q >> 1) * c.N + col(c, 0)) * 2;  // scale group of 16 k: (k0 + 32s)/16 + (q >> 1)
+    }
+    __device__ static __forceinline__ void load(Raw& raw, const BCtx& c, int k0) {
+        const int nb = c.N >> 1;
+#pragma unroll
+        for (int s = 0; s < 2; ++s) {
+            const int so = (k0 + 16 * s) * nb + (c.n0 >> 1);
+            raw.r[s][0] = ldg_b128(c.rw, c.vw, so);
+            raw.r[s][1] = ldg_b128(c.rw, c.vw, so + 16);
+            raw.sc[s] = ldg_b64(c.rs, c.vs, (((k0 + 32 * s) >> 4) * c.N + c.n0) * 2);
+        }
+    }
+    __device__ static __forceinline__ void frags(const Raw& raw, const BCtx& c, int s, u32x4_t out[4]) {
+        const int sh = 16 * (c.w & 1);
+        const float sc[4] = {bf16_lo(raw.sc[s][0]), bf16_hi(raw.sc[s][0]), bf16_lo(raw.sc[s][1]),
+                             bf16_hi(raw.sc[s][1])};
+#pragma unroll
+        for (int j = 0; j < 8; j += 2) {
+            const uint32_t a = raw.r[s][j >> 2][j & 3] >> sh, b = raw.r[s][(j + 1) >> 2][(j + 1) & 3] >> sh;
+            const f32x2_t a01 = e2m1_pair_to_f32<0>(a), a23 = e2m1_pair_to_f32<1>(a);
+            const f32x2_t b01 = e2m1_pair_to_f32<0>(b), b23 = e2m1_pair_to_f32<1>(b);
+            out[0][j >> 1] = pack_bf16_rne(a01[0] * sc[0], b01[0] * sc[0]);
+            out[1][j >> 1] = pack_bf16_rne(a01[1] * sc[1], b01[1] * sc[1]);
+            out[2][j >> 1] = pack_bf16_rne(a23[0] * sc[2], b23[0] * sc[2]);
+            out[3][j >> 1] = pack_bf16_rne(a23[1] * sc[3], b23[1] * sc[3]);
+        }
+    }
+};
+
+// ------------------------------------------------------- int8 / reference fp8, [K, N]
+// Lane (i, q) loads the dword with columns 64w + 4i + [0,4) of each of its 8 k rows.
+template <int FMT>
+struct BTraitsByte {
+    static constexpr int BK = 64, NS = 2;
+    struct Raw {
+        uint32_t r[2][8];
+        float s8;  // fp8: scale of the 128x128 block of this step
+    };
+    __device__ static __forceinline__ int a_chunk(int s, int q) { return 4 * s + q; }
+    __device__ static __forceinline__ int col(const BCtx& c, int t) { return 64 * c.w + 4 * c.i + t; }
+    __device__ static __forceinline__ void init(BCtx& c) {
+        c.vw = 8 * c.q * c.N + col(c, 0);
+        c.vs = 0;
+    }
+    __device__ static __forceinline__ void load(Raw& raw, const BCtx& c, int k0) {
+#pragma unroll
+        for (int s = 0; s < 2; ++s)
+#pragma unroll
+            for (int j = 0; j < 8; ++j) raw.r[s][j] = ldg_b32(c.rw, c.vw, (k0 + 32 * s + j) * c.N + c.n0);
+        if (FMT == MOE_FMT_FP8_REF) raw.s8 = c.s8[(k0 >> 7) * (c.N >> 7) + ((c.n0 + 64 * c.w) >> 7)];
+    }
+};
+
+template <>
+struct BTraits<MOE_FMT_INT8> : BTraitsByte<MOE_FMT_INT8> {
+    // per-channel scale and offset of this lane's 4 columns, fixed for the whole tile
+    float sc[4], of[4];
+    __device__ __forceinline__ void prepare_m(const BCtx& c) {
+        const u32x2_t s = *reinterpret_cast<const u32x2_t*>(c.sg + c.n0 + col(c, 0));
+        const u32x2_t o = *reinterpret_cast<const u32x2_t*>(c.og + c.n0 + col(c, 0));
+        sc[0] = bf16_lo(s[0]); sc[1] = bf16_hi(s[0]); sc[2] = bf16_lo(s[1]); sc[3] = bf16_hi(s[1]);
+        of[0] = bf16_lo(o[0]); of[1] = bf16_hi(o[0]); of[2] = bf16_lo(o[1]); of[3] = bf16_hi(o[1]);
+    }
+    __device__ __forceinline__ void frags_m(const Raw& raw, const BCtx&, int s, u32x4_t out[4]) const {
+#pragma unroll
+        for (int j = 0; j < 8; j += 2) {
+            const uint32_t a = raw.r[s][j], b = raw.r[s][j + 1];
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                const float qa = (float)(int)(int8_t)(a >> (8 * t)), qb = (float)(int)(int8_t)(b >> (8 * t));
+                // (q + offset) * scale as two rounded fp32 operations
+                out[t][j >> 1] = pack_bf16_rne(__fmul_rn(__fadd_rn(qa, of[t]), sc[t]),
+                                               __fmul_rn(__fadd_rn(qb, of[t]), sc[t]));
+            }
+        }
+    }
+};
+
+template <>
+struct BTraits<MOE_FMT_FP8_REF> : BTraitsByte<MOE_FMT_FP8_REF> {
+    __device__ __forceinline__ void prepare_m(const BCtx&) {}
+    __device__ __forceinline__ void frags_m(const Raw& raw, const BCtx&, int s, u32x4_t out[4]) const {
+#pragma unroll
+        for (int j = 0; j < 8; j += 2) {
+            const uint32_t a = raw.r[s][j], b = raw.r[s][j + 1];
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+                out[t][j >> 1] = pack_bf16_rne(e4m3_ref_to_f32((a >> (8 * t)) & 0xffu) * raw.s8,
+                                               e4m3_ref_to_f32((b >> (8 * t)) & 0xffu) * raw.s8);
+        }
+    }
+};
+
+// -------------------------------------------------------- fp4 block-32, [N, K/2]
+// K-contiguous: MFMA t, lane (i, q) owns column 64w + 16t + i and loads the 16 bytes
+// holding k = k0 + 32q + [0,32) (exactly one scale block); sub-step s uses
+// k = k0 + 32q + 8s + [0,8), so the matching x chunk is 4q + s.
+template <>
+struct BTraits<MOE_FMT_FP4_B32> {
+    static constexpr int BK = 128, NS = 4;
+    struct Raw {
+        u32x4_t r[4];
+        float sc[4];
+    };
+    __device__ static __forceinline__ int a_chunk(int s, int q) { return 4 * q + s; }
+    __device__ static __forceinline__ int col(const BCtx& c, int t) { return 64 * c.w + 16 * t + c.i; }
+    __device__ static __forceinline__ void init(BCtx& c) {
+        c.vw = (64 * c.w + c.i) * (c.K >> 1) + 16 * c.q;
+        c.vs = ((64 * c.w + c.i) * (c.K >> 5) + c.q) * 2;
+    }
+    __device__ static __forceinline__ void load(Raw& raw, const BCtx& c, int k0) {
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            raw.r[t] = ldg_b128(c.rw, c.vw, (c.n0 + 16 * t) * (c.K >> 1) + (k0 >> 1));
+            raw.sc[t] = bf16_bits_to_f32(
+                __builtin_amdgcn_raw_buffer_load_b16(c.rs, c.vs, ((c.n0 + 16 * t) * (c.K >> 5) + (k0 >> 5)) * 2, 0));
+        }
+    }
+    __device__ static __forceinline__ void frags(const Raw& raw, const BCtx&, int s, u32x4_t out[4]) {
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            const uint32_t wd = raw.r[t][s];
+            out[t][0] = e2m1_pair_scaled_bf16<0>(wd, raw.sc[t]);
+            out[t][1] = e2m1_pair_scaled_bf16<1>(wd, raw.sc[t]);
+            out[t][2] = e2m1_pair_scaled_bf16<2>(wd, raw.sc[t]);
+            out[t][3] = e2m1_pair_scaled_bf16<3>(wd, raw.sc[t]);
+        }
+    }
+};
+
+// ------------------------------------------------------------------ bf16, [N, K]
+// K-contiguous: lane (i, q) loads 32 contiguous bytes, k = k0 + 16q + [0,16); sub-step
+// s uses the half k0 + 16q + 8s + [0,8), so the matching x chunk is 2q + s.
+template <>
+struct BTraits<MOE_FMT_BF16> {
+    static constexpr int BK = 64, NS = 2;
+    struct Raw {
+        u32x4_t r[4][2];
+    };
+    __device__ static __forceinline__ int a_chunk(int s, int q) { return 2 * q + s; }
+    __device__ static __forceinline__ int col(const BCtx& c, int t) { return 64 * c.w + 16 * t + c.i; }
+    __device__ static __forceinline__ void init(BCtx& c) {
+        c.vw = (64 * c.w + c.i) * c.K * 2 + 32 * c.q;
+        c.vs = 0;
+    }
+    __device__ static __forceinline__ void load(Raw& raw, const BCtx& c, int k0) {
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            const int so = ((c.n0 + 16 * t) * c.K + k0) * 2;
+            raw.r[t][0] = ldg_b128(c.rw, c.vw, so);
+            raw.r[t][1] = ldg_b128(c.rw, c.vw, so + 16);
+        }
+    }
+    __device__ static __forceinline__ void frags(const Raw& raw, const BCtx&, int s, u32x4_t out[4]) {
+#pragma unroll
+        for (int t = 0; t < 4; ++t) out[t] = raw.r[t][s];
+    }
+};
+
+// Uniform wrappers: formats with per-tile state (int8) use member functions.
+template <int FMT>
+struct BOps {
+    BTraits<FMT> st;
+    __device__ __forceinline__ void prepare(const BCtx& c) {
+        if constexpr (FMT == MOE_FMT_INT8 || FMT == MOE_FMT_FP8_REF) st.prepare_m(c);
+    }
+    __device__ __forceinline__ void frags(const typename BTraits<FMT>::Raw& raw, const BCtx& c, int s,
+                                          u32x4_t out[4]) const {
+        if constexpr (FMT == MOE_FMT_INT8 || FMT == MOE_FMT_FP8_REF)
+            st.frags_m(raw, c, s, out);
+        else
+            BTraits<FMT>::frags(raw, c, s, out);
+    }
+};
+
+// ---------------------------------------------------------------------------------
+// x tile: rows x BK bf16 in LDS, 16-byte chunks, chunk c of row r stored at
+// position c ^ (r & 7) so that the 8 lanes a ds_read_b128 serves together hit
+// distinct banks both when writing (consecutive chunks of one row) and when
+// reading fragments (same chunk of 8 consecutive rows).
+// ---------------------------------------------------------------------------------
+template <int BK>
+__device__ __forceinline__ int a_lds_unit(int row, int c) {
+    return row * (BK / 8) + (c ^ (row & 7));
+}
+
+template <int FMT, int MT>
+__device__ __forceinline__ void gemm_tile(const GemmParams& P, u32x4_t* lds_a, int g, int64_t row0, int rows,
+                                          int n0) {
+    using T = BTraits<FMT>;
+    constexpr int BK = T::BK, NS = T::NS;
+    constexpr int CPR = BK / 8;               // 16-byte chunks per tile row
+    constexpr int RPP = GM_THREADS / CPR;     // rows loaded per pass
+    constexpr int PASSES = (16 * MT + RPP - 1) / RPP;
+    constexpr int ABUF = 16 * GM_MT_MAX * CPR;  // units per buffer
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    BCtx c;
+    c.K = P.K; c.N = P.N; c.n0 = n0;
+    c.i = lane & 15; c.q = lane >> 4; c.w = __builtin_amdgcn_readfirstlane(tid >> 6);
+    c.gs = 1; c.sg = nullptr; c.og = nullptr; c.s8 = nullptr;
+    const int64_t KN = (int64_t)P.K * P.N;
+    switch (FMT) {
+        case MOE_FMT_INT4:
+            c.rw = make_rsrc(P.w + g * (KN >> 1), KN >> 1);
+            c.rs = make_rsrc(static_cast<const uint16_t*>(P.scale) + (int64_t)g * P.scale_rows * P.N,
+                             (int64_t)P.scale_rows * P.N * 2);
+            c.gs = P.K / P.scale_rows;
+            break;
+        case MOE_FMT_FP4_REF:
+            c.rw = make_rsrc(P.w + g * (KN >> 1), KN >> 1);
+            c.rs = make_rsrc(static_cast<const uint16_t*>(P.scale) + g * (KN >> 4), KN >> 3);
+            break;
+        case MOE_FMT_INT8:
+            c.rw = make_rsrc(P.w + g * KN, KN);
+            c.rs = c.rw;
+            c.sg = static_cast<const uint16_t*>(P.scale) + (int64_t)g * P.N;
+            c.og = P.offset + (int64_t)g * P.N;
+            break;
+        case MOE_FMT_FP8_REF:
+            c.rw = make_rsrc(P.w + g * KN, KN);
+            c.rs = c.rw;
+            c.s8 = static_cast<const float*>(P.scale) + (int64_t)g * (P.K >> 7) * (P.N >> 7);
+            break;
+        case MOE_FMT_FP4_B32:
+            c.rw = make_rsrc(P.w + g * (KN >> 1), KN >> 1);
+            c.rs = make_rsrc(static_cast<const uint16_t*>(P.scale) + g * (KN >> 5), KN >> 4);
+            break;
+        default:
+            c.rw = make_rsrc(P.w + g * KN * 2, KN * 2);
+            c.rs = c.rw;
+            break;
+    }
+    T::init(c);
+    BOps<FMT> ops;
+    ops.prepare(c);
+
+    // x rows of this tile through a buffer resource that ends after the last valid row:
+    // padded rows read as zeros.  This thread loads chunk ac of rows ar + RPP*p.
+    const int ar = tid / CPR, ac = tid % CPR;
+    const rsrc_t rx = make_rsrc(P.x + row0 * (int64_t)P.K, (int64_t)rows * P.K * 2);
+    const int vx = (ar * P.K + ac * 8) * 2;
+
+    f32x4_t acc[MT][4];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int t = 0; t < 4; ++t) acc[mt][t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+
+    u32x4_t areg[PASSES];
+    typename T::Raw raw, raw_next;
+    const int nk = P.K / BK;
+
+    auto load_a = [&](int kt) {
+#pragma unroll
+        for (int p = 0; p < PASSES; ++p)
+            if (PASSES * RPP == 16 * MT || ar + RPP * p < 16 * MT)
+                areg[p] = ldg_b128(rx, vx, (p * RPP * P.K + kt * BK) * 2);
+    };
+    auto store_a = [&](int buf) {
+#pragma unroll
+        for (int p = 0; p < PASSES; ++p)
+            if (PASSES * RPP == 16 * MT || ar + RPP * p < 16 * MT)
+                lds_a[buf * ABUF + a_lds_unit<BK>(ar + RPP * p, ac)] = areg[p];
+    };
+    auto compute = [&](const typename T::Raw& rw, int buf) {
+        const u32x4_t* la = lds_a + buf * ABUF;
+#pragma unroll
+        for (int s = 0; s < NS; ++s) {
+            u32x4_t bf[4];
+            ops.frags(rw, c, s, bf);
+            const int ch = T::a_chunk(s, c.q);
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+                const u32x4_t av = la[a_lds_unit<BK>(16 * mt + c.i, ch)];
+                const bf16x8_t a8 = __builtin_bit_cast(bf16x8_t, av);
+#pragma unroll
+                for (int t = 0; t < 4; ++t)
+                    acc[mt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a8, __builtin_bit_cast(bf16x8_t, bf[t]),
+                                                                         acc[mt][t], 0, 0, 0);
+            }
+        }
+    };
+
+    // Software pipeline: while step kt is computed from LDS buffer kt&1 and `raw`, the x
+    // tile and the packed weights of step kt+1 are in flight to registers; the x tile is
+    // written to the other LDS buffer after the MFMAs, one barrier per step.
+    __syncthreads();  // previous tile's readers are done with both buffers
+    load_a(0);
+    T::load(raw, c, 0);
+    store_a(0);
+    __syncthreads();
+    // The last step prefetches one step past K: buffer loads beyond a slab return 0 and
+    // the x rows it reads are inside the tensor; neither is used.
+    for (int kt = 0; kt < nk; ++kt) {
+        load_a(kt + 1);
+        T::load(raw_next, c, (kt + 1) * BK);
+        compute(raw, kt & 1);
+        // pin the loop-carried accumulators to AGPRs so that every MFMA accumulates in place
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int t = 0; t < 4; ++t) asm volatile("" : "+a"(acc[mt][t]));
+        store_a((kt + 1) & 1);
+        __syncthreads();
+        raw = raw_next;
+    }
+
+    // epilogue: fp32 -> bf16 (RNE), rows beyond the chunk are dropped
+    constexpr bool N_CONTIG = (FMT == MOE_FMT_INT4 || FMT == MOE_FMT_FP4_REF || FMT == MOE_FMT_INT8 ||
+                               FMT == MOE_FMT_FP8_REF);
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int row = 16 * mt + 4 * c.q + r;
+            if (row < rows) {
+                uint16_t* yp = P.y + (row0 + row) * (int64_t)P.N + n0;
+                if (N_CONTIG) {
+                    u32x2_t v;
+                    v[0] = pack_bf16_rne(acc[mt][0][r], acc[mt][1][r]);
+                    v[1] = pack_bf16_rne(acc[mt][2][r], acc[mt][3][r]);
+                    *reinterpret_cast<u32x2_t*>(yp + T::col(c, 0)) = v;
+                } else {
+#pragma unroll
+                    for (int t = 0; t < 4; ++t)
+                        yp[T::col(c, t)] = (uint16_t)(pack_bf16_rne(acc[mt][t][r], 0.f) & 0xffffu);
+                }
+            }
+        }
+}
+
+// ---------------------------------------------------------------------------------
+// Tile scheduler (role of GMMAntiquantProcess::Process,
+// grouped_gemm/op_kernel/grouped_matmul_antiquant.h:241-288).  Expert g with m_g rows
+// has ceil(m_g/16) row blocks, cut into the fewest chunks of <= GM_MT_MAX blocks, as
+// even as possible; each chunk has N/256 tiles.  prefix[] (in LDS) is the exclusive
+// scan of the tile counts.
+// ---------------------------------------------------------------------------------
+__device__ __forceinline__ void expert_chunks(int m, int& chunks, int& bpc) {
+    const int nblk = (m + 15) >> 4;
+    chunks = (nblk + GM_MT_MAX - 1) / GM_MT_MAX;
+    bpc = chunks ? (nblk + chunks - 1) / chunks : 0;
+}
+
+template <int FMT>
+__global__ __launch_bounds__(GM_THREADS) void grouped_gemm_kernel(GemmParams P) {
+    extern __shared__ u32x4_t smem[];
+    constexpr int BK = BTraits<FMT>::BK;
+    u32x4_t* lds_a = smem;                                                         // 2 buffers
+    int* prefix = reinterpret_cast<int*>(smem + 2 * 16 * GM_MT_MAX * (BK / 8));    // [G + 1]
+    const int tid = threadIdx.x;
+    const int ntile_n = P.N / GM_BN;
+
+    // exclusive scan of tiles per expert: each thread takes a contiguous run of experts
+    {
+        __shared__ int part[GM_THREADS];
+        const int per = (P.G + GM_THREADS - 1) / GM_THREADS;
+        const int g0 = tid * per, g1 = min(P.G, g0 + per);
+        int sum = 0;
+        for (int g = g0; g < g1; ++g) {
+            int64_t s = g ? P.gl[g - 1] : 0, e = P.gl[g];
+            s = max((int64_t)0, s); e = min(e, P.M);
+            int chunks, bpc;
+            expert_chunks(e > s ? (int)(e - s) : 0, chunks, bpc);
+            sum += chunks * ntile_n;
+        }
+        part[tid] = sum;
+        __syncthreads();
+        if (tid == 0) {
+            int run = 0;
+            for (int t = 0; t < GM_THREADS; ++t) { const int v = part[t]; part[t] = run; run += v; }
+            prefix[P.G] = run;
+        }
+        __syncthreads();
+        int run = part[tid];
+        for (int g = g0; g < g1; ++g) {
+            int64_t s = g ? P.gl[g - 1] : 0, e = P.gl[g];
+            s = max((int64_t)0, s); e = min(e, P.M);
+            int chunks, bpc;
+            expert_chunks(e > s ? (int)(e - s) : 0, chunks, bpc);
+            prefix[g] = run;
+            run += chunks * ntile_n;
+        }
+        __syncthreads();
+    }
+    const int total = __builtin_amdgcn_readfirstlane(prefix[P.G]);
+
+    // XCD-aware order: workgroup b runs on XCD b % 8; give each XCD a contiguous run of
+    // tiles in every sweep so that its workgroups share x rows in its own L2.
+    const int nwg = gridDim.x;
+    const int per_xcd = (nwg + 7) / 8;
+    const int vid = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+    const int sweep = per_xcd * 8;
+
+    for (int T = vid; T < total; T += sweep) {
+        // largest g with prefix[g] <= T (empty experts have prefix[g] == prefix[g+1])
+        int lo = 0, hi = P.G;
+        while (hi - lo > 1) {
+            const int mid = (lo + hi) >> 1;
+            if (prefix[mid] <= T) lo = mid; else hi = mid;
+        }
+        // everything below is wave-uniform; readfirstlane lets the compiler keep it in SGPRs
+        const int g = __builtin_amdgcn_readfirstlane(lo);
+        const int64_t gbeg = g ? max((int64_t)0, P.gl[g - 1]) : 0, gend = min(P.gl[g], P.M);
+        const int m = __builtin_amdgcn_readfirstlane((int)(gend - gbeg));
+        int chunks, bpc;
+        expert_chunks(m, chunks, bpc);
+        const int local = __builtin_amdgcn_readfirstlane(T - prefix[g]);
+        const int chunk = local / ntile_n, nt = local % ntile_n;
+        const int rbeg = chunk * bpc * 16;
+        const int rows = min(m - rbeg, bpc * 16);
+        const int mt = (rows + 15) >> 4;
+        const int rlo = __builtin_amdgcn_readfirstlane((int)(uint32_t)(gbeg & 0xffffffffLL));
+        const int rhi = __builtin_amdgcn_readfirstlane((int)(gbeg >> 32));
+        const int64_t row0 = (((int64_t)rhi << 32) | (uint32_t)rlo) + rbeg;
+        const int n0 = nt * GM_BN;
+        switch (mt) {
+            case 1: gemm_tile<FMT, 1>(P, lds_a, g, row0, rows, n0); break;
+            case 2: gemm_tile<FMT, 2>(P, lds_a, g, row0, rows, n0); break;
+            case 3: gemm_tile<FMT, 3>(P, lds_a, g, row0, rows, n0); break;
+            case 4: gemm_tile<FMT, 4>(P, lds_a, g, row0, rows, n0); break;
+            case 5: gemm_tile<FMT, 5>(P, lds_a, g, row0, rows, n0); break;
+            case 6: gemm_tile<FMT, 6>(P, lds_a, g, row0, rows, n0); break;
+            case 7: gemm_tile<FMT, 7>(P, lds_a, g, row0, rows, n0); break;
+            case 8: gemm_tile<FMT, 8>(P, lds_a, g, row0, rows, n0); break;
+            case 9: gemm_tile<FMT, 9>(P, lds_a, g, row0, rows, n0); break;
+            case 10: gemm_tile<FMT, 10>(P, lds_a, g, row0, rows, n0); break;
+            case 11: gemm_tile<FMT, 11>(P, lds_a, g, row0, rows, n0); break;
+            default: gemm_tile<FMT, 12>(P, lds_a, g, row0, rows, n0); break;
+        }
+    }
+}
+
+template <int FMT>
+static int launch_gemm_fmt(const moe_grouped_args* a, hipStream_t stream) {
+    constexpr int BK = BTraits<FMT>::BK;
+    GemmParams P;
+    P.x = static_cast<const uint16_t*>(a->x);
+    P.w = static_cast<const uint8_t*>(a->weight);
+    P.scale = a->scale;
+    P.offset = static_cast<const uint16_t*>(a->offset);
+    P.gl = a->group_list;
+    P.y = static_cast<uint16_t*>(a->y);
+    P.M = a->M; P.K = (int)a->K; P.N = (int)a->N; P.G = (int)a->G; P.scale_rows = (int)a->scale_rows;
+
+    const size_t lds = (size_t)2 * 16 * GM_MT_MAX * (BK / 8) * 16 + ((size_t)a->G + 1) * sizeof(int);
+    if (lds > 160 * 1024 - 2048) return MOE_ERR_TOO_LARGE;
+    static bool attr_set = false;  // idempotent; a race only repeats the same call
+    if (!attr_set) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(&grouped_gemm_kernel<FMT>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 2048) != hipSuccess)
+            return MOE_ERR_LAUNCH;
+        attr_set = true;
+    }
+    int dev = 0, cus = 256;
+    if (hipGetDevice(&dev) != hipSuccess) return MOE_ERR_NO_DEVICE;
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return MOE_ERR_NO_DEVICE;
+    // upper bound on the tile count without reading group_list: every expert adds at most
+    // one partly filled chunk
+    const int64_t max_chunks = a->M / (16 * GM_MT_MAX) + a->G;
+    const int64_t max_tiles = max_chunks * (a->N / GM_BN);
+    // a multiple of 8 so that the XCD-aware order covers every tile index
+    const int64_t want = max_tiles < cus ? max_tiles : cus;
+    const int64_t grid = want > 0 ? (want + 7) / 8 * 8 : 8;
+    hipLaunchKernelGGL((grouped_gemm_kernel<FMT>), dim3((unsigned)grid), dim3(GM_THREADS), lds, stream, P);
+    return hipGetLastError() == hipSuccess ? MOE_OK : MOE_ERR_LAUNCH;
+}
+
+int launch_grouped_gemm(const moe_grouped_args* a, hipStream_t stream) {
+    switch (a->format) {
+        case MOE_FMT_FP4_REF: return launch_gemm_fmt<MOE_FMT_FP4_REF>(a, stream);
+        case MOE_FMT_FP8_REF: return launch_gemm_fmt<MOE_FMT_FP8_REF>(a, stream);
+        case MOE_FMT_INT8: return launch_gemm_fmt<MOE_FMT_INT8>(a, stream);
+        case MOE_FMT_INT4: return launch_gemm_fmt<MOE_FMT_INT4>(a, stream);
+        case MOE_FMT_FP4_B32: return launch_gemm_fmt<MOE_FMT_FP4_B32>(a, stream);
+        case MOE_FMT_BF16: return launch_gemm_fmt<MOE_FMT_BF16>(a, stream);
+        default: return MOE_ERR_BAD_FORMAT;
+    }
+}
+
+}  // namespace moe

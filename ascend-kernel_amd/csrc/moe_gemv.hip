@@ -1,0 +1,418 @@
+// Grouped GEMV for MoE decode on gfx950 (few rows per expert).  HBM bound: every
+// weight byte of an expert that owns at least one row is read exactly once per
+// group of 4 rows; experts without rows cost one group_list read.  No MFMA: wide
+// vector loads, packed-bf16 dot products, wavefront shuffles for the reductions.
+// Replaces grouped_soft_gemv (grouped_soft_gemv/op_kernel/grouped_soft_gemv.h:235-293,
+// gemv_impl.h:201-398).  Unlike the reference, more than 4 rows per expert are
+// accepted: rows are taken 4 at a time.
+//
+// Numerics (gemv_impl.h:147-199): weights are decode * scale in fp32, NOT rounded
+// to bf16; fp32 accumulation; one RNE to bf16 at the end (grouped_soft_gemv.h:218-233).
+#include "moe_device.h"
+#include "moe_internal.h"
+
+namespace moe {
+
+constexpr int GV_ROWS = 4;        // activation rows per pass (MAX_BSZ of the reference)
+constexpr int GV_KC = 8192;       // k elements of x staged in LDS per pass (4 rows -> 64 KiB)
+
+__device__ __forceinline__ float dot2_bf16(uint32_t a, uint32_t b, float c) {
+    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, a), __builtin_bit_cast(bf16x2_t, b), c,
+                                           false);
+}
+
+__device__ __forceinline__ void group_rows(const int64_t* gl, int g, int64_t M, int64_t& start, int64_t& end) {
+    start = g ? gl[g - 1] : 0;
+    end = gl[g];
+    if (start < 0) start = 0;
+    if (end > M) end = M;
+}
+
+// ---------------------------------------------------------------------------------
+// K-contiguous containers: MOE_FMT_BF16 [G,N,K] and MOE_FMT_FP4_B32 [G,N,K/2].
+// A workgroup owns 64 weight rows (n) of one expert; each wavefront takes 8 rows at
+// a time and all of K: a lane reads CH consecutive k (16 bytes) of each of the 8
+// rows per step, so a step has 8 independent 1 KiB loads in flight per wavefront.
+// x (<= 4 rows) is staged once in LDS.
+// ---------------------------------------------------------------------------------
+constexpr int GVK_NR_WG = 64;
+constexpr int GVK_NRW = 8;
+
+template <int FMT>
+struct KMajor;
+template <>
+struct KMajor<MOE_FMT_BF16> {
+    static constexpr int CH = 8;  // k per lane per step (16 B of weights)
+};
+template <>
+struct KMajor<MOE_FMT_FP4_B32> {
+    static constexpr int CH = 32;  // one scale block (16 B of codes)
+};
+
+// LDS position (in 16-byte units) of the 8 k starting at k8*8, laid out so that the
+// lanes of a wavefront read consecutive units whatever CH is.
+template <int CH>
+__device__ __forceinline__ int xs_unit(int k8) {
+    constexpr int U = CH / 8;  // units per lane per step
+    if (U == 1) return k8;
+    const int lane_k = k8 / U, c = k8 % U;
+    return ((lane_k >> 6) * U + c) * 64 + (lane_k & 63);
+}
+
+template <int FMT, int MG>
+__device__ __forceinline__ void gemv_kmajor_rows(const uint8_t* __restrict__ wg, const uint16_t* __restrict__ sg,
+                                                 const uint16_t* __restrict__ x, uint16_t* __restrict__ y,
+                                                 u32x4_t* xs, int64_t row0, int n0, int N, int K) {
+    constexpr int CH = KMajor<FMT>::CH;
+    constexpr int U = CH / 8;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int nchunks = (K + GV_KC - 1) / GV_KC;
+    const int64_t wrow_bytes = FMT == MOE_FMT_BF16 ? (int64_t)K * 2 : (int64_t)K / 2;
+
+    for (int it = 0; it < GVK_NR_WG / (4 * GVK_NRW); ++it) {
+        const int n = n0 + (it * 4 + wave) * GVK_NRW;
+        float acc[GVK_NRW][MG];
+#pragma unroll
+        for (int j = 0; j < GVK_NRW; ++j)
+#pragma unroll
+            for (int r = 0; r < MG; ++r) acc[j][r] = 0.f;
+
+        for (int c = 0; c < nchunks; ++c) {
+            const int kc0 = c * GV_KC;
+            const int klen = min(GV_KC, K - kc0);
+            if (nchunks > 1 || it == 0) {
+                __syncthreads();
+                for (int i = threadIdx.x; i < MG * (klen / 8); i += 256) {
+                    const int r = i / (klen / 8), k8 = i % (klen / 8);
+                    xs[r * (GV_KC / 8) + xs_unit<CH>(k8)] =
+                        *reinterpret_cast<const u32x4_t*>(x + (row0 + r) * (int64_t)K + kc0 + k8 * 8);
+                }
+                __syncthreads();
+            }
+            for (int k = lane * CH; k < klen; k += 64 * CH) {
+                u32x4_t w[GVK_NRW];
+#pragma unroll
+                for (int j = 0; j < GVK_NRW; ++j) {
+                    const int nn = min(n + j, N - 1);
+                    const uint8_t* p = wg + nn * wrow_bytes + (FMT == MOE_FMT_BF16 ? (int64_t)(kc0 + k) * 2
+                                                                                    : (int64_t)(kc0 + k) / 2);
+                    w[j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(p));
+                }
+                u32x4_t xv[MG][U];
+#pragma unroll
+                for (int r = 0; r < MG; ++r)
+#pragma unroll
+                    for (int u = 0; u < U; ++u) xv[r][u] = xs[r * (GV_KC / 8) + xs_unit<CH>(k / 8 + u)];
+
+                if (FMT == MOE_FMT_BF16) {
+#pragma unroll
+                    for (int j = 0; j < GVK_NRW; ++j)
+#pragma unroll
+                        for (int r = 0; r < MG; ++r)
+#pragma unroll
+                            for (int d = 0; d < 4; ++d) acc[j][r] = dot2_bf16(w[j][d], xv[r][0][d], acc[j][r]);
+                } else {
+#pragma unroll
+                    for (int j = 0; j < GVK_NRW; ++j) {
+                        const int nn = min(n + j, N - 1);
+                        const float s = bf16_bits_to_f32(sg[(int64_t)nn * (K / 32) + (kc0 + k) / 32]);
+                        float part[MG];
+#pragma unroll
+                        for (int r = 0; r < MG; ++r) part[r] = 0.f;
+#pragma unroll
+                        for (int d = 0; d < 4; ++d) {
+                            // exact e2m1 -> bf16 pairs (scale 1.0); the block scale is applied to the
+                            // 32-element partial sum
+                            uint32_t p0 = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w[j][d], 1.0f, 0));
+                            uint32_t p1 = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w[j][d], 1.0f, 1));
+                            uint32_t p2 = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w[j][d], 1.0f, 2));
+                            uint32_t p3 = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w[j][d], 1.0f, 3));
+#pragma unroll
+                            for (int r = 0; r < MG; ++r) {
+                                part[r] = dot2_bf16(p0, xv[r][d][0], part[r]);
+                                part[r] = dot2_bf16(p1, xv[r][d][1], part[r]);
+                                part[r] = dot2_bf16(p2, xv[r][d][2], part[r]);
+                                part[r] = dot2_bf16(p3, xv[r][d][3], part[r]);
+                            }
+                        }
+#pragma unroll
+                        for (int r = 0; r < MG; ++r) acc[j][r] = fmaf(part[r], s, acc[j][r]);
+                    }
+                }
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < GVK_NRW; ++j)
+#pragma unroll
+            for (int r = 0; r < MG; ++r) {
+                const float v = wave_reduce_sum(acc[j][r]);
+                if (lane == 0 && n + j < N) y[(row0 + r) * (int64_t)N + n + j] = (uint16_t)(pack_bf16_rne(v, 0.f) & 0xffffu);
+            }
+    }
+}
+
+template <int FMT>
+__global__ __launch_bounds__(256) void gemv_kmajor_kernel(const uint16_t* __restrict__ x,
+                                                          const uint8_t* __restrict__ w,
+                                                          const uint16_t* __restrict__ scale,
+                                                          const int64_t* __restrict__ gl, uint16_t* __restrict__ y,
+                                                          int64_t M, int K, int N) {
+    extern __shared__ u32x4_t xs[];
+    const int g = blockIdx.y, n0 = blockIdx.x * GVK_NR_WG;
+    int64_t start, end;
+    group_rows(gl, g, M, start, end);
+    if (end <= start) return;
+    const uint8_t* wg = w + (int64_t)g * N * (FMT == MOE_FMT_BF16 ? (int64_t)K * 2 : (int64_t)K / 2);
+    const uint16_t* sg = FMT == MOE_FMT_BF16 ? nullptr : scale + (int64_t)g * N * (K / 32);
+    for (int64_t row0 = start; row0 < end; row0 += GV_ROWS) {
+        const int mg = (int)min((int64_t)GV_ROWS, end - row0);
+        switch (mg) {
+            case 1: gemv_kmajor_rows<FMT, 1>(wg, sg, x, y, xs, row0, n0, N, K); break;
+            case 2: gemv_kmajor_rows<FMT, 2>(wg, sg, x, y, xs, row0, n0, N, K); break;
+            case 3: gemv_kmajor_rows<FMT, 3>(wg, sg, x, y, xs, row0, n0, N, K); break;
+            default: gemv_kmajor_rows<FMT, 4>(wg, sg, x, y, xs, row0, n0, N, K); break;
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------
+// N-contiguous containers: the reference's "fp4" (pre-shuffled) and "fp8" layouts and
+// plain int4.  A workgroup owns 256 columns of one expert; K is split across the
+// lanes of a wavefront and across the 4 wavefronts (split-K), each thread keeping
+// fp32 accumulators for the columns its 16-byte loads cover; partial sums are
+// combined with wavefront shuffles, then across wavefronts through LDS.
+// ---------------------------------------------------------------------------------
+template <int FMT>
+struct NMajor;
+template <>
+struct NMajor<MOE_FMT_FP8_REF> {
+    static constexpr int NC = 16;      // columns per 16-byte load
+    static constexpr int KSTEP = 16;   // k rows covered by the workgroup per step
+    static constexpr int SHUF_LO = 16; // lane bits >= this select the k slice
+};
+template <>
+struct NMajor<MOE_FMT_INT4> {
+    static constexpr int NC = 32;
+    static constexpr int KSTEP = 32;
+    static constexpr int SHUF_LO = 8;
+};
+template <>
+struct NMajor<MOE_FMT_FP4_REF> {
+    static constexpr int NC = 8;       // 8 columns x 4 k per 16-byte load
+    static constexpr int KSTEP = 64;   // one 64(k) x 128(byte) tile per step
+    static constexpr int SHUF_LO = 0;  // lane bit 0 selects the k half
+};
+
+template <int FMT, int MG>
+__device__ __forceinline__ void gemv_nmajor_rows(const uint8_t* __restrict__ wg, const void* __restrict__ sgv,
+                                                 const uint16_t* __restrict__ x, uint16_t* __restrict__ y,
+                                                 uint16_t* xs, float* red, int64_t row0, int n0, int N, int K,
+                                                 int scale_rows) {
+    using T = NMajor<FMT>;
+    constexpr int NC = T::NC;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+
+    __syncthreads();
+    for (int i = tid; i < MG * (K / 8); i += 256) {
+        const int r = i / (K / 8), k8 = i % (K / 8);
+        reinterpret_cast<u32x4_t*>(xs)[r * (K / 8) + k8] =
+            *reinterpret_cast<const u32x4_t*>(x + (row0 + r) * (int64_t)K + k8 * 8);
+    }
+    __syncthreads();
+
+    float acc[MG][NC];
+#pragma unroll
+    for (int r = 0; r < MG; ++r)
+#pragma unroll
+        for (int c = 0; c < NC; ++c) acc[r][c] = 0.f;
+
+    int ncol0;  // first column (relative to n0) of this thread's accumulators
+    if (FMT == MOE_FMT_FP8_REF) {
+        const int cn = tid & 15, kk = tid >> 4;
+        ncol0 = cn * 16;
+        const float* sg = static_cast<const float*>(sgv);
+        const int sn = N / 128;
+        for (int k = kk; k < K; k += 16) {
+            const u32x4_t wv = __builtin_nontemporal_load(
+                reinterpret_cast<const u32x4_t*>(wg + (int64_t)k * N + n0 + ncol0));
+            const float s = sg[(k >> 7) * sn + ((n0 + ncol0) >> 7)];
+            float xr[MG];
+#pragma unroll
+            for (int r = 0; r < MG; ++r) xr[r] = bf16_bits_to_f32(xs[r * K + k]);
+#pragma unroll
+            for (int c = 0; c < 16; ++c) {
+                const float wf = e4m3_ref_to_f32((wv[c >> 2] >> (8 * (c & 3))) & 0xffu) * s;
+#pragma unroll
+                for (int r = 0; r < MG; ++r) acc[r][c] = fmaf(xr[r], wf, acc[r][c]);
+            }
+        }
+    } else if (FMT == MOE_FMT_INT4) {
+        const int cn = tid & 7, kk = tid >> 3;
+        ncol0 = cn * 32;
+        const uint16_t* sg = static_cast<const uint16_t*>(sgv);
+        const int gs = K / scale_rows;
+        for (int k = kk; k < K; k += 32) {
+            const u32x4_t wv = __builtin_nontemporal_load(
+                reinterpret_cast<const u32x4_t*>(wg + (int64_t)k * (N / 2) + (n0 + ncol0) / 2));
+            const uint16_t* sp = sg + (int64_t)(k / gs) * N + n0 + ncol0;
+            float xr[MG];
+#pragma unroll
+            for (int r = 0; r < MG; ++r) xr[r] = bf16_bits_to_f32(xs[r * K + k]);
+#pragma unroll
+            for (int c8 = 0; c8 < 4; ++c8) {
+                const u32x4_t sv = *reinterpret_cast<const u32x4_t*>(sp + c8 * 8);
+#pragma unroll
+                for (int c = 0; c < 8; ++c) {
+                    const int q = (int)((wv[c8] >> (4 * c)) & 15u) - 8;
+                    const uint32_t sb = sv[c >> 1];
+                    const float wf = (float)q * ((c & 1) ? bf16_hi(sb) : bf16_lo(sb));
+#pragma unroll
+                    for (int r = 0; r < MG; ++r) acc[r][c8 * 8 + c] = fmaf(xr[r], wf, acc[r][c8 * 8 + c]);
+                }
+            }
+        }
+    } else {  // MOE_FMT_FP4_REF
+        // Destination row R = j<<5 | i<<3 | p of tile (a, t) holds k = 64a + 16i + 8j + [0,8)
+        // and n = 256t + 32p + [0,32); its 16-byte unit u holds k offsets 4(u&1) + [0,4)
+        // (one dword each) for the 8 columns 8(u>>1) + [0,8).
+        const int u = tid & 7, rs = tid >> 3;  // rs in [0,32): R = rs + 32*jj
+        const int p = rs & 7, i = rs >> 3, q = u >> 1, h = u & 1;
+        ncol0 = 32 * p + 8 * q;
+        const uint16_t* sg = static_cast<const uint16_t*>(sgv);
+        const int64_t nb = N / 2;
+        for (int a = 0; a < K / 64; ++a) {
+#pragma unroll
+            for (int jj = 0; jj < 2; ++jj) {
+                const int R = rs + 32 * jj;
+                const u32x4_t wv = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(
+                    wg + (int64_t)(a * 64 + R) * nb + (n0 / 2) + 16 * u));
+                const int kbase = 64 * a + 16 * i + 8 * jj + 4 * h;
+                const u32x4_t sv = *reinterpret_cast<const u32x4_t*>(sg + (int64_t)(kbase >> 4) * N + n0 + ncol0);
+#pragma unroll
+                for (int d = 0; d < 4; ++d) {
+                    float xr[MG];
+#pragma unroll
+                    for (int r = 0; r < MG; ++r) xr[r] = bf16_bits_to_f32(xs[r * K + kbase + d]);
+                    const f32x2_t v0 = e2m1_pair_to_f32<0>(wv[d]), v1 = e2m1_pair_to_f32<1>(wv[d]);
+                    const f32x2_t v2 = e2m1_pair_to_f32<2>(wv[d]), v3 = e2m1_pair_to_f32<3>(wv[d]);
+                    const float wf[8] = {v0[0] * bf16_lo(sv[0]), v0[1] * bf16_hi(sv[0]), v1[0] * bf16_lo(sv[1]),
+                                         v1[1] * bf16_hi(sv[1]), v2[0] * bf16_lo(sv[2]), v2[1] * bf16_hi(sv[2]),
+                                         v3[0] * bf16_lo(sv[3]), v3[1] * bf16_hi(sv[3])};
+#pragma unroll
+                    for (int c = 0; c < 8; ++c)
+#pragma unroll
+                        for (int r = 0; r < MG; ++r) acc[r][c] = fmaf(xr[r], wf[c], acc[r][c]);
+                }
+            }
+        }
+    }
+
+    // combine the k slices held by different lanes, then by different wavefronts
+#pragma unroll
+    for (int r = 0; r < MG; ++r)
+#pragma unroll
+        for (int c = 0; c < NC; ++c) {
+            float v = acc[r][c];
+            if (FMT == MOE_FMT_FP4_REF) {
+                v += __shfl_xor(v, 1, 64);
+            } else {
+#pragma unroll
+                for (int off = 32; off >= T::SHUF_LO; off >>= 1) v += __shfl_xor(v, off, 64);
+            }
+            acc[r][c] = v;
+        }
+    const bool writer = FMT == MOE_FMT_FP4_REF ? ((lane & 1) == 0) : (lane < T::SHUF_LO);
+    const int wcol0 = FMT == MOE_FMT_FP4_REF ? 32 * (lane >> 3) + 8 * ((lane & 7) >> 1) : ncol0;
+    if (writer) {
+#pragma unroll
+        for (int r = 0; r < MG; ++r)
+#pragma unroll
+            for (int c = 0; c < NC; ++c) red[(wave * GV_ROWS + r) * 256 + wcol0 + c] = acc[r][c];
+    }
+    __syncthreads();
+    // FP4_REF: the 4 wavefronts hold different i (k), the same columns; others: different kk
+#pragma unroll
+    for (int r = 0; r < MG; ++r) {
+        const float v = red[(0 * GV_ROWS + r) * 256 + tid] + red[(1 * GV_ROWS + r) * 256 + tid] +
+                        red[(2 * GV_ROWS + r) * 256 + tid] + red[(3 * GV_ROWS + r) * 256 + tid];
+        y[(row0 + r) * (int64_t)N + n0 + tid] = (uint16_t)(pack_bf16_rne(v, 0.f) & 0xffffu);
+    }
+}
+
+template <int FMT>
+__global__ __launch_bounds__(256) void gemv_nmajor_kernel(const uint16_t* __restrict__ x,
+                                                          const uint8_t* __restrict__ w,
+                                                          const void* __restrict__ scale,
+                                                          const int64_t* __restrict__ gl, uint16_t* __restrict__ y,
+                                                          int64_t M, int K, int N, int scale_rows) {
+    extern __shared__ u32x4_t smem[];
+    float* red = reinterpret_cast<float*>(smem);                       // [4 waves][4 rows][256]
+    uint16_t* xs = reinterpret_cast<uint16_t*>(red + 4 * GV_ROWS * 256);  // [4 rows][K]
+    const int g = blockIdx.y, n0 = blockIdx.x * 256;
+    int64_t start, end;
+    group_rows(gl, g, M, start, end);
+    if (end <= start) return;
+    const uint8_t* wg;
+    const void* sg;
+    if (FMT == MOE_FMT_FP8_REF) {
+        wg = w + (int64_t)g * K * N;
+        sg = static_cast<const float*>(scale) + (int64_t)g * (K / 128) * (N / 128);
+    } else {
+        wg = w + (int64_t)g * K * (N / 2);
+        sg = static_cast<const uint16_t*>(scale) + (int64_t)g * scale_rows * N;
+    }
+    for (int64_t row0 = start; row0 < end; row0 += GV_ROWS) {
+        const int mg = (int)min((int64_t)GV_ROWS, end - row0);
+        switch (mg) {
+            case 1: gemv_nmajor_rows<FMT, 1>(wg, sg, x, y, xs, red, row0, n0, N, K, scale_rows); break;
+            case 2: gemv_nmajor_rows<FMT, 2>(wg, sg, x, y, xs, red, row0, n0, N, K, scale_rows); break;
+            case 3: gemv_nmajor_rows<FMT, 3>(wg, sg, x, y, xs, red, row0, n0, N, K, scale_rows); break;
+            default: gemv_nmajor_rows<FMT, 4>(wg, sg, x, y, xs, red, row0, n0, N, K, scale_rows); break;
+        }
+    }
+}
+
+template <int FMT>
+static int launch_kmajor(const moe_grouped_args* a, hipStream_t stream) {
+    const int kc = (int)(a->K < GV_KC ? a->K : GV_KC);
+    const size_t lds = (size_t)GV_ROWS * GV_KC / 8 * 16;
+    (void)kc;
+    dim3 grid((unsigned)((a->N + GVK_NR_WG - 1) / GVK_NR_WG), (unsigned)a->G);
+    hipLaunchKernelGGL((gemv_kmajor_kernel<FMT>), grid, dim3(256), lds, stream,
+                       static_cast<const uint16_t*>(a->x), static_cast<const uint8_t*>(a->weight),
+                       static_cast<const uint16_t*>(a->scale), a->group_list, static_cast<uint16_t*>(a->y), a->M,
+                       (int)a->K, (int)a->N);
+    return hipGetLastError() == hipSuccess ? MOE_OK : MOE_ERR_LAUNCH;
+}
+
+template <int FMT>
+static int launch_nmajor(const moe_grouped_args* a, hipStream_t stream) {
+    const size_t lds = (size_t)4 * GV_ROWS * 256 * 4 + (size_t)GV_ROWS * a->K * 2;
+    if (lds > 160 * 1024) return MOE_ERR_TOO_LARGE;
+    static bool attr_set = false;  // idempotent; a race only repeats the same call
+    if (!attr_set) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(&gemv_nmajor_kernel<FMT>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) != hipSuccess)
+            return MOE_ERR_LAUNCH;
+        attr_set = true;
+    }
+    dim3 grid((unsigned)(a->N / 256), (unsigned)a->G);
+    hipLaunchKernelGGL((gemv_nmajor_kernel<FMT>), grid, dim3(256), lds, stream,
+                       static_cast<const uint16_t*>(a->x), static_cast<const uint8_t*>(a->weight), a->scale,
+                       a->group_list, static_cast<uint16_t*>(a->y), a->M, (int)a->K, (int)a->N,
+                       (int)a->scale_rows);
+    return hipGetLastError() == hipSuccess ? MOE_OK : MOE_ERR_LAUNCH;
+}
+
+int launch_grouped_gemv(const moe_grouped_args* a, hipStream_t stream) {
+    switch (a->format) {
+        case MOE_FMT_BF16: return launch_kmajor<MOE_FMT_BF16>(a, stream);
+        case MOE_FMT_FP4_B32: return launch_kmajor<MOE_FMT_FP4_B32>(a, stream);
+        case MOE_FMT_FP4_REF: return launch_nmajor<MOE_FMT_FP4_REF>(a, stream);
+        case MOE_FMT_FP8_REF: return launch_nmajor<MOE_FMT_FP8_REF>(a, stream);
+        case MOE_FMT_INT4: return launch_nmajor<MOE_FMT_INT4>(a, stream);
+        default: return MOE_ERR_BAD_FORMAT;
+    }
+}
+
+}  // namespace moe

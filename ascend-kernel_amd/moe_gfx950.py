@@ -1,0 +1,98 @@
+"""ctypes view of the C ABI in include/moe_gfx950.h (libmoe_gfx950.so).
+
+This is the torch-free way into the kernels: raw device pointers, sizes and a HIP
+stream handle.  `cinfer_ascendc` (the drop-in module with the reference's Python
+API) sits on the same ABI.  There is no CPU fallback: if the library has not been
+built, importing this module raises.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libmoe_gfx950.so")
+
+MOE_OK = 0
+FMT_FP4_REF, FMT_FP8_REF, FMT_INT8, FMT_INT4, FMT_FP4_B32, FMT_BF16 = range(6)
+ERR_NULL_POINTER, ERR_BAD_FORMAT, ERR_BAD_SHAPE, ERR_BAD_ALIGNMENT, ERR_TOO_LARGE, ERR_LAUNCH, ERR_NO_DEVICE = (
+    -1, -2, -3, -4, -5, -6, -7)
+
+# every symbol include/moe_gfx950.h declares
+SYMBOLS = (
+    "moe_abi_version", "moe_strerror", "moe_format_from_compute_type",
+    "moe_dequant_fp4_bf16_validate", "moe_grouped_gemm_validate", "moe_grouped_gemv_validate",
+    "moe_dequant_fp4_bf16_workspace_bytes", "moe_grouped_gemm_workspace_bytes", "moe_grouped_gemv_workspace_bytes",
+    "moe_dequant_fp4_bf16", "moe_grouped_gemm", "moe_grouped_gemv",
+)
+
+
+class GroupedArgs(ctypes.Structure):
+    _fields_ = [("x", ctypes.c_void_p), ("weight", ctypes.c_void_p), ("scale", ctypes.c_void_p),
+                ("offset", ctypes.c_void_p), ("group_list", ctypes.c_void_p), ("y", ctypes.c_void_p),
+                ("M", ctypes.c_int64), ("K", ctypes.c_int64), ("N", ctypes.c_int64), ("G", ctypes.c_int64),
+                ("scale_rows", ctypes.c_int64), ("format", ctypes.c_int32), ("reserved", ctypes.c_int32)]
+
+
+class DequantArgs(ctypes.Structure):
+    _fields_ = [("codes", ctypes.c_void_p), ("scale", ctypes.c_void_p), ("out", ctypes.c_void_p),
+                ("rows", ctypes.c_int64), ("cols", ctypes.c_int64), ("block", ctypes.c_int32),
+                ("reserved", ctypes.c_int32)]
+
+
+if not os.path.exists(LIB_PATH):
+    raise ImportError(f"{LIB_PATH} is missing: build it with `python ascend-kernel_amd/build.py` "
+                      "(there is no CPU fallback)")
+
+lib = ctypes.CDLL(LIB_PATH)
+lib.moe_abi_version.restype = ctypes.c_int
+lib.moe_strerror.restype = ctypes.c_char_p
+lib.moe_strerror.argtypes = [ctypes.c_int]
+lib.moe_format_from_compute_type.restype = ctypes.c_int
+lib.moe_format_from_compute_type.argtypes = [ctypes.c_char_p]
+for _n, _t in (("dequant_fp4_bf16", DequantArgs), ("grouped_gemm", GroupedArgs), ("grouped_gemv", GroupedArgs)):
+    getattr(lib, f"moe_{_n}_validate").restype = ctypes.c_int
+    getattr(lib, f"moe_{_n}_validate").argtypes = [ctypes.POINTER(_t)]
+    getattr(lib, f"moe_{_n}_workspace_bytes").restype = ctypes.c_size_t
+    getattr(lib, f"moe_{_n}_workspace_bytes").argtypes = [ctypes.POINTER(_t)]
+    getattr(lib, f"moe_{_n}").restype = ctypes.c_int
+    getattr(lib, f"moe_{_n}").argtypes = [ctypes.POINTER(_t), ctypes.c_void_p]
+
+
+class MoeError(RuntimeError):
+    def __init__(self, status: int, op: str):
+        self.status = status
+        super().__init__(f"{op}: {strerror(status)} (moe_status {status})")
+
+
+def strerror(status: int) -> str:
+    return lib.moe_strerror(status).decode()
+
+
+def format_from_compute_type(name: str) -> int:
+    return lib.moe_format_from_compute_type(name.encode())
+
+
+def _check(rc: int, op: str) -> None:
+    if rc != MOE_OK:
+        raise MoeError(rc, op)
+
+
+def dequant_fp4_bf16(codes_ptr: int, scale_ptr: int, out_ptr: int, rows: int, cols: int, block: int = 32,
+                     stream: int = 0) -> None:
+    a = DequantArgs(codes_ptr, scale_ptr, out_ptr, rows, cols, block, 0)
+    _check(lib.moe_dequant_fp4_bf16(ctypes.byref(a), ctypes.c_void_p(stream)), "moe_dequant_fp4_bf16")
+
+
+def grouped_args(fmt: int, x_ptr: int, w_ptr: int, scale_ptr, offset_ptr, gl_ptr: int, y_ptr: int, M: int, K: int,
+                 N: int, G: int, scale_rows: int = 1) -> GroupedArgs:
+    return GroupedArgs(x_ptr, w_ptr, scale_ptr or None, offset_ptr or None, gl_ptr, y_ptr, M, K, N, G, scale_rows,
+                       fmt, 0)
+
+
+def grouped_gemm(args: GroupedArgs, stream: int = 0) -> None:
+    _check(lib.moe_grouped_gemm(ctypes.byref(args), ctypes.c_void_p(stream)), "moe_grouped_gemm")
+
+
+def grouped_gemv(args: GroupedArgs, stream: int = 0) -> None:
+    _check(lib.moe_grouped_gemv(ctypes.byref(args), ctypes.c_void_p(stream)), "moe_grouped_gemv")

@@ -1,0 +1,149 @@
+/*
+ * moe_gfx950.h -- C ABI of libmoe_gfx950.so: MI355X (gfx950) kernels for the three
+ * MoE inference ops that QingCheng-AI/ascend-kernel exposes as `cinfer_ascendc`.
+ *
+ * Plain C: raw device pointers, sizes, an opaque stream handle.  No torch types.
+ * Every launch is asynchronous on the given stream, never synchronizes the
+ * device, never copies group_list to the host, allocates nothing and keeps no
+ * state between calls (re-entrant).  All functions return MOE_OK (0) or a
+ * negative moe_status; nothing throws across this boundary.
+ *
+ * What each entry point replaces in the reference (paths relative to its tree):
+ *   moe_grouped_gemm            aclnnGroupedMatmulAntiquant{GetWorkspaceSize,}
+ *                               as called at grouped_gemm/src/grouped_gemm.cpp:145-157,
+ *                               i.e. kernel grouped_matmul_antiquant,
+ *                               grouped_gemm/op_kernel/grouped_matmul_antiquant.cpp:146-162
+ *   moe_grouped_gemv            aclnnGroupedSoftGemv{GetWorkspaceSize,} as called at
+ *                               grouped_soft_gemv/src/grouped_soft_gemv.cpp:141-150,
+ *                               i.e. kernel grouped_soft_gemv,
+ *                               grouped_soft_gemv/op_kernel/grouped_soft_gemv.cpp:24-37
+ *   moe_dequant_fp4_bf16        phase 1 of the GEMM kernel made a stand-alone op:
+ *                               CastWeightProcess, grouped_gemm/op_kernel/grouped_matmul_antiquant.h:537-662
+ *                               + antiquantProcess, grouped_gemm/op_kernel/antiquant_impl.h:146-208
+ *   moe_*_validate              the shape/dtype checks of op_host tiling,
+ *                               grouped_gemm/op_host/grouped_matmul_antiquant_tiling.cpp:246-313
+ *   moe_*_workspace_bytes       the GetWorkspaceSize half of the aclnn pair
+ *                               (grouped_gemm/src/grouped_gemm.cpp:145-154); always 0 here
+ *   moe_format_from_compute_type  the computeType string switch,
+ *                               grouped_gemm/src/grouped_gemm.cpp:129-135
+ */
+#ifndef MOE_GFX950_H
+#define MOE_GFX950_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MOE_GFX950_ABI_VERSION 1
+
+/* hipStream_t, passed opaquely so that this header needs no HIP include. */
+typedef void *moe_stream_t;
+
+typedef enum moe_status {
+    MOE_OK = 0,
+    MOE_ERR_NULL_POINTER = -1,   /* a required pointer is NULL                        */
+    MOE_ERR_BAD_FORMAT = -2,     /* unknown weight format / computeType               */
+    MOE_ERR_BAD_SHAPE = -3,      /* negative size, or a size the format cannot hold   */
+    MOE_ERR_BAD_ALIGNMENT = -4,  /* K/N/cols not a multiple the kernels need, or a
+                                    pointer not aligned to 16 bytes                   */
+    MOE_ERR_TOO_LARGE = -5,      /* M, K, N or G beyond int32 (reference limit,
+                                    grouped_matmul_antiquant_tiling.cpp:260-264)       */
+    MOE_ERR_LAUNCH = -6,         /* hipLaunchKernel reported an error                 */
+    MOE_ERR_NO_DEVICE = -7       /* no gfx950 device / wrong architecture             */
+} moe_status;
+
+/*
+ * Weight containers.  G experts; logical weight of expert g is B[g][k][n] with
+ * y = x . dequant(B).  "scale_rows" below is scale.shape[-2].
+ *
+ * MOE_FMT_FP4_REF  reference computeType "fp4": int8 [G, K, N/2], e2m1 codes packed
+ *                  along N (low nibble = even n) then byte-permuted inside every
+ *                  64(k) x 128(byte) tile exactly as the reference test prepares it
+ *                  (grouped_gemm/test/python/test_group_gemm_fp4.py:105-117, :129-142);
+ *                  scale bf16 [G, K/16, N]; offset ignored (the reference never reads it).
+ *                  K % 64 == 0, N % 256 == 0.
+ * MOE_FMT_FP8_REF  reference computeType "fp8": uint8 [G, K, N] e4m3 bits decoded with
+ *                  the reference's bit trick (0x7F/0xFF give +-480, no NaN);
+ *                  scale fp32 [G, K/128, N/128]; offset ignored.
+ * MOE_FMT_INT8     int8 [G, K, N]; scale bf16 [G, N]; offset bf16 [G, N];
+ *                  W = bf16((float(q) + float(offset)) * float(scale)).
+ * MOE_FMT_INT4     uint8 [G, K, N/2], low nibble = even n, codes 0..15, zero point 8;
+ *                  scale bf16 [G, K/group, N] (group = K / scale_rows, a multiple of 32);
+ *                  W = bf16(float(q - 8) * float(scale)).
+ * MOE_FMT_FP4_B32  uint8 [G, N, K/2] e2m1, K-contiguous, low nibble = even k;
+ *                  scale bf16 [G, N, K/32]; W = bf16(e2m1(code) * float(scale)).
+ *                  One expert is exactly a moe_dequant_fp4_bf16 input of N rows, K cols.
+ * MOE_FMT_BF16     bf16 [G, N, K], K-contiguous; no scale.
+ *
+ * GEMM rounds W to bf16 before the product (reference phase 1); GEMV keeps the
+ * fp32 product un-rounded (grouped_soft_gemv/op_kernel/gemv_impl.h:147-199).
+ */
+typedef enum moe_weight_format {
+    MOE_FMT_FP4_REF = 0,
+    MOE_FMT_FP8_REF = 1,
+    MOE_FMT_INT8 = 2,
+    MOE_FMT_INT4 = 3,
+    MOE_FMT_FP4_B32 = 4,
+    MOE_FMT_BF16 = 5,
+    MOE_FMT_COUNT = 6
+} moe_weight_format;
+
+/* Arguments of both grouped ops.  x, y are row-major bf16; group_list is the
+ * cumulative int64 [G] device tensor of the reference (rows [gl[g-1], gl[g]) belong
+ * to expert g, gl[-1] = 0; rows at or beyond gl[G-1] are not written;
+ * grouped_gemm/op_kernel/grouped_matmul_utils.h:304-320). */
+typedef struct moe_grouped_args {
+    const void *x;             /* bf16 [M, K]                                       */
+    const void *weight;        /* container, see moe_weight_format                  */
+    const void *scale;         /* NULL only for MOE_FMT_BF16                        */
+    const void *offset;        /* read by MOE_FMT_INT8 only; may be NULL otherwise  */
+    const int64_t *group_list; /* device int64 [G], cumulative                      */
+    void *y;                   /* bf16 [M, N]                                       */
+    int64_t M, K, N, G;
+    int64_t scale_rows;        /* scale.shape[-2]; used by FP4_REF (K/16) and INT4  */
+    int32_t format;            /* moe_weight_format                                 */
+    int32_t reserved;          /* must be 0                                         */
+} moe_grouped_args;
+
+/* codes uint8 [rows, cols/2] (even element in the low nibble), scale bf16
+ * [rows, cols/block], out bf16 [rows, cols]; block is 16 or 32.  Bit-exact:
+ * out = RNE_bf16(float(e2m1(code)) * float(scale)), code 8 gives -0.0. */
+typedef struct moe_dequant_args {
+    const void *codes;
+    const void *scale;
+    void *out;
+    int64_t rows, cols;
+    int32_t block;
+    int32_t reserved; /* must be 0 */
+} moe_dequant_args;
+
+int moe_abi_version(void);
+const char *moe_strerror(int status);
+
+/* "fp4" | "fp8" (reference values) | "int8" | "int4" | "fp4_b32" | "bf16";
+ * returns the moe_weight_format or MOE_ERR_BAD_FORMAT. */
+int moe_format_from_compute_type(const char *compute_type);
+
+/* Host-only argument checks (usable without a GPU). */
+int moe_dequant_fp4_bf16_validate(const moe_dequant_args *args);
+int moe_grouped_gemm_validate(const moe_grouped_args *args);
+int moe_grouped_gemv_validate(const moe_grouped_args *args);
+
+/* Device scratch the launch needs: 0 for every op (kept for callers that follow
+ * the reference's two-phase GetWorkspaceSize protocol). */
+size_t moe_dequant_fp4_bf16_workspace_bytes(const moe_dequant_args *args);
+size_t moe_grouped_gemm_workspace_bytes(const moe_grouped_args *args);
+size_t moe_grouped_gemv_workspace_bytes(const moe_grouped_args *args);
+
+/* Launches (validate first, then enqueue on `stream`). */
+int moe_dequant_fp4_bf16(const moe_dequant_args *args, moe_stream_t stream);
+int moe_grouped_gemm(const moe_grouped_args *args, moe_stream_t stream);
+int moe_grouped_gemv(const moe_grouped_args *args, moe_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MOE_GFX950_H */

@@ -1,0 +1,296 @@
+"""GPU parity tests: the HIP kernels, called through the C ABI (and through the
+cinfer_ascendc module), against the CPU oracle on identical seeded inputs.
+
+Bars: FP4 dequant bit-exact; grouped GEMM / GEMV max|d|/max|ref| <= 1e-2 and
+|d| <= 2e-2 * max(1, |ref|), both sides rounded to bf16 (helpers.REL_TOL / ABS_TOL)."""
+import numpy as np
+import pytest
+import torch
+
+import helpers as H
+import oracle
+from oracle import layouts as L
+
+pytestmark = pytest.mark.gpu
+
+
+def _say(msg):
+    print(msg, flush=True)
+
+
+# ------------------------------------------------------------------------ FP4 dequant
+def _dequant_gpu(codes: np.ndarray, scale_bits: np.ndarray, block: int) -> np.ndarray:
+    import moe_gfx950 as mg
+
+    R, C = codes.shape[0], codes.shape[1] * 2
+    d_codes, d_scale = torch.from_numpy(codes).cuda(), H.to_dev(scale_bits)
+    out = torch.full((R, C), 0x7FC0, dtype=torch.int16, device="cuda")
+    mg.dequant_fp4_bf16(d_codes.data_ptr(), d_scale.data_ptr(), out.data_ptr(), R, C, block,
+                        torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    return out.cpu().numpy().view(np.uint16)
+
+
+@pytest.mark.parametrize("R,C,block", [(64, 256, 32), (7, 96, 32), (3, 48, 16), (1, 32, 32), (257, 2048, 32)])
+def test_dequant_bit_exact_small(R, C, block):
+    _say(f"dequant R={R} C={C} block={block}")
+    rng = np.random.default_rng(100 + R)
+    codes = rng.integers(0, 256, (R, C // 2), dtype=np.uint8)
+    scale = H.bits(H.bf16_uniform(rng, 2.0 ** -8, 2.0 ** -2, (R, C // block)))
+    assert np.array_equal(_dequant_gpu(codes, scale, block), oracle.dequant_fp4_bf16(codes, scale, block))
+
+
+def test_dequant_bit_exact_all_codes_and_edge_scales():
+    # every byte value against scales that hit rounding ties, tiny and huge magnitudes, negative scales
+    _say("dequant all codes x edge scales")
+    sc = np.array([0x3F80, 0x3F81, 0x3FFF, 0x0080, 0x0001, 0x7F00, 0xBF80, 0x3C58, 0x4049, 0x0000, 0x8000, 0x3EAB,
+                   0x1234, 0x7E80, 0x00FF, 0x807F], dtype=np.uint16)
+    codes = np.tile(np.arange(256, dtype=np.uint8).reshape(16, 16), (len(sc), 1))  # [16*len, 16] -> 32 cols
+    scale = np.repeat(sc, 16).reshape(-1, 1)
+    got = _dequant_gpu(codes, scale, 32)
+    ref = oracle.dequant_fp4_bf16(codes, scale, 32)
+    assert np.array_equal(got, ref)
+    assert (got[:16][codes[:16] & 0x0F == 8][:0].size == 0)
+    # code 8 is -0.0 whatever the (positive) scale
+    z = _dequant_gpu(np.full((1, 16), 0x88, np.uint8), np.array([[0x3F80]], np.uint16), 32)
+    assert (z == 0x8000).all()
+
+
+def test_dequant_full_size_config():
+    # 7168 x 2048 weight of the benchmark configuration, bit-exact against the oracle
+    _say("dequant 7168x2048")
+    rng = np.random.default_rng(1)
+    codes = rng.integers(0, 256, (7168, 1024), dtype=np.uint8)
+    scale = H.bits(H.bf16_uniform(rng, 2.0 ** -8, 2.0 ** -2, (7168, 64)))
+    assert np.array_equal(_dequant_gpu(codes, scale, 32), oracle.dequant_fp4_bf16(codes, scale, 32))
+
+
+def test_dequant_module_entry_point_and_empty():
+    import cinfer_ascendc
+
+    _say("dequant via module")
+    rng = np.random.default_rng(2)
+    codes = rng.integers(0, 256, (33, 64), dtype=np.uint8)
+    scale = H.bits(H.bf16_uniform(rng, 2.0 ** -8, 2.0 ** -2, (33, 4)))
+    out = torch.empty(33, 128, dtype=torch.bfloat16, device="cuda")
+    cinfer_ascendc.dequant_fp4(weight=torch.from_numpy(codes).cuda(), scale=H.to_dev(scale).view(torch.bfloat16),
+                               output=out)
+    torch.cuda.synchronize()
+    assert np.array_equal(H.bits(out), oracle.dequant_fp4_bf16(codes, scale, 32))
+    cinfer_ascendc.dequant_fp4(torch.empty(0, 64, dtype=torch.uint8, device="cuda"),
+                               torch.empty(0, 4, dtype=torch.bfloat16, device="cuda"),
+                               torch.empty(0, 128, dtype=torch.bfloat16, device="cuda"))
+
+
+# ------------------------------------------------------------------------ grouped GEMM
+GEMM_GROUP_LISTS = {
+    "ref_fp4": [2, 3, 4, 256],        # test_group_gemm_fp4.py:172
+    "ref_fp8": [12, 25, 44, 48],      # test_group_gemm_fp8.py:50
+    "empties": [0, 0, 37, 37, 37, 150, 150, 151],
+    "one_big": [0, 500, 500, 500],    # > 192 rows: several row chunks
+    "all_empty": [0, 0, 0],
+}
+
+
+@pytest.mark.parametrize("fmt", H.FORMATS)
+@pytest.mark.parametrize("gl_name", list(GEMM_GROUP_LISTS))
+def test_gemm_parity_small(fmt, gl_name):
+    gl = GEMM_GROUP_LISTS[gl_name]
+    G, K, N = len(gl), 512, 512
+    _say(f"gemm fmt={fmt} gl={gl_name} G={G} K={K} N={N}")
+    case = H.make_case(fmt, G, K, N, gl, seed=hash((fmt, gl_name)) % 1000, extra_rows=5)
+    got = H.run_cabi(case, H.upload(case), "gemm")
+    ref = H.oracle_out(case)
+    M_used = gl[-1]
+    H.assert_close(got, ref, rows=slice(0, M_used), what=f"{fmt}/{gl_name}")
+    assert (got[M_used:] == 0x7FC0).all(), "rows beyond group_list[-1] were written"
+
+
+@pytest.mark.parametrize("fmt,K,N", [("int4", 7168, 256), ("int8", 4096, 512), ("fp4", 1024, 1024),
+                                     ("fp8", 1536, 768), ("fp4_b32", 7168, 256), ("bf16", 2048, 256),
+                                     ("int4", 2048, 1792)])
+def test_gemm_parity_deep_k_and_wide_n(fmt, K, N):
+    _say(f"gemm deep fmt={fmt} K={K} N={N}")
+    gl = [130, 130, 143, 300, 301]
+    case = H.make_case(fmt, len(gl), K, N, gl, seed=K + N)
+    got = H.run_cabi(case, H.upload(case), "gemm")
+    H.assert_close(got, H.oracle_out(case), what=f"{fmt} K={K} N={N}")
+
+
+def test_gemm_int4_group_size_32_and_64():
+    for group in (32, 64, 256):
+        _say(f"gemm int4 group={group}")
+        case = H.make_case("int4", 3, 512, 256, [20, 20, 77], seed=group, group=group)
+        got = H.run_cabi(case, H.upload(case), "gemm")
+        H.assert_close(got, H.oracle_out(case), what=f"int4 group {group}")
+
+
+def test_gemm_reference_fp4_test_shape_via_module():
+    """The reference's own fp4 GEMM test (test_group_gemm_fp4.py:164-230): G=4, dim 256,
+    block 16, the same weight for every expert, group_list [2,3,4,256], called with its
+    keyword order; checked at the reference's atol 0.15 and at this project's bar."""
+    import cinfer_ascendc
+
+    _say("gemm reference fp4 test shape")
+    dim, block, G = 256, 16, 4
+    g = torch.Generator().manual_seed(0)
+    b = torch.randn(dim, dim // block, block, generator=g)
+    b_s_2 = b.abs().max() / (448 * 6)
+    b_s = torch.clamp(b.amax(dim=2, keepdim=True) / (6 * b_s_2), -448, 448)
+    levels = torch.tensor(L.E2M1_LEVELS)
+    bq = b / (b_s * b_s_2)
+    idx = (bq.abs().unsqueeze(-1) - levels).abs().argmin(-1)          # snap to the e2m1 grid
+    codes = (idx.to(torch.uint8) | ((bq < 0).to(torch.uint8) << 3)).view(dim, dim).numpy()
+    ckpt = np.repeat(L.pack_nibbles_last(codes)[None], G, 0)          # [G, N, K/2]
+    scale_nk = (b_s.view(dim, dim // block) * b_s_2).to(torch.bfloat16)   # merged two-level scale, :86-94
+    w1w3 = L.fp4ref_from_checkpoint(ckpt)
+    new_scale = scale_nk.t().contiguous().unsqueeze(0).repeat(G, 1, 1)    # [G, K/16, N], :185-186
+    x = torch.randn(dim, dim, generator=g).to(torch.bfloat16)
+    expert_tokens = torch.tensor([2, 3, 4, 256], dtype=torch.int64)
+    output = torch.zeros(dim, dim, dtype=torch.bfloat16, device="cuda")
+    cinfer_ascendc.grouped_gemm(
+        x.cuda(), torch.from_numpy(w1w3).cuda(), output=output,
+        antiquantOffsetOptional=torch.zeros_like(new_scale).cuda(), antiquantScaleOptional=new_scale.cuda(),
+        groupListOptional=expert_tokens.cuda(), computeType="fp4")
+    torch.cuda.synchronize()
+    # expected value exactly as the reference test builds it (:199-217), torch on the CPU
+    lut = torch.tensor([0, .5, 1, 1.5, 2, 3, 4, 6, -0., -.5, -1, -1.5, -2, -3, -4, -6], dtype=torch.bfloat16)
+    w = lut[torch.from_numpy(codes.astype(np.int64))]                                     # [N, K]
+    for i in range(dim // block):
+        w[:, i * block:(i + 1) * block] *= scale_nk[:, i].unsqueeze(-1)
+    exp = (x.float() @ w.t().float()).to(torch.bfloat16)
+    assert torch.allclose(exp, output.cpu(), atol=0.15)
+    H.assert_close(H.bits(output), H.bits(exp), what="reference fp4 test")
+
+
+def test_gemm_reference_fp8_test_shape_all_ones_x():
+    """The reference's fp8 GEMM test (test_group_gemm_fp8.py:35-71): G=4, M=48, K=512,
+    N=1536, x = ones, randn fp32 block scales, group_list [12,25,44,48]; with x = 1 the
+    output is the column sums of the dequantized weight."""
+    import cinfer_ascendc
+
+    _say("gemm reference fp8 test shape")
+    rng = np.random.default_rng(3)
+    G, M, K, N = 4, 48, 512, 1536
+    w = rng.integers(0, 255, (G, K, N), dtype=np.uint8)
+    scale = rng.standard_normal((G, 4, 12)).astype(np.float32)
+    gl = [12, 25, 44, 48]
+    out = torch.zeros(M, N, dtype=torch.bfloat16, device="cuda")
+    scale_d = torch.from_numpy(scale).cuda()
+    cinfer_ascendc.grouped_gemm(
+        torch.ones(M, K, dtype=torch.bfloat16, device="cuda"), torch.from_numpy(w).cuda(), output=out,
+        antiquantOffsetOptional=torch.zeros_like(scale_d), antiquantScaleOptional=scale_d,
+        groupListOptional=torch.tensor(gl).cuda(), computeType="fp8")
+    torch.cuda.synchronize()
+    Wd = L.fp8ref_dequant_numpy(w, scale, True).astype(np.float64)
+    exp = np.zeros((M, N))
+    prev = 0
+    for g, end in enumerate(gl):
+        exp[prev:end] = Wd[g].sum(0)
+        prev = end
+    got = out.float().cpu().numpy()
+    assert np.allclose(got, exp, atol=0.02 + 2 ** -8 * np.abs(exp).max())   # reference atol + one bf16 ulp
+    H.assert_close(H.bits(out), oracle.f32_to_bf16_bits(exp.astype(np.float32)), what="reference fp8 test")
+
+
+def test_gemm_linearity_and_determinism():
+    # y(x1 + x2) == y(x1) + y(x2) up to rounding; two launches give identical bits
+    _say("gemm linearity")
+    gl = [100, 260, 300]
+    case = H.make_case("int4", 3, 1024, 512, gl, seed=5)
+    dev = H.upload(case)
+    y1 = H.run_cabi(case, dev, "gemm")
+    assert np.array_equal(y1, H.run_cabi(case, dev, "gemm"))
+    case2 = dict(case)
+    x2 = oracle.f32_to_bf16_bits(oracle.bf16_bits_to_f32(case["x"]) * 2.0)   # exact scaling by 2
+    case2["x"] = x2
+    y2 = H.run_cabi(case2, H.upload(case2), "gemm")
+    assert np.array_equal(oracle.bf16_bits_to_f32(y2), 2.0 * oracle.bf16_bits_to_f32(y1))
+
+
+# ------------------------------------------------------------------------ grouped GEMV
+GEMV_GROUP_LISTS = {
+    "ref": [1, 2, 3, 4],                       # test_group_soft_gemv_fp4.py:172
+    "ragged": [0, 4, 4, 6, 7, 7, 11],
+    "more_than_4": [9, 9, 10],                 # beyond the reference's MAX_BSZ: rows taken 4 at a time
+    "all_empty": [0, 0],
+}
+
+
+@pytest.mark.parametrize("fmt", H.GEMV_FORMATS)
+@pytest.mark.parametrize("gl_name", list(GEMV_GROUP_LISTS))
+def test_gemv_parity_small(fmt, gl_name):
+    gl = GEMV_GROUP_LISTS[gl_name]
+    G, K, N = len(gl), 1024, 512
+    _say(f"gemv fmt={fmt} gl={gl_name}")
+    case = H.make_case(fmt, G, K, N, gl, seed=hash((fmt, gl_name, 1)) % 1000, extra_rows=3)
+    got = H.run_cabi(case, H.upload(case), "gemv")
+    ref = H.oracle_out(case, gemv=True)
+    H.assert_close(got, ref, rows=slice(0, gl[-1]), what=f"gemv {fmt}/{gl_name}")
+    assert (got[gl[-1]:] == 0x7FC0).all()
+
+
+@pytest.mark.parametrize("fmt,K,N", [("bf16", 7168, 2048), ("fp4_b32", 7168, 2048), ("fp4", 7168, 512),
+                                     ("fp8", 7168, 256), ("bf16", 9216, 200), ("fp4_b32", 16384, 64)])
+def test_gemv_parity_decode_shapes(fmt, K, N):
+    _say(f"gemv decode fmt={fmt} K={K} N={N}")
+    gl = [3, 3, 7, 8]
+    case = H.make_case(fmt, 4, K, N, gl, seed=K % 97)
+    got = H.run_cabi(case, H.upload(case), "gemv")
+    H.assert_close(got, H.oracle_out(case, gemv=True), what=f"gemv {fmt} K={K} N={N}")
+
+
+def test_gemv_reference_fp8_test_shape_via_module():
+    """test_group_soft_gemv_fp8.py:37-88: G=4, M=4, K=512, N=1536, x = ones, expected value
+    from fp32 (un-rounded) weights, rtol 0.02."""
+    import cinfer_ascendc
+
+    _say("gemv reference fp8 test shape")
+    rng = np.random.default_rng(4)
+    G, M, K, N = 4, 4, 512, 1536
+    w = rng.integers(0, 255, (G, K, N), dtype=np.uint8)
+    scale = rng.standard_normal((G, 4, 12)).astype(np.float32)
+    out = torch.zeros(M, N, dtype=torch.bfloat16, device="cuda")
+    cinfer_ascendc.grouped_soft_gemv(torch.ones(M, K, dtype=torch.bfloat16, device="cuda"), torch.from_numpy(w).cuda(),
+                                     output=out, scale=torch.from_numpy(scale).cuda(),
+                                     groupList=torch.tensor([1, 2, 3, 4]).cuda(), computeType="fp8")
+    torch.cuda.synchronize()
+    Wd = L.fp8ref_dequant_numpy(w, scale, False).astype(np.float64)
+    exp = np.stack([Wd[g].sum(0) for g in range(G)])
+    exp_bf16 = torch.from_numpy(exp.astype(np.float32)).to(torch.bfloat16)
+    assert torch.allclose(out.cpu(), exp_bf16, rtol=0.02, atol=2 ** -8 * float(np.abs(exp).max()))
+    H.assert_close(H.bits(out), H.bits(exp_bf16), what="reference gemv fp8 test")
+
+
+def test_gemv_matches_gemm_on_the_same_inputs():
+    # the two ops differ only in weight rounding; on bf16 weights they must agree to rounding
+    _say("gemv vs gemm bf16")
+    case = H.make_case("bf16", 4, 2048, 256, [2, 2, 5, 9], seed=6)
+    dev = H.upload(case)
+    a, b = H.run_cabi(case, dev, "gemv"), H.run_cabi(case, dev, "gemm")
+    H.assert_close(a, b, what="gemv vs gemm")
+
+
+# -------------------------------------------------- error behaviour through the module
+def test_module_errors_on_gpu_tensors():
+    import cinfer_ascendc
+
+    x = torch.zeros(4, 256, dtype=torch.bfloat16, device="cuda")
+    w = torch.zeros(2, 256, 128, dtype=torch.int8, device="cuda")
+    s = torch.zeros(2, 16, 256, dtype=torch.bfloat16, device="cuda")
+    gl = torch.tensor([2, 4], device="cuda")
+    y = torch.zeros(4, 256, dtype=torch.bfloat16, device="cuda")
+    cinfer_ascendc.grouped_gemm(x, w, s, s, gl, "fp4", y)          # valid call
+    with pytest.raises(RuntimeError, match="Invalid compute type"):
+        cinfer_ascendc.grouped_gemm(x, w, s, s, gl, "fp5", y)
+    with pytest.raises(RuntimeError, match="shape"):
+        cinfer_ascendc.grouped_gemm(x, w, s[:, :8].contiguous(), s, gl, "fp4", y)
+    with pytest.raises(RuntimeError, match="dtype"):
+        cinfer_ascendc.grouped_gemm(x.float(), w, s, s, gl, "fp4", y)
+    with pytest.raises(RuntimeError, match="contiguous"):
+        cinfer_ascendc.grouped_gemm(x, w, s, s, gl, "fp4", torch.zeros(256, 4, dtype=torch.bfloat16, device="cuda").t())
+    with pytest.raises(RuntimeError, match="alignment"):
+        cinfer_ascendc.grouped_gemm(torch.zeros(4, 96, dtype=torch.bfloat16, device="cuda"),
+                                    torch.zeros(2, 96, 128, dtype=torch.int8, device="cuda"),
+                                    torch.zeros(2, 6, 256, dtype=torch.bfloat16, device="cuda"), s, gl, "fp4", y)
+    torch.cuda.synchronize()
