@@ -50,7 +50,6 @@ def test_dequant_bit_exact_all_codes_and_edge_scales():
     got = _dequant_gpu(codes, scale, 32)
     ref = oracle.dequant_fp4_bf16(codes, scale, 32)
     assert np.array_equal(got, ref)
-    assert (got[:16][codes[:16] & 0x0F == 8][:0].size == 0)
     # code 8 is -0.0 whatever the (positive) scale
     z = _dequant_gpu(np.full((1, 16), 0x88, np.uint8), np.array([[0x3F80]], np.uint16), 32)
     assert (z == 0x8000).all()
