@@ -1,0 +1,295 @@
+#!/usr/bin/env python3
+"""Benchmark of the MoE antiquant ops on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload dsv3_int4_prefill] [--no-extra] [--no-cpu]
+
+A step is one pass of the hot path over one batch of synthetic input that is already
+resident in HBM.  The headline workload is the DeepSeek-V3-shaped int4-antiquant MoE
+prefill: 256 experts, 4096 tokens x top-8 = 32768 sorted rows, gate_up (K=7168, N=4096)
+followed by down (K=2048, N=7168), int4 weights with zero point 8 and bf16 per-group-128
+scales.  One JSON line is printed: whole-step TFLOP/s, the roofline of the dominant kernel
+(measured with events on the launch stream), the CPU oracle timed on a bounded sample of
+the same workload, and -- unless --no-extra -- the other benchmark configurations
+(FP4 dequant, grouped GEMV, int8 GEMM, fused FP4 GEMM at decode shape vs dequant + bf16
+GEMM) as GB/s or TFLOP/s with their own roofline fractions.
+
+Everything on the GPU goes through the C ABI of libmoe_gfx950.so; the oracle is used only
+for the cpu_baseline figure.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(ROOT, "ascend-kernel_amd"))
+sys.path.insert(0, ROOT)
+
+PEAK_HBM_GBS = 8000.0        # MI355X HBM3E, 8 TB/s
+PEAK_BF16_TFLOPS = 2500.0    # MI355X dense bf16 MFMA, 2.5 PFLOP/s
+
+
+def routed_counts(torch, tokens, experts, topk, gen, max_rows=None):
+    """Rows per expert for top-k routing of softmax(N(0,1)) logits (softmax is monotone)."""
+    while True:
+        logits = torch.randn(tokens, experts, generator=gen)
+        ids = logits.topk(topk, dim=1).indices.reshape(-1)
+        counts = torch.bincount(ids, minlength=experts)
+        if max_rows is None or int(counts.max()) <= max_rows:
+            return counts
+
+
+class Op:
+    """One launch of a grouped op through the C ABI with fixed device tensors."""
+
+    def __init__(self, mg, torch, op, fmt, x, w, scale, offset, gl, y, scale_rows=1):
+        self.mg, self.torch, self.op = mg, torch, op
+        self.keep = (x, w, scale, offset, gl, y)
+        p = lambda t: 0 if t is None else t.data_ptr()
+        if fmt in ("fp4_b32", "bf16"):
+            N, K = w.shape[1], x.shape[1]
+        else:
+            K, N = x.shape[1], y.shape[1]
+        self.args = mg.grouped_args(mg.format_from_compute_type(fmt), p(x), p(w), p(scale), p(offset), p(gl), p(y),
+                                    x.shape[0], K, N, gl.shape[0], scale_rows)
+        self.fn = mg.grouped_gemm if op == "gemm" else mg.grouped_gemv
+
+    def __call__(self):
+        self.fn(self.args, self.torch.cuda.current_stream().cuda_stream)
+
+
+def time_launches(torch, fns, iters, warmup):
+    """Average duration (s) of each callable in fns, measured with events recorded on the
+    launch stream around every single launch."""
+    for _ in range(warmup):
+        for f in fns:
+            f()
+    torch.cuda.synchronize()
+    ev = [[(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in fns]
+          for _ in range(iters)]
+    for i in range(iters):
+        for j, f in enumerate(fns):
+            ev[i][j][0].record()
+            f()
+            ev[i][j][1].record()
+    torch.cuda.synchronize()
+    return [sum(ev[i][j][0].elapsed_time(ev[i][j][1]) for i in range(iters)) / iters * 1e-3 for j in range(len(fns))]
+
+
+def bf16_normal(torch, shape, std=1.0):
+    return (torch.randn(shape, device="cuda", dtype=torch.float32) * std).to(torch.bfloat16)
+
+
+def bf16_uniform(torch, shape, lo, hi):
+    return (torch.rand(shape, device="cuda", dtype=torch.float32) * (hi - lo) + lo).to(torch.bfloat16)
+
+
+# --------------------------------------------------------------------------- workloads
+def build_dsv3_int4_prefill(torch, mg, gen):
+    G, tokens, topk, H, I = 256, 4096, 8, 7168, 2048
+    counts = routed_counts(torch, tokens, G, topk, gen)
+    gl = counts.cumsum(0).to(torch.int64).cuda()
+    M = tokens * topk
+    ops, flops = [], []
+    for name, K, N in (("gate_up", H, 2 * I), ("down", I, H)):
+        x = bf16_normal(torch, (M, K))
+        w = torch.randint(0, 256, (G, K, N // 2), dtype=torch.uint8, device="cuda")   # two uniform nibbles per byte
+        s = bf16_uniform(torch, (G, K // 128, N), 1e-3, 1e-2)
+        y = torch.empty(M, N, dtype=torch.bfloat16, device="cuda")
+        ops.append(Op(mg, torch, "gemm", "int4", x, w, s, None, gl, y, scale_rows=K // 128))
+        flops.append(2.0 * M * K * N)
+    return dict(ops=ops, flops=flops, names=["gate_up", "down"], M=M, G=G,
+                desc="DeepSeek-V3 MoE prefill, int4 antiquant: 256 experts, 4096 tokens x top-8 = 32768 rows, "
+                     "gate_up K=7168 N=4096 + down K=2048 N=7168, zero point 8, bf16 scales per 128 k")
+
+
+def run_extra(torch, mg, gen, iters, warmup):
+    out = {}
+    # c1: FP4 e2m1 -> BF16 dequant of a 7168 x 2048 weight, per-32 bf16 scales
+    R, C = 7168, 2048
+    nbuf = 16   # 16 x 37.6 MB > 2 x the 256 MB Infinity Cache: the rotating variant reads and writes cold lines
+    codes = [torch.randint(0, 256, (R, C // 2), dtype=torch.uint8, device="cuda") for _ in range(nbuf)]
+    scales = [bf16_uniform(torch, (R, C // 32), 2.0 ** -8, 2.0 ** -2) for _ in range(nbuf)]
+    outs = [torch.empty(R, C, dtype=torch.bfloat16, device="cuda") for _ in range(nbuf)]
+    stream = lambda: torch.cuda.current_stream().cuda_stream
+    state = {"i": 0}
+
+    def dq_rot():
+        i = state["i"] = (state["i"] + 1) % nbuf
+        mg.dequant_fp4_bf16(codes[i].data_ptr(), scales[i].data_ptr(), outs[i].data_ptr(), R, C, 32, stream())
+
+    def dq_same():
+        mg.dequant_fp4_bf16(codes[0].data_ptr(), scales[0].data_ptr(), outs[0].data_ptr(), R, C, 32, stream())
+
+    nbytes = R * C // 2 + R * (C // 32) * 2 + R * C * 2
+    t_rot, = time_launches(torch, [dq_rot], max(iters, 64), warmup + nbuf)
+    t_same, = time_launches(torch, [dq_same], max(iters, 64), warmup)
+    out["fp4_dequant_7168x2048"] = dict(bytes=nbytes, us=t_rot * 1e6, GBps=nbytes / t_rot / 1e9,
+                                        frac_hbm=nbytes / t_rot / 1e9 / PEAK_HBM_GBS, us_same_buffer=t_same * 1e6,
+                                        GBps_same_buffer=nbytes / t_same / 1e9,
+                                        note="rotating over 16 buffer sets (cold) / same buffers (Infinity Cache warm)")
+    del codes, scales, outs
+
+    # c2: grouped GEMV decode, 64 experts, 32 rows (4 tokens x top-8), K=7168, N=2048, bf16 weights [G,N,K]
+    G, K, N = 64, 7168, 2048
+    counts = routed_counts(torch, 4, G, 8, gen, max_rows=4)
+    gl = counts.cumsum(0).to(torch.int64).cuda()
+    M = int(counts.sum())
+    A = int((counts > 0).sum())
+    x = bf16_normal(torch, (M, K))
+    w = bf16_normal(torch, (G, N, K), 0.02)
+    y = torch.empty(M, N, dtype=torch.bfloat16, device="cuda")
+    op = Op(mg, torch, "gemv", "bf16", x, w, None, None, gl, y)
+    t, = time_launches(torch, [op], iters, warmup)
+    nbytes = A * N * K * 2 + M * K * 2 + M * N * 2
+    out["grouped_gemv_bf16_64e"] = dict(active_experts=A, rows=M, bytes=nbytes, us=t * 1e6, GBps=nbytes / t / 1e9,
+                                        frac_hbm=nbytes / t / 1e9 / PEAK_HBM_GBS)
+    del x, w, y, op
+
+    # c3: int8 antiquant grouped GEMM, 8 experts, multinomial 4096 rows, K=4096, N=14336
+    G, M, K, N = 8, 4096, 4096, 14336
+    counts = torch.distributions.Multinomial(M, torch.full((G,), 1.0 / G)).sample().to(torch.int64)
+    gl = counts.cumsum(0).cuda()
+    x = bf16_normal(torch, (M, K))
+    w = torch.randint(-127, 128, (G, K, N), dtype=torch.int8, device="cuda")
+    s = bf16_uniform(torch, (G, N), 1e-3, 1e-2)
+    o = bf16_uniform(torch, (G, N), -2.0, 2.0)
+    y = torch.empty(M, N, dtype=torch.bfloat16, device="cuda")
+    op = Op(mg, torch, "gemm", "int8", x, w, s, o, gl, y)
+    t, = time_launches(torch, [op], iters, warmup)
+    fl = 2.0 * M * K * N
+    out["grouped_gemm_int8_8e"] = dict(flops=fl, us=t * 1e6, TFLOPs=fl / t / 1e12,
+                                       frac_mfma=fl / t / 1e12 / PEAK_BF16_TFLOPS)
+    del x, w, s, o, y, op
+
+    # c5: fused FP4 (e2m1, per-32 bf16 scales) grouped GEMM at decode shape vs dequant + bf16 grouped GEMM
+    G, K, N = 256, 7168, 2048
+    counts = routed_counts(torch, 64, G, 8, gen)
+    gl = counts.cumsum(0).to(torch.int64).cuda()
+    M = int(counts.sum())
+    A = int((counts > 0).sum())
+    x = bf16_normal(torch, (M, K))
+    w = torch.randint(0, 256, (G, N, K // 2), dtype=torch.uint8, device="cuda")
+    s = bf16_uniform(torch, (G, N, K // 32), 2.0 ** -8, 2.0 ** -2)
+    y = torch.empty(M, N, dtype=torch.bfloat16, device="cuda")
+    fused = Op(mg, torch, "gemm", "fp4_b32", x, w, s, None, gl, y)
+    wd = torch.empty(G, N, K, dtype=torch.bfloat16, device="cuda")
+    y2 = torch.empty(M, N, dtype=torch.bfloat16, device="cuda")
+
+    def dq_all():
+        mg.dequant_fp4_bf16(w.data_ptr(), s.data_ptr(), wd.data_ptr(), G * N, K, 32, stream())
+
+    sep = Op(mg, torch, "gemm", "bf16", x, wd, None, None, gl, y2)
+    t_f, t_d, t_s = time_launches(torch, [fused, dq_all, sep], max(iters // 2, 5), warmup)
+    nbytes = A * (N * K // 2 + N * (K // 32) * 2) + M * K * 2 + M * N * 2
+    diff = float((y.float() - y2.float()).abs().max())
+    out["fused_fp4_gemm_decode_256e"] = dict(active_experts=A, rows=M, bytes=nbytes, us=t_f * 1e6,
+                                             GBps=nbytes / t_f / 1e9, frac_hbm=nbytes / t_f / 1e9 / PEAK_HBM_GBS,
+                                             separate_us=(t_d + t_s) * 1e6, separate_dequant_us=t_d * 1e6,
+                                             separate_gemm_us=t_s * 1e6, speedup_vs_separate=(t_d + t_s) / t_f,
+                                             max_abs_diff_fused_vs_separate=diff)
+    return out
+
+
+def cpu_baseline(torch, seed):
+    """The CPU oracle on a bounded sample of the headline workload: the gate_up GEMM
+    (K=7168, N=4096, int4, group 128) for 4 experts' worth of rows."""
+    import numpy as np
+
+    import oracle
+
+    rng = np.random.default_rng(seed)
+    G, K, N = 4, 7168, 4096
+    counts = rng.multinomial(512, np.full(G, 1.0 / G))
+    gl = np.cumsum(counts).astype(np.int64)
+    M = int(gl[-1])
+    x = torch.from_numpy(rng.standard_normal((M, K)).astype(np.float32)).to(torch.bfloat16)
+    xb = x.view(torch.int16).numpy().view(np.uint16)
+    w = rng.integers(0, 256, (G, K, N // 2), dtype=np.uint8)
+    s = torch.from_numpy(rng.uniform(1e-3, 1e-2, (G, K // 128, N)).astype(np.float32)).to(torch.bfloat16)
+    sb = s.view(torch.int16).numpy().view(np.uint16)
+    oracle.lib()
+    t0 = time.perf_counter()
+    oracle.grouped_gemm(oracle.FMT_INT4, xb, w, sb, None, gl)
+    dt = time.perf_counter() - t0
+    fl = 2.0 * M * K * N
+    return dict(value=fl / dt / 1e12, unit="TFLOP/s", cores=oracle.num_threads(), kind="port",
+                sample=f"gate_up GEMM of {G} experts ({M} rows, K={K}, N={N}, int4 group 128): "
+                       f"{fl / 1e9:.1f} GFLOP in {dt:.2f} s on the oracle's OpenMP loops (dequant included)")
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="dsv3_int4_prefill")
+    ap.add_argument("--no-extra", action="store_true", help="skip the other benchmark configurations")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU oracle baseline")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        sys.exit("bench.py: this build runs on one GPU only (--gpus 1); the ops shard by expert across GPUs, "
+                 "with the token exchange left to the caller")
+    if args.workload != "dsv3_int4_prefill":
+        sys.exit("bench.py: the only headline workload is dsv3_int4_prefill")
+
+    import torch
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible")
+    import moe_gfx950 as mg   # raises if the HIP library has not been built
+
+    torch.cuda.set_device(0)
+    gen = torch.Generator().manual_seed(0)
+    torch.manual_seed(0)
+
+    wl = build_dsv3_int4_prefill(torch, mg, gen)
+    ops = wl["ops"]
+    for _ in range(args.warmup):
+        for op in ops:
+            op()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        for op in ops:
+            op()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    step_flops = sum(wl["flops"])
+    value = step_flops * args.steps / dt / 1e12
+
+    # per-launch durations of the dominant kernel (the int4 grouped GEMM), events on the launch stream
+    t_each = time_launches(torch, ops, args.steps, 1)
+    avg_launch = sum(t_each) / len(t_each)
+    achieved = (step_flops / len(ops)) / avg_launch / 1e12
+    roofline = dict(bound="mfma", achieved=achieved, peak=PEAK_BF16_TFLOPS, unit="TFLOP/s",
+                    frac=achieved / PEAK_BF16_TFLOPS, traffic=None,
+                    kernel="moe::grouped_gemm_kernel<int4>",
+                    per_launch={n: dict(us=t * 1e6, TFLOPs=f / t / 1e12, frac=f / t / 1e12 / PEAK_BF16_TFLOPS)
+                                for n, t, f in zip(wl["names"], t_each, wl["flops"])})
+    del wl, ops
+    torch.cuda.empty_cache()
+
+    result = {
+        "metric": "grouped-GEMM TFLOPS + GEMV/dequant HBM GB/s (% of MI355X peak), DSV3 MoE",
+        "value": value, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": dt / args.steps * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "dsv3_int4_prefill: 256 experts, 4096 tokens x top-8 (32768 rows), gate_up "
+                               "7168->4096 + down 2048->7168, int4 zp8 group-128 bf16 scales, bf16 activations",
+                   "flops_per_step": step_flops},
+        "roofline": roofline,
+    }
+    if not args.no_extra:
+        result["workloads"] = run_extra(torch, mg, gen, max(args.steps, 20), args.warmup)
+        torch.cuda.empty_cache()
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline(torch, 0)
+    print(json.dumps(result), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -48,6 +48,7 @@ def lib() -> ctypes.CDLL:
             build()
         L = ctypes.CDLL(_LIB_PATH)
         vp, i64, i32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int
+        L.orc_num_threads.restype = ctypes.c_int
         L.orc_e2m1_decode.restype = ctypes.c_float
         L.orc_e2m1_decode.argtypes = [ctypes.c_uint8]
         L.orc_e4m3_decode.restype = ctypes.c_float
@@ -79,6 +80,10 @@ def _c(a, dtype=None):
     if dtype is not None and a.dtype != dtype:
         raise TypeError(f"expected {dtype}, got {a.dtype}")
     return a
+
+
+def num_threads() -> int:
+    return int(lib().orc_num_threads())
 
 
 def e2m1_decode(code: int) -> float:

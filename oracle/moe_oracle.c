@@ -28,6 +28,9 @@
  *   parity unpinned beyond that formula.
  */
 #include <math.h>
+#ifdef _OPENMP
+#include <omp.h>
+#endif
 #include <stdint.h>
 #include <stdlib.h>
 #include <string.h>
@@ -56,6 +59,15 @@ static inline uint16_t f32_to_bf16_rne(float f) {
     if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x0040u); /* quiet NaN */
     u += 0x7fffu + ((u >> 16) & 1u);
     return (uint16_t)(u >> 16);
+}
+
+/* Threads the parallel loops of this file use. */
+int orc_num_threads(void) {
+#ifdef _OPENMP
+    return omp_get_max_threads();
+#else
+    return 1;
+#endif
 }
 
 uint16_t orc_f32_to_bf16(float f) { return f32_to_bf16_rne(f); }
