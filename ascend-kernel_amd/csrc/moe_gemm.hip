@@ -26,7 +26,7 @@
 namespace moe {
 
 constexpr int GM_BN = 256;     // columns per workgroup
-constexpr int GM_MT_MAX = 12;  // 16-row blocks per tile (192 rows)
+constexpr int GM_MT_MAX = 12;  // 16-row blocks per tile the LDS buffers are sized for (192 rows)
 constexpr int GM_THREADS = 256;
 
 struct GemmParams {
@@ -79,6 +79,8 @@ struct BTraits;
 template <>
 struct BTraits<MOE_FMT_INT4> {
     static constexpr int BK = 64, NS = 2;
+    static constexpr bool DOUBLE_RAW = false;
+    static constexpr int MT_MAX = 11;  // 176 rows: the largest tile that keeps every value in registers
     struct Raw {
         uint32_t r[2][8];
         u32x2_t sc[2];
@@ -91,15 +93,12 @@ struct BTraits<MOE_FMT_INT4> {
         c.vw = 8 * c.q * (c.N >> 1) + 64 * (c.w >> 1) + 4 * c.i;
         c.vs = col(c, 0) * 2;
     }
-    __device__ static __forceinline__ void load(Raw& raw, const BCtx& c, int k0) {
+    __device__ static __forceinline__ void load_sub(Raw& raw, const BCtx& c, int k0, int s) {
         const int nb = c.N >> 1;
 #pragma unroll
-        for (int s = 0; s < 2; ++s) {
-#pragma unroll
-            for (int j = 0; j < 8; ++j) raw.r[s][j] = ldg_b32(c.rw, c.vw, (k0 + 32 * s + j) * nb + (c.n0 >> 1));
-            // a 32-k sub-step never straddles a scale group (group % 32 == 0)
-            raw.sc[s] = ldg_b64(c.rs, c.vs, (((k0 + 32 * s) / c.gs) * c.N + c.n0) * 2);
-        }
+        for (int j = 0; j < 8; ++j) raw.r[s][j] = ldg_b32(c.rw, c.vw, (k0 + 32 * s + j) * nb + (c.n0 >> 1));
+        // a 32-k sub-step never straddles a scale group (group % 32 == 0)
+        raw.sc[s] = ldg_b64(c.rs, c.vs, (((k0 + 32 * s) / c.gs) * c.N + c.n0) * 2);
     }
     __device__ static __forceinline__ void frags(const Raw& raw, const BCtx& c, int s, u32x4_t out[4]) {
         const int sh = 16 * (c.w & 1);
@@ -126,6 +125,8 @@ struct BTraits<MOE_FMT_INT4> {
 template <>
 struct BTraits<MOE_FMT_FP4_REF> {
     static constexpr int BK = 64, NS = 2;
+    static constexpr bool DOUBLE_RAW = false;
+    static constexpr int MT_MAX = 11;  // 176 rows: the largest tile that keeps every value in registers
     struct Raw {
         u32x4_t r[2][2];
         u32x2_t sc[2];
@@ -141,15 +142,12 @@ struct BTraits<MOE_FMT_FP4_REF> {
         c.vw = R0 * (c.N >> 1) + 32 * qq;
         c.vs = ((c.q >> 1) * c.N + col(c, 0)) * 2;  // scale group of 16 k: (k0 + 32s)/16 + (q >> 1)
     }
-    __device__ static __forceinline__ void load(Raw& raw, const BCtx& c, int k0) {
+    __device__ static __forceinline__ void load_sub(Raw& raw, const BCtx& c, int k0, int s) {
         const int nb = c.N >> 1;
-#pragma unroll
-        for (int s = 0; s < 2; ++s) {
-            const int so = (k0 + 16 * s) * nb + (c.n0 >> 1);
-            raw.r[s][0] = ldg_b128(c.rw, c.vw, so);
-            raw.r[s][1] = ldg_b128(c.rw, c.vw, so + 16);
-            raw.sc[s] = ldg_b64(c.rs, c.vs, (((k0 + 32 * s) >> 4) * c.N + c.n0) * 2);
-        }
+        const int so = (k0 + 16 * s) * nb + (c.n0 >> 1);
+        raw.r[s][0] = ldg_b128(c.rw, c.vw, so);
+        raw.r[s][1] = ldg_b128(c.rw, c.vw, so + 16);
+        raw.sc[s] = ldg_b64(c.rs, c.vs, (((k0 + 32 * s) >> 4) * c.N + c.n0) * 2);
     }
     __device__ static __forceinline__ void frags(const Raw& raw, const BCtx& c, int s, u32x4_t out[4]) {
         const int sh = 16 * (c.w & 1);
@@ -173,9 +171,11 @@ struct BTraits<MOE_FMT_FP4_REF> {
 template <int FMT>
 struct BTraitsByte {
     static constexpr int BK = 64, NS = 2;
+    static constexpr bool DOUBLE_RAW = false;
+    static constexpr int MT_MAX = 11;  // 176 rows: the largest tile that keeps every value in registers
     struct Raw {
         uint32_t r[2][8];
-        float s8;  // fp8: scale of the 128x128 block of this step
+        float s8[2];  // fp8: scale of the 128x128 block of each sub-step
     };
     __device__ static __forceinline__ int a_chunk(int s, int q) { return 4 * s + q; }
     __device__ static __forceinline__ int col(const BCtx& c, int t) { return 64 * c.w + 4 * c.i + t; }
@@ -183,12 +183,14 @@ struct BTraitsByte {
         c.vw = 8 * c.q * c.N + col(c, 0);
         c.vs = 0;
     }
-    __device__ static __forceinline__ void load(Raw& raw, const BCtx& c, int k0) {
+    __device__ static __forceinline__ void load_sub(Raw& raw, const BCtx& c, int k0, int s) {
 #pragma unroll
-        for (int s = 0; s < 2; ++s)
-#pragma unroll
-            for (int j = 0; j < 8; ++j) raw.r[s][j] = ldg_b32(c.rw, c.vw, (k0 + 32 * s + j) * c.N + c.n0);
-        if (FMT == MOE_FMT_FP8_REF) raw.s8 = c.s8[(k0 >> 7) * (c.N >> 7) + ((c.n0 + 64 * c.w) >> 7)];
+        for (int j = 0; j < 8; ++j) raw.r[s][j] = ldg_b32(c.rw, c.vw, (k0 + 32 * s + j) * c.N + c.n0);
+        if (FMT == MOE_FMT_FP8_REF) {
+            // the one-step-ahead prefetch may point past K: clamp the block row (value unused then)
+            const int kb = min(k0 >> 7, (c.K >> 7) - 1);
+            raw.s8[s] = c.s8[kb * (c.N >> 7) + ((c.n0 + 64 * c.w) >> 7)];
+        }
     }
 };
 
@@ -226,8 +228,8 @@ struct BTraits<MOE_FMT_FP8_REF> : BTraitsByte<MOE_FMT_FP8_REF> {
             const uint32_t a = raw.r[s][j], b = raw.r[s][j + 1];
 #pragma unroll
             for (int t = 0; t < 4; ++t)
-                out[t][j >> 1] = pack_bf16_rne(e4m3_ref_to_f32((a >> (8 * t)) & 0xffu) * raw.s8,
-                                               e4m3_ref_to_f32((b >> (8 * t)) & 0xffu) * raw.s8);
+                out[t][j >> 1] = pack_bf16_rne(e4m3_ref_to_f32((a >> (8 * t)) & 0xffu) * raw.s8[s],
+                                               e4m3_ref_to_f32((b >> (8 * t)) & 0xffu) * raw.s8[s]);
         }
     }
 };
@@ -249,7 +251,12 @@ struct BTraits<MOE_FMT_FP4_B32> {
         c.vw = (64 * c.w + c.i) * (c.K >> 1) + 16 * c.q;
         c.vs = ((64 * c.w + c.i) * (c.K >> 5) + c.q) * 2;
     }
-    __device__ static __forceinline__ void load(Raw& raw, const BCtx& c, int k0) {
+    // One 16-byte load per t serves all 4 sub-steps, so the registers cannot be reloaded
+    // sub-step by sub-step: the next step is loaded into a second set at sub-step 0.
+    static constexpr bool DOUBLE_RAW = true;
+    static constexpr int MT_MAX = 10;  // larger tiles spill: BK = 128 doubles the x staging registers
+    __device__ static __forceinline__ void load_sub(Raw& raw, const BCtx& c, int k0, int s) {
+        if (s != 0) return;
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
             raw.r[t] = ldg_b128(c.rw, c.vw, (c.n0 + 16 * t) * (c.K >> 1) + (k0 >> 1));
@@ -275,6 +282,8 @@ struct BTraits<MOE_FMT_FP4_B32> {
 template <>
 struct BTraits<MOE_FMT_BF16> {
     static constexpr int BK = 64, NS = 2;
+    static constexpr bool DOUBLE_RAW = false;
+    static constexpr int MT_MAX = 11;  // 176 rows: the largest tile that keeps every value in registers
     struct Raw {
         u32x4_t r[4][2];
     };
@@ -284,13 +293,9 @@ struct BTraits<MOE_FMT_BF16> {
         c.vw = (64 * c.w + c.i) * c.K * 2 + 32 * c.q;
         c.vs = 0;
     }
-    __device__ static __forceinline__ void load(Raw& raw, const BCtx& c, int k0) {
+    __device__ static __forceinline__ void load_sub(Raw& raw, const BCtx& c, int k0, int s) {
 #pragma unroll
-        for (int t = 0; t < 4; ++t) {
-            const int so = ((c.n0 + 16 * t) * c.K + k0) * 2;
-            raw.r[t][0] = ldg_b128(c.rw, c.vw, so);
-            raw.r[t][1] = ldg_b128(c.rw, c.vw, so + 16);
-        }
+        for (int t = 0; t < 4; ++t) raw.r[t][s] = ldg_b128(c.rw, c.vw, ((c.n0 + 16 * t) * c.K + k0) * 2 + 16 * s);
     }
     __device__ static __forceinline__ void frags(const Raw& raw, const BCtx&, int s, u32x4_t out[4]) {
 #pragma unroll
@@ -404,12 +409,28 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& P, u32x4_t* lds_a, i
             if (PASSES * RPP == 16 * MT || ar + RPP * p < 16 * MT)
                 lds_a[buf * ABUF + a_lds_unit<BK>(ar + RPP * p, ac)] = areg[p];
     };
-    auto compute = [&](const typename T::Raw& rw, int buf) {
-        const u32x4_t* la = lds_a + buf * ABUF;
+
+    // Software pipeline, one barrier per k step.  Step kt computes from LDS buffer kt&1 and
+    // from `raw`; as soon as the fragments of a sub-step have been decoded, the same
+    // registers are reloaded with that sub-step of step kt+1 (formats whose loads span all
+    // sub-steps use a second register set instead), and the x tile of step kt+1
+    // travels through registers into the other LDS buffer.  The last step prefetches one
+    // step past K: buffer loads beyond a slab return 0 and the x rows it reads are inside
+    // the tensor; neither is used.
+    __syncthreads();  // previous tile's readers are done with both buffers
+    load_a(0);
+#pragma unroll
+    for (int s = 0; s < NS; ++s) T::load_sub(raw, c, 0, s);
+    store_a(0);
+    __syncthreads();
+    for (int kt = 0; kt < nk; ++kt) {
+        load_a(kt + 1);
+        const u32x4_t* la = lds_a + (kt & 1) * ABUF;
 #pragma unroll
         for (int s = 0; s < NS; ++s) {
             u32x4_t bf[4];
-            ops.frags(rw, c, s, bf);
+            ops.frags(raw, c, s, bf);
+            T::load_sub(T::DOUBLE_RAW ? raw_next : raw, c, (kt + 1) * BK, s);
             const int ch = T::a_chunk(s, c.q);
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt) {
@@ -421,30 +442,9 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& P, u32x4_t* lds_a, i
                                                                          acc[mt][t], 0, 0, 0);
             }
         }
-    };
-
-    // Software pipeline: while step kt is computed from LDS buffer kt&1 and `raw`, the x
-    // tile and the packed weights of step kt+1 are in flight to registers; the x tile is
-    // written to the other LDS buffer after the MFMAs, one barrier per step.
-    __syncthreads();  // previous tile's readers are done with both buffers
-    load_a(0);
-    T::load(raw, c, 0);
-    store_a(0);
-    __syncthreads();
-    // The last step prefetches one step past K: buffer loads beyond a slab return 0 and
-    // the x rows it reads are inside the tensor; neither is used.
-    for (int kt = 0; kt < nk; ++kt) {
-        load_a(kt + 1);
-        T::load(raw_next, c, (kt + 1) * BK);
-        compute(raw, kt & 1);
-        // pin the loop-carried accumulators to AGPRs so that every MFMA accumulates in place
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-            for (int t = 0; t < 4; ++t) asm volatile("" : "+a"(acc[mt][t]));
         store_a((kt + 1) & 1);
         __syncthreads();
-        raw = raw_next;
+        if (T::DOUBLE_RAW) raw = raw_next;
     }
 
     // epilogue: fp32 -> bf16 (RNE), rows beyond the chunk are dropped
@@ -474,13 +474,14 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& P, u32x4_t* lds_a, i
 // ---------------------------------------------------------------------------------
 // Tile scheduler (role of GMMAntiquantProcess::Process,
 // grouped_gemm/op_kernel/grouped_matmul_antiquant.h:241-288).  Expert g with m_g rows
-// has ceil(m_g/16) row blocks, cut into the fewest chunks of <= GM_MT_MAX blocks, as
+// has ceil(m_g/16) row blocks, cut into the fewest chunks of <= MT_MAX blocks, as
 // even as possible; each chunk has N/256 tiles.  prefix[] (in LDS) is the exclusive
 // scan of the tile counts.
 // ---------------------------------------------------------------------------------
+template <int MT_MAX>
 __device__ __forceinline__ void expert_chunks(int m, int& chunks, int& bpc) {
     const int nblk = (m + 15) >> 4;
-    chunks = (nblk + GM_MT_MAX - 1) / GM_MT_MAX;
+    chunks = (nblk + MT_MAX - 1) / MT_MAX;
     bpc = chunks ? (nblk + chunks - 1) / chunks : 0;
 }
 
@@ -503,7 +504,7 @@ __global__ __launch_bounds__(GM_THREADS) void grouped_gemm_kernel(GemmParams P) 
             int64_t s = g ? P.gl[g - 1] : 0, e = P.gl[g];
             s = max((int64_t)0, s); e = min(e, P.M);
             int chunks, bpc;
-            expert_chunks(e > s ? (int)(e - s) : 0, chunks, bpc);
+            expert_chunks<BTraits<FMT>::MT_MAX>(e > s ? (int)(e - s) : 0, chunks, bpc);
             sum += chunks * ntile_n;
         }
         part[tid] = sum;
@@ -519,7 +520,7 @@ __global__ __launch_bounds__(GM_THREADS) void grouped_gemm_kernel(GemmParams P) 
             int64_t s = g ? P.gl[g - 1] : 0, e = P.gl[g];
             s = max((int64_t)0, s); e = min(e, P.M);
             int chunks, bpc;
-            expert_chunks(e > s ? (int)(e - s) : 0, chunks, bpc);
+            expert_chunks<BTraits<FMT>::MT_MAX>(e > s ? (int)(e - s) : 0, chunks, bpc);
             prefix[g] = run;
             run += chunks * ntile_n;
         }
@@ -546,7 +547,7 @@ __global__ __launch_bounds__(GM_THREADS) void grouped_gemm_kernel(GemmParams P) 
         const int64_t gbeg = g ? max((int64_t)0, P.gl[g - 1]) : 0, gend = min(P.gl[g], P.M);
         const int m = __builtin_amdgcn_readfirstlane((int)(gend - gbeg));
         int chunks, bpc;
-        expert_chunks(m, chunks, bpc);
+        expert_chunks<BTraits<FMT>::MT_MAX>(m, chunks, bpc);
         const int local = __builtin_amdgcn_readfirstlane(T - prefix[g]);
         const int chunk = local / ntile_n, nt = local % ntile_n;
         const int rbeg = chunk * bpc * 16;
@@ -567,8 +568,12 @@ __global__ __launch_bounds__(GM_THREADS) void grouped_gemm_kernel(GemmParams P) 
             case 8: gemm_tile<FMT, 8>(P, lds_a, g, row0, rows, n0); break;
             case 9: gemm_tile<FMT, 9>(P, lds_a, g, row0, rows, n0); break;
             case 10: gemm_tile<FMT, 10>(P, lds_a, g, row0, rows, n0); break;
-            case 11: gemm_tile<FMT, 11>(P, lds_a, g, row0, rows, n0); break;
-            default: gemm_tile<FMT, 12>(P, lds_a, g, row0, rows, n0); break;
+            case 11:
+                if constexpr (BTraits<FMT>::MT_MAX >= 11) gemm_tile<FMT, 11>(P, lds_a, g, row0, rows, n0);
+                break;
+            default:
+                if constexpr (BTraits<FMT>::MT_MAX >= 12) gemm_tile<FMT, 12>(P, lds_a, g, row0, rows, n0);
+                break;
         }
     }
 }
@@ -599,7 +604,7 @@ static int launch_gemm_fmt(const moe_grouped_args* a, hipStream_t stream) {
     if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return MOE_ERR_NO_DEVICE;
     // upper bound on the tile count without reading group_list: every expert adds at most
     // one partly filled chunk
-    const int64_t max_chunks = a->M / (16 * GM_MT_MAX) + a->G;
+    const int64_t max_chunks = a->M / (16 * BTraits<FMT>::MT_MAX) + a->G;
     const int64_t max_tiles = max_chunks * (a->N / GM_BN);
     // a multiple of 8 so that the XCD-aware order covers every tile index
     const int64_t want = max_tiles < cus ? max_tiles : cus;

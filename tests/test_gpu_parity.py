@@ -3,6 +3,8 @@ cinfer_ascendc module), against the CPU oracle on identical seeded inputs.
 
 Bars: FP4 dequant bit-exact; grouped GEMM / GEMV max|d|/max|ref| <= 1e-2 and
 |d| <= 2e-2 * max(1, |ref|), both sides rounded to bf16 (helpers.REL_TOL / ABS_TOL)."""
+import zlib
+
 import numpy as np
 import pytest
 import torch
@@ -97,7 +99,7 @@ def test_gemm_parity_small(fmt, gl_name):
     gl = GEMM_GROUP_LISTS[gl_name]
     G, K, N = len(gl), 512, 512
     _say(f"gemm fmt={fmt} gl={gl_name} G={G} K={K} N={N}")
-    case = H.make_case(fmt, G, K, N, gl, seed=hash((fmt, gl_name)) % 1000, extra_rows=5)
+    case = H.make_case(fmt, G, K, N, gl, seed=zlib.crc32(f"{fmt}/{gl_name}".encode()) % 1000, extra_rows=5)
     got = H.run_cabi(case, H.upload(case), "gemm")
     ref = H.oracle_out(case)
     M_used = gl[-1]
@@ -222,7 +224,7 @@ def test_gemv_parity_small(fmt, gl_name):
     gl = GEMV_GROUP_LISTS[gl_name]
     G, K, N = len(gl), 1024, 512
     _say(f"gemv fmt={fmt} gl={gl_name}")
-    case = H.make_case(fmt, G, K, N, gl, seed=hash((fmt, gl_name, 1)) % 1000, extra_rows=3)
+    case = H.make_case(fmt, G, K, N, gl, seed=zlib.crc32(f"gemv/{fmt}/{gl_name}".encode()) % 1000, extra_rows=3)
     got = H.run_cabi(case, H.upload(case), "gemv")
     ref = H.oracle_out(case, gemv=True)
     H.assert_close(got, ref, rows=slice(0, gl[-1]), what=f"gemv {fmt}/{gl_name}")
