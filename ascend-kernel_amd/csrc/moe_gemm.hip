@@ -67,18 +67,25 @@ struct BCtx {
     const float* s8;     // fp8: scale blocks of the expert
     int K, N, n0, gs;    // gs = k per scale group (int4)
     int i, q, w;         // lane & 15, lane >> 4, wavefront (scalar)
+    uint32_t mlo, mhi;   // 0x0f0f / 0xf0f0, opaque to the optimizer (int4 decode)
 };
 
 template <int FMT>
 struct BTraits;
 
 // ------------------------------------------------------------------ int4, [K, N/2]
-// Lane (i, q) of wavefront w loads, for each of its 8 k rows, the dword holding the
-// 8 columns 128(w>>1) + 8i + [0,8); wavefronts 2p and 2p+1 read the same dwords and
-// use nibbles 0-3 and 4-7.  MFMA t gets nibble 4(w&1) + t.
+// Lane (i, q) of wavefront w owns the 4 columns 128(w>>1) + 8i + 4(w&1) + [0,4): for each
+// of its 8 k rows it loads the dword holding the 8 columns 128(w>>1) + 8i + [0,8) and
+// shifts its half down (wavefronts 2p and 2p+1 read the same dwords).  MFMA t gets
+// nibble t of that half.
+// Decode: byte b of (v & 0x0f0f) is nibble 2b, byte b of (v & 0xf0f0) is
+// 16 * nibble 2b+1; v_cvt_f32_ubyteN turns either into fp32 and one fma applies
+// scale (or scale/16) and the zero point: q*s - 8s = (q - 8)*s exactly (<= 12 significant
+// bits), so the bf16 weight equals RNE_bf16((q - 8) * scale).
 template <>
 struct BTraits<MOE_FMT_INT4> {
     static constexpr int BK = 64, NS = 2;
+    static constexpr int VALU_SUB = 116;  // decode instructions per 32-k sub-step (interleave hint)
     static constexpr bool DOUBLE_RAW = false;
     static constexpr int MT_MAX = 11;  // 176 rows: the largest tile that keeps every value in registers
     struct Raw {
@@ -96,23 +103,30 @@ struct BTraits<MOE_FMT_INT4> {
     __device__ static __forceinline__ void load_sub(Raw& raw, const BCtx& c, int k0, int s) {
         const int nb = c.N >> 1;
 #pragma unroll
-        for (int j = 0; j < 8; ++j) raw.r[s][j] = ldg_b32(c.rw, c.vw, (k0 + 32 * s + j) * nb + (c.n0 >> 1));
+        for (int j = 0; j < 8; ++j)
+            raw.r[s][j] = ldg_b32(c.rw, c.vw, (k0 + 32 * s + j) * nb + (c.n0 >> 1));
         // a 32-k sub-step never straddles a scale group (group % 32 == 0)
         raw.sc[s] = ldg_b64(c.rs, c.vs, (((k0 + 32 * s) / c.gs) * c.N + c.n0) * 2);
     }
+    // Byte -> fp32 converts.  The nibble masks come from BCtx as values the compiler cannot
+    // see through; with literal masks it folds them into every extraction and spends an
+    // extra instruction per element instead of using v_cvt_f32_ubyte0 / ubyte1 directly.
+    __device__ static __forceinline__ float ubyte0(uint32_t v) { return (float)(v & 0xffu); }
+    __device__ static __forceinline__ float ubyte1(uint32_t v) { return (float)((v >> 8) & 0xffu); }
     __device__ static __forceinline__ void frags(const Raw& raw, const BCtx& c, int s, u32x4_t out[4]) {
         const int sh = 16 * (c.w & 1);
-        const float sc[4] = {bf16_lo(raw.sc[s][0]), bf16_hi(raw.sc[s][0]), bf16_lo(raw.sc[s][1]),
-                             bf16_hi(raw.sc[s][1])};
+        const float s0 = bf16_lo(raw.sc[s][0]), s1 = bf16_hi(raw.sc[s][0]);
+        const float s2 = bf16_lo(raw.sc[s][1]), s3 = bf16_hi(raw.sc[s][1]);
+        const float h1 = s1 * 0.0625f, h3 = s3 * 0.0625f;           // odd nibbles arrive times 16
+        const float z0 = -8.f * s0, z1 = -8.f * s1, z2 = -8.f * s2, z3 = -8.f * s3;
 #pragma unroll
         for (int j = 0; j < 8; j += 2) {
             const uint32_t a = raw.r[s][j] >> sh, b = raw.r[s][j + 1] >> sh;
-#pragma unroll
-            for (int t = 0; t < 4; ++t) {
-                const float fa = (float)((int)((a >> (4 * t)) & 15u) - 8) * sc[t];
-                const float fb = (float)((int)((b >> (4 * t)) & 15u) - 8) * sc[t];
-                out[t][j >> 1] = pack_bf16_rne(fa, fb);
-            }
+            const uint32_t al = a & c.mlo, ah = a & c.mhi, bl = b & c.mlo, bh = b & c.mhi;
+            out[0][j >> 1] = pack_bf16_rne(fmaf(ubyte0(al), s0, z0), fmaf(ubyte0(bl), s0, z0));
+            out[1][j >> 1] = pack_bf16_rne(fmaf(ubyte0(ah), h1, z1), fmaf(ubyte0(bh), h1, z1));
+            out[2][j >> 1] = pack_bf16_rne(fmaf(ubyte1(al), s2, z2), fmaf(ubyte1(bl), s2, z2));
+            out[3][j >> 1] = pack_bf16_rne(fmaf(ubyte1(ah), h3, z3), fmaf(ubyte1(bh), h3, z3));
         }
     }
 };
@@ -125,6 +139,7 @@ struct BTraits<MOE_FMT_INT4> {
 template <>
 struct BTraits<MOE_FMT_FP4_REF> {
     static constexpr int BK = 64, NS = 2;
+    static constexpr int VALU_SUB = 84;
     static constexpr bool DOUBLE_RAW = false;
     static constexpr int MT_MAX = 11;  // 176 rows: the largest tile that keeps every value in registers
     struct Raw {
@@ -171,6 +186,7 @@ struct BTraits<MOE_FMT_FP4_REF> {
 template <int FMT>
 struct BTraitsByte {
     static constexpr int BK = 64, NS = 2;
+    static constexpr int VALU_SUB = FMT == MOE_FMT_INT8 ? 120 : 210;
     static constexpr bool DOUBLE_RAW = false;
     static constexpr int MT_MAX = 11;  // 176 rows: the largest tile that keeps every value in registers
     struct Raw {
@@ -252,11 +268,12 @@ struct BTraits<MOE_FMT_FP4_B32> {
         c.vs = ((64 * c.w + c.i) * (c.K >> 5) + c.q) * 2;
     }
     // One 16-byte load per t serves all 4 sub-steps, so the registers cannot be reloaded
-    // sub-step by sub-step: the next step is loaded into a second set at sub-step 0.
+    // sub-step by sub-step: a whole step is loaded into a second register set (load_sub
+    // ignores its sub-step argument and is called once per step).
     static constexpr bool DOUBLE_RAW = true;
+    static constexpr int VALU_SUB = 64;  // decode instructions per 32-k sub-step (interleave hint)
     static constexpr int MT_MAX = 10;  // larger tiles spill: BK = 128 doubles the x staging registers
-    __device__ static __forceinline__ void load_sub(Raw& raw, const BCtx& c, int k0, int s) {
-        if (s != 0) return;
+    __device__ static __forceinline__ void load_sub(Raw& raw, const BCtx& c, int k0, int) {
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
             raw.r[t] = ldg_b128(c.rw, c.vw, (c.n0 + 16 * t) * (c.K >> 1) + (k0 >> 1));
@@ -282,6 +299,7 @@ struct BTraits<MOE_FMT_FP4_B32> {
 template <>
 struct BTraits<MOE_FMT_BF16> {
     static constexpr int BK = 64, NS = 2;
+    static constexpr int VALU_SUB = 0;
     static constexpr bool DOUBLE_RAW = false;
     static constexpr int MT_MAX = 11;  // 176 rows: the largest tile that keeps every value in registers
     struct Raw {
@@ -345,6 +363,8 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& P, u32x4_t* lds_a, i
     c.K = P.K; c.N = P.N; c.n0 = n0;
     c.i = lane & 15; c.q = lane >> 4; c.w = __builtin_amdgcn_readfirstlane(tid >> 6);
     c.gs = 1; c.sg = nullptr; c.og = nullptr; c.s8 = nullptr;
+    c.mlo = 0x0f0fu; c.mhi = 0xf0f0u;
+    asm volatile("" : "+s"(c.mlo), "+s"(c.mhi));
     const int64_t KN = (int64_t)P.K * P.N;
     switch (FMT) {
         case MOE_FMT_INT4:
@@ -410,41 +430,83 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& P, u32x4_t* lds_a, i
                 lds_a[buf * ABUF + a_lds_unit<BK>(ar + RPP * p, ac)] = areg[p];
     };
 
-    // Software pipeline, one barrier per k step.  Step kt computes from LDS buffer kt&1 and
-    // from `raw`; as soon as the fragments of a sub-step have been decoded, the same
-    // registers are reloaded with that sub-step of step kt+1 (formats whose loads span all
-    // sub-steps use a second register set instead), and the x tile of step kt+1
-    // travels through registers into the other LDS buffer.  The last step prefetches one
-    // step past K: buffer loads beyond a slab return 0 and the x rows it reads are inside
-    // the tensor; neither is used.
+    // Software pipeline, one barrier per k step (BK = NS sub-steps of 32 k).
+    //  * weights: the fragments of sub-step f+1 are decoded (VALU) while the MFMAs of
+    //    sub-step f run; as soon as a sub-step's packed registers have been decoded they
+    //    are reloaded with the same sub-step of the next k step (formats whose loads span a
+    //    whole step keep a second register set), so every weight load has one full k step
+    //    to land;
+    //  * x: fragments come from LDS through a ring of 4 registers sets, read RING
+    //    fragments ahead of their MFMAs; the x tile of step kt+1 travels through registers
+    //    into the other LDS buffer;
+    //  * sched_group_barrier pins the interleave: per x fragment one LDS read, then 4 times
+    //    (one MFMA + a share of the decode VALU work).
+    // The last steps prefetch past K: buffer loads beyond a slab return 0 and the x rows
+    // read are inside the tensor; neither is used.
+    constexpr int RING = 3, F = NS * MT;
+    constexpr int VPM = T::VALU_SUB == 0 ? 0 : (T::VALU_SUB + 4 * MT - 1) / (4 * MT);
+
     __syncthreads();  // previous tile's readers are done with both buffers
     load_a(0);
 #pragma unroll
-    for (int s = 0; s < NS; ++s) T::load_sub(raw, c, 0, s);
+    for (int s = 0; s < (T::DOUBLE_RAW ? 1 : NS); ++s) T::load_sub(raw, c, 0, s);
     store_a(0);
+    u32x4_t bf[4], bf_next[4];
+    ops.frags(raw, c, 0, bf);
+    if (T::DOUBLE_RAW)
+        T::load_sub(raw_next, c, BK, 0);
+    else
+        T::load_sub(raw, c, BK, 0);
     __syncthreads();
+
     for (int kt = 0; kt < nk; ++kt) {
         load_a(kt + 1);
         const u32x4_t* la = lds_a + (kt & 1) * ABUF;
+        u32x4_t afr[4];
+        auto read_a = [&](int f) {
+            afr[f & 3] = la[a_lds_unit<BK>(16 * (f % MT) + c.i, T::a_chunk(f / MT, c.q))];
+        };
+#pragma unroll
+        for (int f = 0; f < (RING < F ? RING : F); ++f) read_a(f);
 #pragma unroll
         for (int s = 0; s < NS; ++s) {
-            u32x4_t bf[4];
-            ops.frags(raw, c, s, bf);
-            T::load_sub(T::DOUBLE_RAW ? raw_next : raw, c, (kt + 1) * BK, s);
-            const int ch = T::a_chunk(s, c.q);
+            // decode the next sub-step's fragments, then refill the registers just consumed
+            if (s + 1 < NS) {
+                ops.frags(raw, c, s + 1, bf_next);
+                if (!T::DOUBLE_RAW) T::load_sub(raw, c, (kt + 1) * BK, s + 1);
+            } else {
+                if (T::DOUBLE_RAW) raw = raw_next;
+                ops.frags(raw, c, 0, bf_next);
+                if (T::DOUBLE_RAW)
+                    T::load_sub(raw_next, c, (kt + 2) * BK, 0);
+                else
+                    T::load_sub(raw, c, (kt + 2) * BK, 0);
+            }
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt) {
-                const u32x4_t av = la[a_lds_unit<BK>(16 * mt + c.i, ch)];
-                const bf16x8_t a8 = __builtin_bit_cast(bf16x8_t, av);
+                const int f = s * MT + mt;
+                if (f + RING < F) read_a(f + RING);
+                const bf16x8_t a8 = __builtin_bit_cast(bf16x8_t, afr[f & 3]);
 #pragma unroll
                 for (int t = 0; t < 4; ++t)
                     acc[mt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a8, __builtin_bit_cast(bf16x8_t, bf[t]),
                                                                          acc[mt][t], 0, 0, 0);
             }
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // one LDS read
+#pragma unroll
+                for (int t = 0; t < 4; ++t) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);             // one MFMA
+                    if (VPM) __builtin_amdgcn_sched_group_barrier(0x002, VPM, 0);  // decode VALU
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int t = 0; t < 4; ++t) bf[t] = bf_next[t];
         }
         store_a((kt + 1) & 1);
         __syncthreads();
-        if (T::DOUBLE_RAW) raw = raw_next;
     }
 
     // epilogue: fp32 -> bf16 (RNE), rows beyond the chunk are dropped
