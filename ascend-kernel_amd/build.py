@@ -39,8 +39,8 @@ def build_kernels(jobs: int = 4) -> str:
     os.makedirs(os.path.join(HERE, "build"), exist_ok=True)
     for src in KERNEL_SOURCES:
         obj = os.path.join(HERE, "build", src + ".o")
-        cmd = [HIPCC, *HIP_FLAGS, "-x", "hip", "-I", os.path.join(ROOT, "include"), "-I", CSRC, "-c",
-               os.path.join(CSRC, src), "-o", obj]
+        cmd = [HIPCC, *HIP_FLAGS, "-Rpass-analysis=kernel-resource-usage", "-x", "hip", "-I",
+               os.path.join(ROOT, "include"), "-I", CSRC, "-c", os.path.join(CSRC, src), "-o", obj]
         print("+", " ".join(cmd), flush=True)
         procs.append((src, subprocess.Popen(cmd, stderr=subprocess.PIPE, text=True)))
         objs.append(obj)
@@ -51,14 +51,31 @@ def build_kernels(jobs: int = 4) -> str:
     return LIB
 
 
+def _check_resources(src: str, remarks: list) -> None:
+    """The GEMM accumulators are updated by inline-asm MFMAs whose latency the compiler does
+    not track: they must stay in registers.  Any scratch use in a GEMM kernel means that
+    they (or the loops around them) were not fully promoted -- refuse such a build."""
+    name = None
+    for line in remarks:
+        if "Function Name:" in line:
+            name = line.split("Function Name:")[1].split()[0]
+        elif "ScratchSize [bytes/lane]:" in line and name and "grouped_gemm_kernel" in name:
+            scratch = int(line.split("ScratchSize [bytes/lane]:")[1].split()[0])
+            if scratch:
+                raise RuntimeError(f"{src}: {name} uses {scratch} bytes of scratch per lane")
+
+
 def _wait(procs):
     for src, p in procs:
         _, err = p.communicate()
-        err = "\n".join(l for l in err.splitlines() if "packed-fp32-ops" not in l)
+        lines = err.splitlines()
+        remarks = [l for l in lines if "-Rpass-analysis" in l]
+        err = "\n".join(l for l in lines if "packed-fp32-ops" not in l and "-Rpass-analysis" not in l)
         if err.strip():
             print(err, file=sys.stderr)
         if p.returncode:
             raise RuntimeError(f"hipcc failed on {src}")
+        _check_resources(src, remarks)
     procs.clear()
 
 

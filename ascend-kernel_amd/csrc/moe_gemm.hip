@@ -58,6 +58,15 @@ __device__ __forceinline__ u32x4_t ldg_b128(rsrc_t r, int voff, int soff) {
     return __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, 0);
 }
 
+// D = A * B + D with the accumulator tied to AGPRs.  Written as inline asm because the
+// compiler, given many live accumulators, stops accumulating in place and shuttles them
+// through copies, which halves the MFMA rate.  Hazards: A/B come from VALU or waited
+// loads (interlocked); accumulators are only read by other MFMAs until the epilogue,
+// which waits out the MFMA latency first.
+__device__ __forceinline__ void mfma_16x16x32(f32x4_t& acc, const u32x4_t& a, const u32x4_t& b) {
+    asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
+}
+
 // Per-lane view of one tile for the weight loaders.
 struct BCtx {
     rsrc_t rw, rs;       // weight / scale slab of the expert
@@ -65,11 +74,21 @@ struct BCtx {
     const uint16_t* sg;  // int8: scale / offset rows of the expert
     const uint16_t* og;
     const float* s8;     // fp8: scale blocks of the expert
-    int K, N, n0, gs;    // gs = k per scale group (int4)
+    int K, N, n0;
+    uint32_t gmul;       // int4: floor(2^32 / (group/32)) + 1 turns sub-step -> scale row into a
+                         // multiply (exact below 2^16 sub-steps); 0 when the group is 32
     int i, q, w;         // lane & 15, lane >> 4, wavefront (scalar)
     uint32_t mlo, mhi;   // 0x0f0f / 0xf0f0, opaque to the optimizer (int4 decode)
 };
 
+// Each weight container provides
+//   Raw        packed registers of one k step (or one sub-step ring, see load_sub)
+//   load_sub   global loads of 32-k sub-step s of the step starting at k0
+//   Dq         the decode, cut into units so that it can be interleaved with MFMAs:
+//              prep(raw, c, s) once per sub-step, then unit(raw, c, s, p, t, out) for
+//              p, t in [0,4) writes dword p (k pair) of the fragment of MFMA t
+//   a_chunk    which 16-byte chunk of the x tile row matches the k values of (s, q)
+//   col        output column (relative to n0) of MFMA t in this lane
 template <int FMT>
 struct BTraits;
 
@@ -85,7 +104,6 @@ struct BTraits;
 template <>
 struct BTraits<MOE_FMT_INT4> {
     static constexpr int BK = 64, NS = 2;
-    static constexpr int VALU_SUB = 116;  // decode instructions per 32-k sub-step (interleave hint)
     static constexpr bool DOUBLE_RAW = false;
     static constexpr int MT_MAX = 11;  // 176 rows: the largest tile that keeps every value in registers
     struct Raw {
@@ -106,29 +124,36 @@ struct BTraits<MOE_FMT_INT4> {
         for (int j = 0; j < 8; ++j)
             raw.r[s][j] = ldg_b32(c.rw, c.vw, (k0 + 32 * s + j) * nb + (c.n0 >> 1));
         // a 32-k sub-step never straddles a scale group (group % 32 == 0)
-        raw.sc[s] = ldg_b64(c.rs, c.vs, (((k0 + 32 * s) / c.gs) * c.N + c.n0) * 2);
+        const uint32_t sub = (uint32_t)((k0 >> 5) + s);
+        const int grow = c.gmul ? (int)__umulhi(sub, c.gmul) : (int)sub;
+        raw.sc[s] = ldg_b64(c.rs, c.vs, (grow * c.N + c.n0) * 2);
     }
-    // Byte -> fp32 converts.  The nibble masks come from BCtx as values the compiler cannot
-    // see through; with literal masks it folds them into every extraction and spends an
-    // extra instruction per element instead of using v_cvt_f32_ubyte0 / ubyte1 directly.
+    // The nibble masks come from BCtx as values the compiler cannot see through; with literal
+    // masks it folds them into every extraction and spends an extra instruction per element
+    // instead of using v_cvt_f32_ubyte0 / ubyte1 directly.
     __device__ static __forceinline__ float ubyte0(uint32_t v) { return (float)(v & 0xffu); }
     __device__ static __forceinline__ float ubyte1(uint32_t v) { return (float)((v >> 8) & 0xffu); }
-    __device__ static __forceinline__ void frags(const Raw& raw, const BCtx& c, int s, u32x4_t out[4]) {
-        const int sh = 16 * (c.w & 1);
-        const float s0 = bf16_lo(raw.sc[s][0]), s1 = bf16_hi(raw.sc[s][0]);
-        const float s2 = bf16_lo(raw.sc[s][1]), s3 = bf16_hi(raw.sc[s][1]);
-        const float h1 = s1 * 0.0625f, h3 = s3 * 0.0625f;           // odd nibbles arrive times 16
-        const float z0 = -8.f * s0, z1 = -8.f * s1, z2 = -8.f * s2, z3 = -8.f * s3;
-#pragma unroll
-        for (int j = 0; j < 8; j += 2) {
-            const uint32_t a = raw.r[s][j] >> sh, b = raw.r[s][j + 1] >> sh;
-            const uint32_t al = a & c.mlo, ah = a & c.mhi, bl = b & c.mlo, bh = b & c.mhi;
-            out[0][j >> 1] = pack_bf16_rne(fmaf(ubyte0(al), s0, z0), fmaf(ubyte0(bl), s0, z0));
-            out[1][j >> 1] = pack_bf16_rne(fmaf(ubyte0(ah), h1, z1), fmaf(ubyte0(bh), h1, z1));
-            out[2][j >> 1] = pack_bf16_rne(fmaf(ubyte1(al), s2, z2), fmaf(ubyte1(bl), s2, z2));
-            out[3][j >> 1] = pack_bf16_rne(fmaf(ubyte1(ah), h3, z3), fmaf(ubyte1(bh), h3, z3));
+    struct Dq {
+        float m[4], z[4];        // multiplier and zero-point term of the 4 columns
+        uint32_t al, ah, bl, bh; // masked halves of the two k rows of the current pair
+        __device__ __forceinline__ void init_tile(const BCtx&) {}
+        __device__ __forceinline__ void prep(const Raw& raw, const BCtx&, int s) {
+            const float s0 = bf16_lo(raw.sc[s][0]), s1 = bf16_hi(raw.sc[s][0]);
+            const float s2 = bf16_lo(raw.sc[s][1]), s3 = bf16_hi(raw.sc[s][1]);
+            m[0] = s0; m[1] = s1 * 0.0625f; m[2] = s2; m[3] = s3 * 0.0625f;  // odd nibbles arrive times 16
+            z[0] = -8.f * s0; z[1] = -8.f * s1; z[2] = -8.f * s2; z[3] = -8.f * s3;
         }
-    }
+        __device__ __forceinline__ void unit(const Raw& raw, const BCtx& c, int s, int p, int t, u32x4_t out[4]) {
+            if (t == 0) {
+                const int sh = 16 * (c.w & 1);
+                const uint32_t a = raw.r[s][2 * p] >> sh, b = raw.r[s][2 * p + 1] >> sh;
+                al = a & c.mlo; ah = a & c.mhi; bl = b & c.mlo; bh = b & c.mhi;
+            }
+            const uint32_t ua = (t & 1) ? ah : al, ub = (t & 1) ? bh : bl;
+            const float fa = (t & 2) ? ubyte1(ua) : ubyte0(ua), fb = (t & 2) ? ubyte1(ub) : ubyte0(ub);
+            out[t][p] = pack_bf16_rne(fmaf(fa, m[t], z[t]), fmaf(fb, m[t], z[t]));
+        }
+    };
 };
 
 // ---------------------------------------------- reference "fp4": pre-shuffled [K, N/2]
@@ -139,9 +164,8 @@ struct BTraits<MOE_FMT_INT4> {
 template <>
 struct BTraits<MOE_FMT_FP4_REF> {
     static constexpr int BK = 64, NS = 2;
-    static constexpr int VALU_SUB = 84;
     static constexpr bool DOUBLE_RAW = false;
-    static constexpr int MT_MAX = 11;  // 176 rows: the largest tile that keeps every value in registers
+    static constexpr int MT_MAX = 11;
     struct Raw {
         u32x4_t r[2][2];
         u32x2_t sc[2];
@@ -164,21 +188,25 @@ struct BTraits<MOE_FMT_FP4_REF> {
         raw.r[s][1] = ldg_b128(c.rw, c.vw, so + 16);
         raw.sc[s] = ldg_b64(c.rs, c.vs, (((k0 + 32 * s) >> 4) * c.N + c.n0) * 2);
     }
-    __device__ static __forceinline__ void frags(const Raw& raw, const BCtx& c, int s, u32x4_t out[4]) {
-        const int sh = 16 * (c.w & 1);
-        const float sc[4] = {bf16_lo(raw.sc[s][0]), bf16_hi(raw.sc[s][0]), bf16_lo(raw.sc[s][1]),
-                             bf16_hi(raw.sc[s][1])};
-#pragma unroll
-        for (int j = 0; j < 8; j += 2) {
-            const uint32_t a = raw.r[s][j >> 2][j & 3] >> sh, b = raw.r[s][(j + 1) >> 2][(j + 1) & 3] >> sh;
-            const f32x2_t a01 = e2m1_pair_to_f32<0>(a), a23 = e2m1_pair_to_f32<1>(a);
-            const f32x2_t b01 = e2m1_pair_to_f32<0>(b), b23 = e2m1_pair_to_f32<1>(b);
-            out[0][j >> 1] = pack_bf16_rne(a01[0] * sc[0], b01[0] * sc[0]);
-            out[1][j >> 1] = pack_bf16_rne(a01[1] * sc[1], b01[1] * sc[1]);
-            out[2][j >> 1] = pack_bf16_rne(a23[0] * sc[2], b23[0] * sc[2]);
-            out[3][j >> 1] = pack_bf16_rne(a23[1] * sc[3], b23[1] * sc[3]);
+    struct Dq {
+        float sc[4];
+        f32x2_t va, vb;  // decoded pair of the current byte for the two k rows
+        __device__ __forceinline__ void init_tile(const BCtx&) {}
+        __device__ __forceinline__ void prep(const Raw& raw, const BCtx&, int s) {
+            sc[0] = bf16_lo(raw.sc[s][0]); sc[1] = bf16_hi(raw.sc[s][0]);
+            sc[2] = bf16_lo(raw.sc[s][1]); sc[3] = bf16_hi(raw.sc[s][1]);
         }
-    }
+        __device__ __forceinline__ void unit(const Raw& raw, const BCtx& c, int s, int p, int t, u32x4_t out[4]) {
+            if ((t & 1) == 0) {
+                const int sh = 16 * (c.w & 1);
+                const int j = 2 * p;
+                const uint32_t a = raw.r[s][j >> 2][j & 3] >> sh, b = raw.r[s][(j + 1) >> 2][(j + 1) & 3] >> sh;
+                if (t == 0) { va = e2m1_pair_to_f32<0>(a); vb = e2m1_pair_to_f32<0>(b); }
+                else        { va = e2m1_pair_to_f32<1>(a); vb = e2m1_pair_to_f32<1>(b); }
+            }
+            out[t][p] = pack_bf16_rne(va[t & 1] * sc[t], vb[t & 1] * sc[t]);
+        }
+    };
 };
 
 // ------------------------------------------------------- int8 / reference fp8, [K, N]
@@ -186,9 +214,8 @@ struct BTraits<MOE_FMT_FP4_REF> {
 template <int FMT>
 struct BTraitsByte {
     static constexpr int BK = 64, NS = 2;
-    static constexpr int VALU_SUB = FMT == MOE_FMT_INT8 ? 120 : 210;
     static constexpr bool DOUBLE_RAW = false;
-    static constexpr int MT_MAX = 11;  // 176 rows: the largest tile that keeps every value in registers
+    static constexpr int MT_MAX = 11;
     struct Raw {
         uint32_t r[2][8];
         float s8[2];  // fp8: scale of the 128x128 block of each sub-step
@@ -203,7 +230,7 @@ struct BTraitsByte {
 #pragma unroll
         for (int j = 0; j < 8; ++j) raw.r[s][j] = ldg_b32(c.rw, c.vw, (k0 + 32 * s + j) * c.N + c.n0);
         if (FMT == MOE_FMT_FP8_REF) {
-            // the one-step-ahead prefetch may point past K: clamp the block row (value unused then)
+            // the prefetch may point past K: clamp the block row (value unused then)
             const int kb = min(k0 >> 7, (c.K >> 7) - 1);
             raw.s8[s] = c.s8[kb * (c.N >> 7) + ((c.n0 + 64 * c.w) >> 7)];
         }
@@ -212,42 +239,35 @@ struct BTraitsByte {
 
 template <>
 struct BTraits<MOE_FMT_INT8> : BTraitsByte<MOE_FMT_INT8> {
-    // per-channel scale and offset of this lane's 4 columns, fixed for the whole tile
-    float sc[4], of[4];
-    __device__ __forceinline__ void prepare_m(const BCtx& c) {
-        const u32x2_t s = *reinterpret_cast<const u32x2_t*>(c.sg + c.n0 + col(c, 0));
-        const u32x2_t o = *reinterpret_cast<const u32x2_t*>(c.og + c.n0 + col(c, 0));
-        sc[0] = bf16_lo(s[0]); sc[1] = bf16_hi(s[0]); sc[2] = bf16_lo(s[1]); sc[3] = bf16_hi(s[1]);
-        of[0] = bf16_lo(o[0]); of[1] = bf16_hi(o[0]); of[2] = bf16_lo(o[1]); of[3] = bf16_hi(o[1]);
-    }
-    __device__ __forceinline__ void frags_m(const Raw& raw, const BCtx&, int s, u32x4_t out[4]) const {
-#pragma unroll
-        for (int j = 0; j < 8; j += 2) {
-            const uint32_t a = raw.r[s][j], b = raw.r[s][j + 1];
-#pragma unroll
-            for (int t = 0; t < 4; ++t) {
-                const float qa = (float)(int)(int8_t)(a >> (8 * t)), qb = (float)(int)(int8_t)(b >> (8 * t));
-                // (q + offset) * scale as two rounded fp32 operations
-                out[t][j >> 1] = pack_bf16_rne(__fmul_rn(__fadd_rn(qa, of[t]), sc[t]),
-                                               __fmul_rn(__fadd_rn(qb, of[t]), sc[t]));
-            }
+    struct Dq {
+        float sc[4], of[4];  // per-channel scale and offset of this lane's 4 columns, fixed for the tile
+        __device__ __forceinline__ void init_tile(const BCtx& c) {
+            const u32x2_t s = *reinterpret_cast<const u32x2_t*>(c.sg + c.n0 + col(c, 0));
+            const u32x2_t o = *reinterpret_cast<const u32x2_t*>(c.og + c.n0 + col(c, 0));
+            sc[0] = bf16_lo(s[0]); sc[1] = bf16_hi(s[0]); sc[2] = bf16_lo(s[1]); sc[3] = bf16_hi(s[1]);
+            of[0] = bf16_lo(o[0]); of[1] = bf16_hi(o[0]); of[2] = bf16_lo(o[1]); of[3] = bf16_hi(o[1]);
         }
-    }
+        __device__ __forceinline__ void prep(const Raw&, const BCtx&, int) {}
+        __device__ __forceinline__ void unit(const Raw& raw, const BCtx&, int s, int p, int t, u32x4_t out[4]) {
+            const uint32_t a = raw.r[s][2 * p], b = raw.r[s][2 * p + 1];
+            const float qa = (float)(int)(int8_t)(a >> (8 * t)), qb = (float)(int)(int8_t)(b >> (8 * t));
+            // (q + offset) * scale as two rounded fp32 operations
+            out[t][p] = pack_bf16_rne(__fmul_rn(__fadd_rn(qa, of[t]), sc[t]), __fmul_rn(__fadd_rn(qb, of[t]), sc[t]));
+        }
+    };
 };
 
 template <>
 struct BTraits<MOE_FMT_FP8_REF> : BTraitsByte<MOE_FMT_FP8_REF> {
-    __device__ __forceinline__ void prepare_m(const BCtx&) {}
-    __device__ __forceinline__ void frags_m(const Raw& raw, const BCtx&, int s, u32x4_t out[4]) const {
-#pragma unroll
-        for (int j = 0; j < 8; j += 2) {
-            const uint32_t a = raw.r[s][j], b = raw.r[s][j + 1];
-#pragma unroll
-            for (int t = 0; t < 4; ++t)
-                out[t][j >> 1] = pack_bf16_rne(e4m3_ref_to_f32((a >> (8 * t)) & 0xffu) * raw.s8[s],
-                                               e4m3_ref_to_f32((b >> (8 * t)) & 0xffu) * raw.s8[s]);
+    struct Dq {
+        __device__ __forceinline__ void init_tile(const BCtx&) {}
+        __device__ __forceinline__ void prep(const Raw&, const BCtx&, int) {}
+        __device__ __forceinline__ void unit(const Raw& raw, const BCtx&, int s, int p, int t, u32x4_t out[4]) {
+            const uint32_t a = raw.r[s][2 * p], b = raw.r[s][2 * p + 1];
+            out[t][p] = pack_bf16_rne(e4m3_ref_to_f32((a >> (8 * t)) & 0xffu) * raw.s8[s],
+                                      e4m3_ref_to_f32((b >> (8 * t)) & 0xffu) * raw.s8[s]);
         }
-    }
+    };
 };
 
 // -------------------------------------------------------- fp4 block-32, [N, K/2]
@@ -257,6 +277,11 @@ struct BTraits<MOE_FMT_FP8_REF> : BTraitsByte<MOE_FMT_FP8_REF> {
 template <>
 struct BTraits<MOE_FMT_FP4_B32> {
     static constexpr int BK = 128, NS = 4;
+    // One 16-byte load per t serves all 4 sub-steps, so the registers cannot be reloaded
+    // sub-step by sub-step: a whole step is loaded into a second register set (load_sub
+    // ignores its sub-step argument and is called once per step).
+    static constexpr bool DOUBLE_RAW = true;
+    static constexpr int MT_MAX = 10;  // larger tiles spill: BK = 128 doubles the x staging registers
     struct Raw {
         u32x4_t r[4];
         float sc[4];
@@ -267,12 +292,6 @@ struct BTraits<MOE_FMT_FP4_B32> {
         c.vw = (64 * c.w + c.i) * (c.K >> 1) + 16 * c.q;
         c.vs = ((64 * c.w + c.i) * (c.K >> 5) + c.q) * 2;
     }
-    // One 16-byte load per t serves all 4 sub-steps, so the registers cannot be reloaded
-    // sub-step by sub-step: a whole step is loaded into a second register set (load_sub
-    // ignores its sub-step argument and is called once per step).
-    static constexpr bool DOUBLE_RAW = true;
-    static constexpr int VALU_SUB = 64;  // decode instructions per 32-k sub-step (interleave hint)
-    static constexpr int MT_MAX = 10;  // larger tiles spill: BK = 128 doubles the x staging registers
     __device__ static __forceinline__ void load_sub(Raw& raw, const BCtx& c, int k0, int) {
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
@@ -281,16 +300,17 @@ struct BTraits<MOE_FMT_FP4_B32> {
                 __builtin_amdgcn_raw_buffer_load_b16(c.rs, c.vs, ((c.n0 + 16 * t) * (c.K >> 5) + (k0 >> 5)) * 2, 0));
         }
     }
-    __device__ static __forceinline__ void frags(const Raw& raw, const BCtx&, int s, u32x4_t out[4]) {
-#pragma unroll
-        for (int t = 0; t < 4; ++t) {
+    struct Dq {
+        __device__ __forceinline__ void init_tile(const BCtx&) {}
+        __device__ __forceinline__ void prep(const Raw&, const BCtx&, int) {}
+        __device__ __forceinline__ void unit(const Raw& raw, const BCtx&, int s, int p, int t, u32x4_t out[4]) {
             const uint32_t wd = raw.r[t][s];
-            out[t][0] = e2m1_pair_scaled_bf16<0>(wd, raw.sc[t]);
-            out[t][1] = e2m1_pair_scaled_bf16<1>(wd, raw.sc[t]);
-            out[t][2] = e2m1_pair_scaled_bf16<2>(wd, raw.sc[t]);
-            out[t][3] = e2m1_pair_scaled_bf16<3>(wd, raw.sc[t]);
+            out[t][p] = p == 0   ? e2m1_pair_scaled_bf16<0>(wd, raw.sc[t])
+                        : p == 1 ? e2m1_pair_scaled_bf16<1>(wd, raw.sc[t])
+                        : p == 2 ? e2m1_pair_scaled_bf16<2>(wd, raw.sc[t])
+                                 : e2m1_pair_scaled_bf16<3>(wd, raw.sc[t]);
         }
-    }
+    };
 };
 
 // ------------------------------------------------------------------ bf16, [N, K]
@@ -299,9 +319,8 @@ struct BTraits<MOE_FMT_FP4_B32> {
 template <>
 struct BTraits<MOE_FMT_BF16> {
     static constexpr int BK = 64, NS = 2;
-    static constexpr int VALU_SUB = 0;
     static constexpr bool DOUBLE_RAW = false;
-    static constexpr int MT_MAX = 11;  // 176 rows: the largest tile that keeps every value in registers
+    static constexpr int MT_MAX = 11;
     struct Raw {
         u32x4_t r[4][2];
     };
@@ -315,26 +334,13 @@ struct BTraits<MOE_FMT_BF16> {
 #pragma unroll
         for (int t = 0; t < 4; ++t) raw.r[t][s] = ldg_b128(c.rw, c.vw, ((c.n0 + 16 * t) * c.K + k0) * 2 + 16 * s);
     }
-    __device__ static __forceinline__ void frags(const Raw& raw, const BCtx&, int s, u32x4_t out[4]) {
-#pragma unroll
-        for (int t = 0; t < 4; ++t) out[t] = raw.r[t][s];
-    }
-};
-
-// Uniform wrappers: formats with per-tile state (int8) use member functions.
-template <int FMT>
-struct BOps {
-    BTraits<FMT> st;
-    __device__ __forceinline__ void prepare(const BCtx& c) {
-        if constexpr (FMT == MOE_FMT_INT8 || FMT == MOE_FMT_FP8_REF) st.prepare_m(c);
-    }
-    __device__ __forceinline__ void frags(const typename BTraits<FMT>::Raw& raw, const BCtx& c, int s,
-                                          u32x4_t out[4]) const {
-        if constexpr (FMT == MOE_FMT_INT8 || FMT == MOE_FMT_FP8_REF)
-            st.frags_m(raw, c, s, out);
-        else
-            BTraits<FMT>::frags(raw, c, s, out);
-    }
+    struct Dq {
+        __device__ __forceinline__ void init_tile(const BCtx&) {}
+        __device__ __forceinline__ void prep(const Raw&, const BCtx&, int) {}
+        __device__ __forceinline__ void unit(const Raw& raw, const BCtx&, int s, int p, int t, u32x4_t out[4]) {
+            out[t][p] = raw.r[t][s][p];
+        }
+    };
 };
 
 // ---------------------------------------------------------------------------------
@@ -362,7 +368,7 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& P, u32x4_t* lds_a, i
     BCtx c;
     c.K = P.K; c.N = P.N; c.n0 = n0;
     c.i = lane & 15; c.q = lane >> 4; c.w = __builtin_amdgcn_readfirstlane(tid >> 6);
-    c.gs = 1; c.sg = nullptr; c.og = nullptr; c.s8 = nullptr;
+    c.gmul = 0; c.sg = nullptr; c.og = nullptr; c.s8 = nullptr;
     c.mlo = 0x0f0fu; c.mhi = 0xf0f0u;
     asm volatile("" : "+s"(c.mlo), "+s"(c.mhi));
     const int64_t KN = (int64_t)P.K * P.N;
@@ -371,7 +377,10 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& P, u32x4_t* lds_a, i
             c.rw = make_rsrc(P.w + g * (KN >> 1), KN >> 1);
             c.rs = make_rsrc(static_cast<const uint16_t*>(P.scale) + (int64_t)g * P.scale_rows * P.N,
                              (int64_t)P.scale_rows * P.N * 2);
-            c.gs = P.K / P.scale_rows;
+            {
+                const uint32_t per = (uint32_t)((P.K / P.scale_rows) >> 5);  // sub-steps per scale group
+                c.gmul = per == 1 ? 0u : 0xffffffffu / per + 1u;
+            }
             break;
         case MOE_FMT_FP4_REF:
             c.rw = make_rsrc(P.w + g * (KN >> 1), KN >> 1);
@@ -398,8 +407,8 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& P, u32x4_t* lds_a, i
             break;
     }
     T::init(c);
-    BOps<FMT> ops;
-    ops.prepare(c);
+    typename T::Dq dq;
+    dq.init_tile(c);
 
     // x rows of this tile through a buffer resource that ends after the last valid row:
     // padded rows read as zeros.  This thread loads chunk ac of rows ar + RPP*p.
@@ -430,29 +439,33 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& P, u32x4_t* lds_a, i
                 lds_a[buf * ABUF + a_lds_unit<BK>(ar + RPP * p, ac)] = areg[p];
     };
 
-    // Software pipeline, one barrier per k step (BK = NS sub-steps of 32 k).
-    //  * weights: the fragments of sub-step f+1 are decoded (VALU) while the MFMAs of
-    //    sub-step f run; as soon as a sub-step's packed registers have been decoded they
-    //    are reloaded with the same sub-step of the next k step (formats whose loads span a
-    //    whole step keep a second register set), so every weight load has one full k step
-    //    to land;
-    //  * x: fragments come from LDS through a ring of 4 registers sets, read RING
+    // Software pipeline, one barrier per k step (BK = NS sub-steps of 32 k), every
+    // instruction placed by hand (sched_barrier after each MFMA slot):
+    //  * weights: while the MFMAs of sub-step f run, the fragments of sub-step f+1 are
+    //    decoded, one unit (two elements of one column) at a time between MFMAs; as soon as
+    //    a sub-step's packed registers have been decoded they are reloaded with the same
+    //    sub-step of the next k step (formats whose loads span a whole step keep a second
+    //    register set), so every weight load has one full k step to land;
+    //  * x: fragments come from LDS through a ring of 4 register sets, read RING
     //    fragments ahead of their MFMAs; the x tile of step kt+1 travels through registers
-    //    into the other LDS buffer;
-    //  * sched_group_barrier pins the interleave: per x fragment one LDS read, then 4 times
-    //    (one MFMA + a share of the decode VALU work).
+    //    into the other LDS buffer.
     // The last steps prefetch past K: buffer loads beyond a slab return 0 and the x rows
     // read are inside the tensor; neither is used.
     constexpr int RING = 3, F = NS * MT;
-    constexpr int VPM = T::VALU_SUB == 0 ? 0 : (T::VALU_SUB + 4 * MT - 1) / (4 * MT);
+    constexpr int SLOTS = 4 * MT;   // MFMAs per sub-step
+    constexpr int UNITS = 17;       // prep + 16 decode units per sub-step
 
     __syncthreads();  // previous tile's readers are done with both buffers
     load_a(0);
 #pragma unroll
     for (int s = 0; s < (T::DOUBLE_RAW ? 1 : NS); ++s) T::load_sub(raw, c, 0, s);
     store_a(0);
-    u32x4_t bf[4], bf_next[4];
-    ops.frags(raw, c, 0, bf);
+    u32x4_t bf[2][4];
+    dq.prep(raw, c, 0);
+#pragma unroll
+    for (int p = 0; p < 4; ++p)
+#pragma unroll
+        for (int t = 0; t < 4; ++t) dq.unit(raw, c, 0, p, t, bf[0]);
     if (T::DOUBLE_RAW)
         T::load_sub(raw_next, c, BK, 0);
     else
@@ -468,46 +481,42 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& P, u32x4_t* lds_a, i
         };
 #pragma unroll
         for (int f = 0; f < (RING < F ? RING : F); ++f) read_a(f);
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int s = 0; s < NS; ++s) {
-            // decode the next sub-step's fragments, then refill the registers just consumed
-            if (s + 1 < NS) {
-                ops.frags(raw, c, s + 1, bf_next);
-                if (!T::DOUBLE_RAW) T::load_sub(raw, c, (kt + 1) * BK, s + 1);
-            } else {
-                if (T::DOUBLE_RAW) raw = raw_next;
-                ops.frags(raw, c, 0, bf_next);
-                if (T::DOUBLE_RAW)
-                    T::load_sub(raw_next, c, (kt + 2) * BK, 0);
-                else
-                    T::load_sub(raw, c, (kt + 2) * BK, 0);
-            }
+            const int sn = (s + 1) % NS;                 // sub-step being decoded
+            u32x4_t* bcur = bf[s & 1];
+            u32x4_t* bnxt = bf[(s + 1) & 1];
+            if (T::DOUBLE_RAW && sn == 0) raw = raw_next;  // the next step's registers become current
 #pragma unroll
-            for (int mt = 0; mt < MT; ++mt) {
-                const int f = s * MT + mt;
-                if (f + RING < F) read_a(f + RING);
-                const bf16x8_t a8 = __builtin_bit_cast(bf16x8_t, afr[f & 3]);
+            for (int slot = 0; slot < SLOTS; ++slot) {
+                const int mt = slot >> 2, t = slot & 3, f = s * MT + mt;
+                if (t == 0 && f + RING < F) read_a(f + RING);
+                mfma_16x16x32(acc[mt][t], afr[f & 3], bcur[t]);
+                // decode units u with floor(u * SLOTS / UNITS) == slot
 #pragma unroll
-                for (int t = 0; t < 4; ++t)
-                    acc[mt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a8, __builtin_bit_cast(bf16x8_t, bf[t]),
-                                                                         acc[mt][t], 0, 0, 0);
-            }
-#pragma unroll
-            for (int mt = 0; mt < MT; ++mt) {
-                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // one LDS read
-#pragma unroll
-                for (int t = 0; t < 4; ++t) {
-                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);             // one MFMA
-                    if (VPM) __builtin_amdgcn_sched_group_barrier(0x002, VPM, 0);  // decode VALU
+                for (int u = (slot * UNITS + SLOTS - 1) / SLOTS; u < ((slot + 1) * UNITS + SLOTS - 1) / SLOTS; ++u) {
+                    if (u == 0)
+                        dq.prep(raw, c, sn);
+                    else
+                        dq.unit(raw, c, sn, (u - 1) >> 2, (u - 1) & 3, bnxt);
                 }
+                if (slot == ((UNITS - 1) * SLOTS) / UNITS) {
+                    // everything of sub-step sn has been decoded: refill its registers
+                    if (T::DOUBLE_RAW) {
+                        if (sn == 0) T::load_sub(raw_next, c, (kt + 2) * BK, 0);
+                    } else {
+                        T::load_sub(raw, c, (kt + (sn == 0 ? 2 : 1)) * BK, sn);
+                    }
+                }
+                __builtin_amdgcn_sched_barrier(0);
             }
-            __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for (int t = 0; t < 4; ++t) bf[t] = bf_next[t];
         }
         store_a((kt + 1) & 1);
         __syncthreads();
     }
+    // the accumulators were last written by MFMAs the compiler cannot see: wait out their latency
+    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
 
     // epilogue: fp32 -> bf16 (RNE), rows beyond the chunk are dropped
     constexpr bool N_CONTIG = (FMT == MOE_FMT_INT4 || FMT == MOE_FMT_FP4_REF || FMT == MOE_FMT_INT8 ||
