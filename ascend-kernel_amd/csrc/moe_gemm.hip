@@ -93,10 +93,15 @@ template <int FMT>
 struct BTraits;
 
 // ------------------------------------------------------------------ int4, [K, N/2]
-// Lane (i, q) of wavefront w owns the 4 columns 128(w>>1) + 8i + 4(w&1) + [0,4): for each
-// of its 8 k rows it loads the dword holding the 8 columns 128(w>>1) + 8i + [0,8) and
-// shifts its half down (wavefronts 2p and 2p+1 read the same dwords).  MFMA t gets
-// nibble t of that half.
+// Lane (i, q) of wavefront w owns the 4 columns 128(w>>1) + 8i + 4(w&1) + [0,4), i.e. half
+// of the dword holding the 8 columns 128(w>>1) + 8i + [0,8) of each of its 8 k rows
+// (wavefronts 2p and 2p+1 use the two halves of the same dwords).  MFMA t gets nibble t
+// of that half.
+// The packed 64(k) x 128 B tile of a k step goes HBM -> registers -> LDS with two
+// coalesced 16-byte loads per thread (the vector-memory address unit handles a 16-byte
+// load in the time of a 4-byte one), and each lane then picks its dwords from LDS.  In
+// LDS the two 64-byte halves of the rows with odd (row >> 3) are swapped, so that the
+// four q groups of a wavefront read from both halves of the banks.
 // Decode: byte b of (v & 0x0f0f) is nibble 2b, byte b of (v & 0xf0f0) is
 // 16 * nibble 2b+1; v_cvt_f32_ubyteN turns either into fp32 and one fma applies
 // scale (or scale/16) and the zero point: q*s - 8s = (q - 8)*s exactly (<= 12 significant
@@ -106,6 +111,8 @@ struct BTraits<MOE_FMT_INT4> {
     static constexpr int BK = 64, NS = 2;
     static constexpr bool DOUBLE_RAW = false;
     static constexpr int MT_MAX = 11;  // 176 rows: the largest tile that keeps every value in registers
+    static constexpr int B_LDS_UNITS = 64 * 8;  // 16-byte units of one packed tile in LDS (0: no LDS staging)
+    static constexpr int B_LOADS = 2;           // 16-byte global loads per thread per k step
     struct Raw {
         uint32_t r[2][8];
         u32x2_t sc[2];
@@ -115,15 +122,34 @@ struct BTraits<MOE_FMT_INT4> {
         return 128 * (c.w >> 1) + 8 * c.i + 4 * (c.w & 1) + t;
     }
     __device__ static __forceinline__ void init(BCtx& c) {
-        c.vw = 8 * c.q * (c.N >> 1) + 64 * (c.w >> 1) + 4 * c.i;
+        const int tid = 64 * c.w + 16 * c.q + c.i;
+        c.vw = (tid >> 3) * (c.N >> 1) + (tid & 7) * 16;   // staging: row tid>>3 (+32), chunk tid&7
         c.vs = col(c, 0) * 2;
     }
-    __device__ static __forceinline__ void load_sub(Raw& raw, const BCtx& c, int k0, int s) {
+    // global -> registers: rows (tid >> 3) + 32h of the tile of the step starting at k0
+    __device__ static __forceinline__ void stage_load(u32x4_t breg[B_LOADS], const BCtx& c, int k0) {
         const int nb = c.N >> 1;
 #pragma unroll
-        for (int j = 0; j < 8; ++j)
-            raw.r[s][j] = ldg_b32(c.rw, c.vw, (k0 + 32 * s + j) * nb + (c.n0 >> 1));
-        // a 32-k sub-step never straddles a scale group (group % 32 == 0)
+        for (int h = 0; h < B_LOADS; ++h) breg[h] = ldg_b128(c.rw, c.vw, (k0 + 32 * h) * nb + (c.n0 >> 1));
+    }
+    // registers -> LDS tile
+    __device__ static __forceinline__ void stage_store(u32x4_t* tile, const u32x4_t breg[B_LOADS], const BCtx& c) {
+        const int tid = 64 * c.w + 16 * c.q + c.i;
+        const int r = tid >> 3, ch = tid & 7;
+#pragma unroll
+        for (int h = 0; h < B_LOADS; ++h) tile[(r + 32 * h) * 8 + (ch ^ (4 * ((r >> 3) & 1)))] = breg[h];
+    }
+    // LDS tile -> this lane's dwords of sub-step s
+    __device__ static __forceinline__ void load_sub(Raw& raw, const BCtx& c, int, int s, const u32x4_t* tile) {
+        const uint32_t* t32 = reinterpret_cast<const uint32_t*>(tile);
+        const int d = 16 * (c.w >> 1) + c.i;  // dword of the row
+        const int unit = (d >> 2) ^ (4 * (c.q & 1));
+#pragma unroll
+        for (int j = 0; j < 8; ++j) raw.r[s][j] = t32[((32 * s + 8 * c.q + j) * 8 + unit) * 4 + (d & 3)];
+    }
+    // The scales of sub-step s of the step starting at k0 come straight from global memory, a
+    // full step ahead.  A 32-k sub-step never straddles a scale group (group % 32 == 0).
+    __device__ static __forceinline__ void load_scale(Raw& raw, const BCtx& c, int k0, int s) {
         const uint32_t sub = (uint32_t)((k0 >> 5) + s);
         const int grow = c.gmul ? (int)__umulhi(sub, c.gmul) : (int)sub;
         raw.sc[s] = ldg_b64(c.rs, c.vs, (grow * c.N + c.n0) * 2);
@@ -164,12 +190,16 @@ struct BTraits<MOE_FMT_INT4> {
 template <>
 struct BTraits<MOE_FMT_FP4_REF> {
     static constexpr int BK = 64, NS = 2;
+    static constexpr int B_LDS_UNITS = 0, B_LOADS = 1;
     static constexpr bool DOUBLE_RAW = false;
     static constexpr int MT_MAX = 11;
     struct Raw {
         u32x4_t r[2][2];
         u32x2_t sc[2];
     };
+    __device__ static __forceinline__ void stage_load(u32x4_t*, const BCtx&, int) {}
+    __device__ static __forceinline__ void stage_store(u32x4_t*, const u32x4_t*, const BCtx&) {}
+    __device__ static __forceinline__ void load_scale(Raw&, const BCtx&, int, int) {}
     __device__ static __forceinline__ int a_chunk(int s, int q) { return 4 * s + q; }
     __device__ static __forceinline__ int col(const BCtx& c, int t) {
         return 128 * (c.w >> 1) + 8 * c.i + 4 * (c.w & 1) + t;
@@ -181,7 +211,7 @@ struct BTraits<MOE_FMT_FP4_REF> {
         c.vw = R0 * (c.N >> 1) + 32 * qq;
         c.vs = ((c.q >> 1) * c.N + col(c, 0)) * 2;  // scale group of 16 k: (k0 + 32s)/16 + (q >> 1)
     }
-    __device__ static __forceinline__ void load_sub(Raw& raw, const BCtx& c, int k0, int s) {
+    __device__ static __forceinline__ void load_sub(Raw& raw, const BCtx& c, int k0, int s, const u32x4_t*) {
         const int nb = c.N >> 1;
         const int so = (k0 + 16 * s) * nb + (c.n0 >> 1);
         raw.r[s][0] = ldg_b128(c.rw, c.vw, so);
@@ -214,19 +244,23 @@ struct BTraits<MOE_FMT_FP4_REF> {
 template <int FMT>
 struct BTraitsByte {
     static constexpr int BK = 64, NS = 2;
+    static constexpr int B_LDS_UNITS = 0, B_LOADS = 1;
     static constexpr bool DOUBLE_RAW = false;
     static constexpr int MT_MAX = 11;
     struct Raw {
         uint32_t r[2][8];
         float s8[2];  // fp8: scale of the 128x128 block of each sub-step
     };
+    __device__ static __forceinline__ void stage_load(u32x4_t*, const BCtx&, int) {}
+    __device__ static __forceinline__ void stage_store(u32x4_t*, const u32x4_t*, const BCtx&) {}
+    __device__ static __forceinline__ void load_scale(Raw&, const BCtx&, int, int) {}
     __device__ static __forceinline__ int a_chunk(int s, int q) { return 4 * s + q; }
     __device__ static __forceinline__ int col(const BCtx& c, int t) { return 64 * c.w + 4 * c.i + t; }
     __device__ static __forceinline__ void init(BCtx& c) {
         c.vw = 8 * c.q * c.N + col(c, 0);
         c.vs = 0;
     }
-    __device__ static __forceinline__ void load_sub(Raw& raw, const BCtx& c, int k0, int s) {
+    __device__ static __forceinline__ void load_sub(Raw& raw, const BCtx& c, int k0, int s, const u32x4_t*) {
 #pragma unroll
         for (int j = 0; j < 8; ++j) raw.r[s][j] = ldg_b32(c.rw, c.vw, (k0 + 32 * s + j) * c.N + c.n0);
         if (FMT == MOE_FMT_FP8_REF) {
@@ -277,6 +311,7 @@ struct BTraits<MOE_FMT_FP8_REF> : BTraitsByte<MOE_FMT_FP8_REF> {
 template <>
 struct BTraits<MOE_FMT_FP4_B32> {
     static constexpr int BK = 128, NS = 4;
+    static constexpr int B_LDS_UNITS = 0, B_LOADS = 1;
     // One 16-byte load per t serves all 4 sub-steps, so the registers cannot be reloaded
     // sub-step by sub-step: a whole step is loaded into a second register set (load_sub
     // ignores its sub-step argument and is called once per step).
@@ -286,13 +321,16 @@ struct BTraits<MOE_FMT_FP4_B32> {
         u32x4_t r[4];
         float sc[4];
     };
+    __device__ static __forceinline__ void stage_load(u32x4_t*, const BCtx&, int) {}
+    __device__ static __forceinline__ void stage_store(u32x4_t*, const u32x4_t*, const BCtx&) {}
+    __device__ static __forceinline__ void load_scale(Raw&, const BCtx&, int, int) {}
     __device__ static __forceinline__ int a_chunk(int s, int q) { return 4 * q + s; }
     __device__ static __forceinline__ int col(const BCtx& c, int t) { return 64 * c.w + 16 * t + c.i; }
     __device__ static __forceinline__ void init(BCtx& c) {
         c.vw = (64 * c.w + c.i) * (c.K >> 1) + 16 * c.q;
         c.vs = ((64 * c.w + c.i) * (c.K >> 5) + c.q) * 2;
     }
-    __device__ static __forceinline__ void load_sub(Raw& raw, const BCtx& c, int k0, int) {
+    __device__ static __forceinline__ void load_sub(Raw& raw, const BCtx& c, int k0, int, const u32x4_t*) {
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
             raw.r[t] = ldg_b128(c.rw, c.vw, (c.n0 + 16 * t) * (c.K >> 1) + (k0 >> 1));
@@ -319,18 +357,22 @@ struct BTraits<MOE_FMT_FP4_B32> {
 template <>
 struct BTraits<MOE_FMT_BF16> {
     static constexpr int BK = 64, NS = 2;
+    static constexpr int B_LDS_UNITS = 0, B_LOADS = 1;
     static constexpr bool DOUBLE_RAW = false;
     static constexpr int MT_MAX = 11;
     struct Raw {
         u32x4_t r[4][2];
     };
+    __device__ static __forceinline__ void stage_load(u32x4_t*, const BCtx&, int) {}
+    __device__ static __forceinline__ void stage_store(u32x4_t*, const u32x4_t*, const BCtx&) {}
+    __device__ static __forceinline__ void load_scale(Raw&, const BCtx&, int, int) {}
     __device__ static __forceinline__ int a_chunk(int s, int q) { return 2 * q + s; }
     __device__ static __forceinline__ int col(const BCtx& c, int t) { return 64 * c.w + 16 * t + c.i; }
     __device__ static __forceinline__ void init(BCtx& c) {
         c.vw = (64 * c.w + c.i) * c.K * 2 + 32 * c.q;
         c.vs = 0;
     }
-    __device__ static __forceinline__ void load_sub(Raw& raw, const BCtx& c, int k0, int s) {
+    __device__ static __forceinline__ void load_sub(Raw& raw, const BCtx& c, int k0, int s, const u32x4_t*) {
 #pragma unroll
         for (int t = 0; t < 4; ++t) raw.r[t][s] = ldg_b128(c.rw, c.vw, ((c.n0 + 16 * t) * c.K + k0) * 2 + 16 * s);
     }
@@ -355,8 +397,8 @@ __device__ __forceinline__ int a_lds_unit(int row, int c) {
 }
 
 template <int FMT, int MT>
-__device__ __forceinline__ void gemm_tile(const GemmParams& P, u32x4_t* lds_a, int g, int64_t row0, int rows,
-                                          int n0) {
+__device__ __forceinline__ void gemm_tile(const GemmParams& P, u32x4_t* lds_a, u32x4_t* lds_b, int g, int64_t row0,
+                                          int rows, int n0) {
     using T = BTraits<FMT>;
     constexpr int BK = T::BK, NS = T::NS;
     constexpr int CPR = BK / 8;               // 16-byte chunks per tile row
@@ -443,9 +485,11 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& P, u32x4_t* lds_a, i
     // instruction placed by hand (sched_barrier after each MFMA slot):
     //  * weights: while the MFMAs of sub-step f run, the fragments of sub-step f+1 are
     //    decoded, one unit (two elements of one column) at a time between MFMAs; as soon as
-    //    a sub-step's packed registers have been decoded they are reloaded with the same
-    //    sub-step of the next k step (formats whose loads span a whole step keep a second
-    //    register set), so every weight load has one full k step to land;
+    //    a sub-step's packed registers have been decoded they are refilled with the same
+    //    sub-step of the next k step -- straight from global memory a full step ahead
+    //    (formats whose loads span a whole step keep a second register set), or, for the
+    //    staged formats, from the LDS copy of the next step's packed tile, which itself was
+    //    fetched with wide loads one step earlier and written before the last barrier;
     //  * x: fragments come from LDS through a ring of 4 register sets, read RING
     //    fragments ahead of their MFMAs; the x tile of step kt+1 travels through registers
     //    into the other LDS buffer.
@@ -455,25 +499,50 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& P, u32x4_t* lds_a, i
     constexpr int SLOTS = 4 * MT;   // MFMAs per sub-step
     constexpr int UNITS = 17;       // prep + 16 decode units per sub-step
 
+    constexpr bool STAGED = T::B_LDS_UNITS > 0;   // packed weights travel through LDS like the x tile
+    u32x4_t breg[T::B_LOADS];
+    auto btile = [&](int kt) { return lds_b + (kt & 1) * T::B_LDS_UNITS; };
+
     __syncthreads();  // previous tile's readers are done with both buffers
     load_a(0);
-#pragma unroll
-    for (int s = 0; s < (T::DOUBLE_RAW ? 1 : NS); ++s) T::load_sub(raw, c, 0, s);
+    if (STAGED) {
+        T::stage_load(breg, c, 0);
+        T::stage_store(btile(0), breg, c);
+        T::stage_load(breg, c, BK);
+    }
     store_a(0);
+    if (STAGED) {
+        __syncthreads();
+        T::stage_store(btile(1), breg, c);
+    }
+#pragma unroll
+    for (int s = 0; s < (T::DOUBLE_RAW ? 1 : NS); ++s) {
+        T::load_sub(raw, c, 0, s, btile(0));
+        T::load_scale(raw, c, 0, s);
+    }
     u32x4_t bf[2][4];
     dq.prep(raw, c, 0);
 #pragma unroll
     for (int p = 0; p < 4; ++p)
 #pragma unroll
         for (int t = 0; t < 4; ++t) dq.unit(raw, c, 0, p, t, bf[0]);
-    if (T::DOUBLE_RAW)
-        T::load_sub(raw_next, c, BK, 0);
-    else
-        T::load_sub(raw, c, BK, 0);
     __syncthreads();
+    // raw[0] <- sub-step 0 of step 1 (direct formats: loaded a full step ahead; staged: read at the
+    // top of each step from the tile written during the previous one)
+    if (!STAGED) {
+        if (T::DOUBLE_RAW)
+            T::load_sub(raw_next, c, BK, 0, nullptr);
+        else
+            T::load_sub(raw, c, BK, 0, nullptr);
+    }
+    T::load_scale(raw, c, BK, 0);
 
     for (int kt = 0; kt < nk; ++kt) {
         load_a(kt + 1);
+        if (STAGED) {
+            T::stage_load(breg, c, (kt + 2) * BK);
+            T::load_sub(raw, c, (kt + 1) * BK, 0, btile(kt + 1));
+        }
         const u32x4_t* la = lds_a + (kt & 1) * ABUF;
         u32x4_t afr[4];
         auto read_a = [&](int f) {
@@ -503,16 +572,20 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& P, u32x4_t* lds_a, i
                 }
                 if (slot == ((UNITS - 1) * SLOTS) / UNITS) {
                     // everything of sub-step sn has been decoded: refill its registers
-                    if (T::DOUBLE_RAW) {
-                        if (sn == 0) T::load_sub(raw_next, c, (kt + 2) * BK, 0);
+                    T::load_scale(raw, c, (kt + (sn == 0 ? 2 : 1)) * BK, sn);
+                    if (STAGED) {
+                        if (sn != 0) T::load_sub(raw, c, (kt + 1) * BK, sn, btile(kt + 1));
+                    } else if (T::DOUBLE_RAW) {
+                        if (sn == 0) T::load_sub(raw_next, c, (kt + 2) * BK, 0, nullptr);
                     } else {
-                        T::load_sub(raw, c, (kt + (sn == 0 ? 2 : 1)) * BK, sn);
+                        T::load_sub(raw, c, (kt + (sn == 0 ? 2 : 1)) * BK, sn, nullptr);
                     }
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
         store_a((kt + 1) & 1);
+        if (STAGED) T::stage_store(btile(kt + 2), breg, c);
         __syncthreads();
     }
     // the accumulators were last written by MFMAs the compiler cannot see: wait out their latency
@@ -561,7 +634,8 @@ __global__ __launch_bounds__(GM_THREADS) void grouped_gemm_kernel(GemmParams P) 
     extern __shared__ u32x4_t smem[];
     constexpr int BK = BTraits<FMT>::BK;
     u32x4_t* lds_a = smem;                                                         // 2 buffers
-    int* prefix = reinterpret_cast<int*>(smem + 2 * 16 * GM_MT_MAX * (BK / 8));    // [G + 1]
+    u32x4_t* lds_b = smem + 2 * 16 * GM_MT_MAX * (BK / 8);                         // 2 packed weight tiles
+    int* prefix = reinterpret_cast<int*>(lds_b + 2 * BTraits<FMT>::B_LDS_UNITS);   // [G + 1]
     const int tid = threadIdx.x;
     const int ntile_n = P.N / GM_BN;
 
@@ -629,21 +703,21 @@ __global__ __launch_bounds__(GM_THREADS) void grouped_gemm_kernel(GemmParams P) 
         const int64_t row0 = (((int64_t)rhi << 32) | (uint32_t)rlo) + rbeg;
         const int n0 = nt * GM_BN;
         switch (mt) {
-            case 1: gemm_tile<FMT, 1>(P, lds_a, g, row0, rows, n0); break;
-            case 2: gemm_tile<FMT, 2>(P, lds_a, g, row0, rows, n0); break;
-            case 3: gemm_tile<FMT, 3>(P, lds_a, g, row0, rows, n0); break;
-            case 4: gemm_tile<FMT, 4>(P, lds_a, g, row0, rows, n0); break;
-            case 5: gemm_tile<FMT, 5>(P, lds_a, g, row0, rows, n0); break;
-            case 6: gemm_tile<FMT, 6>(P, lds_a, g, row0, rows, n0); break;
-            case 7: gemm_tile<FMT, 7>(P, lds_a, g, row0, rows, n0); break;
-            case 8: gemm_tile<FMT, 8>(P, lds_a, g, row0, rows, n0); break;
-            case 9: gemm_tile<FMT, 9>(P, lds_a, g, row0, rows, n0); break;
-            case 10: gemm_tile<FMT, 10>(P, lds_a, g, row0, rows, n0); break;
+            case 1: gemm_tile<FMT, 1>(P, lds_a, lds_b, g, row0, rows, n0); break;
+            case 2: gemm_tile<FMT, 2>(P, lds_a, lds_b, g, row0, rows, n0); break;
+            case 3: gemm_tile<FMT, 3>(P, lds_a, lds_b, g, row0, rows, n0); break;
+            case 4: gemm_tile<FMT, 4>(P, lds_a, lds_b, g, row0, rows, n0); break;
+            case 5: gemm_tile<FMT, 5>(P, lds_a, lds_b, g, row0, rows, n0); break;
+            case 6: gemm_tile<FMT, 6>(P, lds_a, lds_b, g, row0, rows, n0); break;
+            case 7: gemm_tile<FMT, 7>(P, lds_a, lds_b, g, row0, rows, n0); break;
+            case 8: gemm_tile<FMT, 8>(P, lds_a, lds_b, g, row0, rows, n0); break;
+            case 9: gemm_tile<FMT, 9>(P, lds_a, lds_b, g, row0, rows, n0); break;
+            case 10: gemm_tile<FMT, 10>(P, lds_a, lds_b, g, row0, rows, n0); break;
             case 11:
-                if constexpr (BTraits<FMT>::MT_MAX >= 11) gemm_tile<FMT, 11>(P, lds_a, g, row0, rows, n0);
+                if constexpr (BTraits<FMT>::MT_MAX >= 11) gemm_tile<FMT, 11>(P, lds_a, lds_b, g, row0, rows, n0);
                 break;
             default:
-                if constexpr (BTraits<FMT>::MT_MAX >= 12) gemm_tile<FMT, 12>(P, lds_a, g, row0, rows, n0);
+                if constexpr (BTraits<FMT>::MT_MAX >= 12) gemm_tile<FMT, 12>(P, lds_a, lds_b, g, row0, rows, n0);
                 break;
         }
     }
@@ -661,7 +735,8 @@ static int launch_gemm_fmt(const moe_grouped_args* a, hipStream_t stream) {
     P.y = static_cast<uint16_t*>(a->y);
     P.M = a->M; P.K = (int)a->K; P.N = (int)a->N; P.G = (int)a->G; P.scale_rows = (int)a->scale_rows;
 
-    const size_t lds = (size_t)2 * 16 * GM_MT_MAX * (BK / 8) * 16 + ((size_t)a->G + 1) * sizeof(int);
+    const size_t lds = (size_t)2 * 16 * GM_MT_MAX * (BK / 8) * 16 + (size_t)2 * BTraits<FMT>::B_LDS_UNITS * 16 +
+                       ((size_t)a->G + 1) * sizeof(int);
     if (lds > 160 * 1024 - 2048) return MOE_ERR_TOO_LARGE;
     static bool attr_set = false;  // idempotent; a race only repeats the same call
     if (!attr_set) {
