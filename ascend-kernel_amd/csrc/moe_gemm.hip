@@ -110,7 +110,7 @@ template <>
 struct BTraits<MOE_FMT_INT4> {
     static constexpr int BK = 64, NS = 2;
     static constexpr bool DOUBLE_RAW = false;
-    static constexpr int MT_MAX = 11;  // 176 rows: the largest tile that keeps every value in registers
+    static constexpr int MT_MAX = 10;  // 160 rows: the largest tile that keeps every value in registers
     static constexpr int B_LDS_UNITS = 64 * 8;  // 16-byte units of one packed tile in LDS (0: no LDS staging)
     static constexpr int B_LOADS = 2;           // 16-byte global loads per thread per k step
     struct Raw {
@@ -468,17 +468,17 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& P, u32x4_t* lds_a, u
     typename T::Raw raw, raw_next;
     const int nk = P.K / BK;
 
+    // Every pass is done by all threads: rows past the tile read as zeros (they lie beyond the
+    // buffer resource) and land in LDS rows that exist (the buffers hold 16 * GM_MT_MAX rows)
+    // but are never read.  No divergent branch, so the loop body stays one scheduling region.
+    static_assert(PASSES * RPP <= 16 * GM_MT_MAX, "x tile passes overrun the LDS buffer");
     auto load_a = [&](int kt) {
 #pragma unroll
-        for (int p = 0; p < PASSES; ++p)
-            if (PASSES * RPP == 16 * MT || ar + RPP * p < 16 * MT)
-                areg[p] = ldg_b128(rx, vx, (p * RPP * P.K + kt * BK) * 2);
+        for (int p = 0; p < PASSES; ++p) areg[p] = ldg_b128(rx, vx, (p * RPP * P.K + kt * BK) * 2);
     };
     auto store_a = [&](int buf) {
 #pragma unroll
-        for (int p = 0; p < PASSES; ++p)
-            if (PASSES * RPP == 16 * MT || ar + RPP * p < 16 * MT)
-                lds_a[buf * ABUF + a_lds_unit<BK>(ar + RPP * p, ac)] = areg[p];
+        for (int p = 0; p < PASSES; ++p) lds_a[buf * ABUF + a_lds_unit<BK>(ar + RPP * p, ac)] = areg[p];
     };
 
     // Software pipeline, one barrier per k step (BK = NS sub-steps of 32 k), every
@@ -500,7 +500,7 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& P, u32x4_t* lds_a, u
     constexpr int UNITS = 17;       // prep + 16 decode units per sub-step
 
     constexpr bool STAGED = T::B_LDS_UNITS > 0;   // packed weights travel through LDS like the x tile
-    u32x4_t breg[T::B_LOADS];
+    u32x4_t breg[T::B_LOADS], breg2[T::B_LOADS];
     auto btile = [&](int kt) { return lds_b + (kt & 1) * T::B_LDS_UNITS; };
 
     __syncthreads();  // previous tile's readers are done with both buffers
@@ -514,6 +514,7 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& P, u32x4_t* lds_a, u
     if (STAGED) {
         __syncthreads();
         T::stage_store(btile(1), breg, c);
+        T::stage_load(breg, c, 2 * BK);
     }
 #pragma unroll
     for (int s = 0; s < (T::DOUBLE_RAW ? 1 : NS); ++s) {
@@ -537,10 +538,13 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& P, u32x4_t* lds_a, u
     }
     T::load_scale(raw, c, BK, 0);
 
-    for (int kt = 0; kt < nk; ++kt) {
+    // One k step.  Staged formats fetch their packed tile two steps before it is written to
+    // LDS (three before it is used): `bload` receives tile kt+3, `bstore` (loaded during the
+    // previous step) is written as tile kt+2 at the end of this step.
+    auto step = [&](int kt, u32x4_t* bload, const u32x4_t* bstore) {
         load_a(kt + 1);
         if (STAGED) {
-            T::stage_load(breg, c, (kt + 2) * BK);
+            T::stage_load(bload, c, (kt + 3) * BK);
             T::load_sub(raw, c, (kt + 1) * BK, 0, btile(kt + 1));
         }
         const u32x4_t* la = lds_a + (kt & 1) * ABUF;
@@ -585,8 +589,16 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& P, u32x4_t* lds_a, u
             }
         }
         store_a((kt + 1) & 1);
-        if (STAGED) T::stage_store(btile(kt + 2), breg, c);
+        if (STAGED) T::stage_store(btile(kt + 2), bstore, c);
         __syncthreads();
+    };
+    if (STAGED) {
+        for (int kt = 0; kt < nk; kt += 2) {
+            step(kt, breg2, breg);
+            if (kt + 1 < nk) step(kt + 1, breg, breg2);
+        }
+    } else {
+        for (int kt = 0; kt < nk; ++kt) step(kt, breg, breg);
     }
     // the accumulators were last written by MFMAs the compiler cannot see: wait out their latency
     asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
