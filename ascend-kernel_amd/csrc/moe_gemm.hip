@@ -67,6 +67,17 @@ __device__ __forceinline__ void mfma_16x16x32(f32x4_t& acc, const u32x4_t& a, co
     asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
 }
 
+// Ties a value to the chain of volatile asm statements (the MFMAs): whatever is computed
+// from the returned value is emitted after every earlier volatile asm, whatever produced the
+// argument before every later one.  Emits no instruction.  Used to pin each decode unit
+// between two MFMAs; sched_barrier alone only constrains the machine scheduler, not the
+// instruction order chosen at selection time.
+template <typename V>
+__device__ __forceinline__ V pinned(V v) {
+    asm volatile("" : "+v"(v));
+    return v;
+}
+
 // Per-lane view of one tile for the weight loaders.
 struct BCtx {
     rsrc_t rw, rs;       // weight / scale slab of the expert
@@ -164,20 +175,20 @@ struct BTraits<MOE_FMT_INT4> {
         uint32_t al, ah, bl, bh; // masked halves of the two k rows of the current pair
         __device__ __forceinline__ void init_tile(const BCtx&) {}
         __device__ __forceinline__ void prep(const Raw& raw, const BCtx&, int s) {
-            const float s0 = bf16_lo(raw.sc[s][0]), s1 = bf16_hi(raw.sc[s][0]);
-            const float s2 = bf16_lo(raw.sc[s][1]), s3 = bf16_hi(raw.sc[s][1]);
+            const uint32_t sa = pinned(raw.sc[s][0]), sb = pinned(raw.sc[s][1]);
+            const float s0 = bf16_lo(sa), s1 = bf16_hi(sa), s2 = bf16_lo(sb), s3 = bf16_hi(sb);
             m[0] = s0; m[1] = s1 * 0.0625f; m[2] = s2; m[3] = s3 * 0.0625f;  // odd nibbles arrive times 16
             z[0] = -8.f * s0; z[1] = -8.f * s1; z[2] = -8.f * s2; z[3] = -8.f * s3;
         }
         __device__ __forceinline__ void unit(const Raw& raw, const BCtx& c, int s, int p, int t, u32x4_t out[4]) {
             if (t == 0) {
                 const int sh = 16 * (c.w & 1);
-                const uint32_t a = raw.r[s][2 * p] >> sh, b = raw.r[s][2 * p + 1] >> sh;
+                const uint32_t a = pinned(raw.r[s][2 * p]) >> sh, b = raw.r[s][2 * p + 1] >> sh;
                 al = a & c.mlo; ah = a & c.mhi; bl = b & c.mlo; bh = b & c.mhi;
             }
-            const uint32_t ua = (t & 1) ? ah : al, ub = (t & 1) ? bh : bl;
+            const uint32_t ua = pinned((t & 1) ? ah : al), ub = (t & 1) ? bh : bl;
             const float fa = (t & 2) ? ubyte1(ua) : ubyte0(ua), fb = (t & 2) ? ubyte1(ub) : ubyte0(ub);
-            out[t][p] = pack_bf16_rne(fmaf(fa, m[t], z[t]), fmaf(fb, m[t], z[t]));
+            out[t][p] = pinned(pack_bf16_rne(fmaf(fa, m[t], z[t]), fmaf(fb, m[t], z[t])));
         }
     };
 };
@@ -230,11 +241,11 @@ struct BTraits<MOE_FMT_FP4_REF> {
             if ((t & 1) == 0) {
                 const int sh = 16 * (c.w & 1);
                 const int j = 2 * p;
-                const uint32_t a = raw.r[s][j >> 2][j & 3] >> sh, b = raw.r[s][(j + 1) >> 2][(j + 1) & 3] >> sh;
+                const uint32_t a = pinned(raw.r[s][j >> 2][j & 3]) >> sh, b = raw.r[s][(j + 1) >> 2][(j + 1) & 3] >> sh;
                 if (t == 0) { va = e2m1_pair_to_f32<0>(a); vb = e2m1_pair_to_f32<0>(b); }
                 else        { va = e2m1_pair_to_f32<1>(a); vb = e2m1_pair_to_f32<1>(b); }
             }
-            out[t][p] = pack_bf16_rne(va[t & 1] * sc[t], vb[t & 1] * sc[t]);
+            out[t][p] = pinned(pack_bf16_rne(pinned(va[t & 1]) * sc[t], vb[t & 1] * sc[t]));
         }
     };
 };
@@ -283,10 +294,10 @@ struct BTraits<MOE_FMT_INT8> : BTraitsByte<MOE_FMT_INT8> {
         }
         __device__ __forceinline__ void prep(const Raw&, const BCtx&, int) {}
         __device__ __forceinline__ void unit(const Raw& raw, const BCtx&, int s, int p, int t, u32x4_t out[4]) {
-            const uint32_t a = raw.r[s][2 * p], b = raw.r[s][2 * p + 1];
+            const uint32_t a = pinned(raw.r[s][2 * p]), b = raw.r[s][2 * p + 1];
             const float qa = (float)(int)(int8_t)(a >> (8 * t)), qb = (float)(int)(int8_t)(b >> (8 * t));
             // (q + offset) * scale as two rounded fp32 operations
-            out[t][p] = pack_bf16_rne(__fmul_rn(__fadd_rn(qa, of[t]), sc[t]), __fmul_rn(__fadd_rn(qb, of[t]), sc[t]));
+            out[t][p] = pinned(pack_bf16_rne(__fmul_rn(__fadd_rn(qa, of[t]), sc[t]), __fmul_rn(__fadd_rn(qb, of[t]), sc[t])));
         }
     };
 };
@@ -297,9 +308,9 @@ struct BTraits<MOE_FMT_FP8_REF> : BTraitsByte<MOE_FMT_FP8_REF> {
         __device__ __forceinline__ void init_tile(const BCtx&) {}
         __device__ __forceinline__ void prep(const Raw&, const BCtx&, int) {}
         __device__ __forceinline__ void unit(const Raw& raw, const BCtx&, int s, int p, int t, u32x4_t out[4]) {
-            const uint32_t a = raw.r[s][2 * p], b = raw.r[s][2 * p + 1];
-            out[t][p] = pack_bf16_rne(e4m3_ref_to_f32((a >> (8 * t)) & 0xffu) * raw.s8[s],
-                                      e4m3_ref_to_f32((b >> (8 * t)) & 0xffu) * raw.s8[s]);
+            const uint32_t a = pinned(raw.r[s][2 * p]), b = raw.r[s][2 * p + 1];
+            out[t][p] = pinned(pack_bf16_rne(e4m3_ref_to_f32((a >> (8 * t)) & 0xffu) * raw.s8[s],
+                                             e4m3_ref_to_f32((b >> (8 * t)) & 0xffu) * raw.s8[s]));
         }
     };
 };
@@ -342,11 +353,11 @@ struct BTraits<MOE_FMT_FP4_B32> {
         __device__ __forceinline__ void init_tile(const BCtx&) {}
         __device__ __forceinline__ void prep(const Raw&, const BCtx&, int) {}
         __device__ __forceinline__ void unit(const Raw& raw, const BCtx&, int s, int p, int t, u32x4_t out[4]) {
-            const uint32_t wd = raw.r[t][s];
-            out[t][p] = p == 0   ? e2m1_pair_scaled_bf16<0>(wd, raw.sc[t])
-                        : p == 1 ? e2m1_pair_scaled_bf16<1>(wd, raw.sc[t])
-                        : p == 2 ? e2m1_pair_scaled_bf16<2>(wd, raw.sc[t])
-                                 : e2m1_pair_scaled_bf16<3>(wd, raw.sc[t]);
+            const uint32_t wd = pinned(raw.r[t][s]);
+            out[t][p] = pinned(p == 0   ? e2m1_pair_scaled_bf16<0>(wd, raw.sc[t])
+                               : p == 1 ? e2m1_pair_scaled_bf16<1>(wd, raw.sc[t])
+                               : p == 2 ? e2m1_pair_scaled_bf16<2>(wd, raw.sc[t])
+                                        : e2m1_pair_scaled_bf16<3>(wd, raw.sc[t]));
         }
     };
 };
@@ -380,7 +391,7 @@ struct BTraits<MOE_FMT_BF16> {
         __device__ __forceinline__ void init_tile(const BCtx&) {}
         __device__ __forceinline__ void prep(const Raw&, const BCtx&, int) {}
         __device__ __forceinline__ void unit(const Raw& raw, const BCtx&, int s, int p, int t, u32x4_t out[4]) {
-            out[t][p] = raw.r[t][s][p];
+            out[t][p] = pinned(raw.r[t][s][p]);
         }
     };
 };
