@@ -552,12 +552,12 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& P, u32x4_t* lds_a, u
     // One k step.  Staged formats fetch their packed tile two steps before it is written to
     // LDS (three before it is used): `bload` receives tile kt+3, `bstore` (loaded during the
     // previous step) is written as tile kt+2 at the end of this step.
+    // Global loads of the next tiles are issued one per MFMA slot at the start of the first
+    // sub-step, the LDS writes one per slot at the end of the last one, so that neither sits
+    // between the barrier and the first MFMA or between the last MFMA and the barrier.
+    constexpr int NW = PASSES + (STAGED ? 1 : 0);   // write slots: one per x pass, one for the packed tile
+    static_assert(NW + 1 <= SLOTS, "not enough MFMA slots to spread the tile transfers over");
     auto step = [&](int kt, u32x4_t* bload, const u32x4_t* bstore) {
-        load_a(kt + 1);
-        if (STAGED) {
-            T::stage_load(bload, c, (kt + 3) * BK);
-            T::load_sub(raw, c, (kt + 1) * BK, 0, btile(kt + 1));
-        }
         const u32x4_t* la = lds_a + (kt & 1) * ABUF;
         u32x4_t afr[4];
         auto read_a = [&](int f) {
@@ -577,6 +577,16 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& P, u32x4_t* lds_a, u
                 const int mt = slot >> 2, t = slot & 3, f = s * MT + mt;
                 if (t == 0 && f + RING < F) read_a(f + RING);
                 mfma_16x16x32(acc[mt][t], afr[f & 3], bcur[t]);
+                if (s == 0) {
+                    // fetch: x tile of step kt+1, packed tile of step kt+3, then this lane's
+                    // dwords of sub-step 0 of step kt+1 from the LDS tile written last step
+                    if (slot < PASSES)
+                        areg[slot] = ldg_b128(rx, vx, (slot * RPP * P.K + (kt + 1) * BK) * 2);
+                    else if (STAGED && slot == PASSES)
+                        T::stage_load(bload, c, (kt + 3) * BK);
+                    else if (STAGED && slot == PASSES + 1)
+                        T::load_sub(raw, c, (kt + 1) * BK, 0, btile(kt + 1));
+                }
                 // decode units u with floor(u * SLOTS / UNITS) == slot
 #pragma unroll
                 for (int u = (slot * UNITS + SLOTS - 1) / SLOTS; u < ((slot + 1) * UNITS + SLOTS - 1) / SLOTS; ++u) {
@@ -596,11 +606,16 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& P, u32x4_t* lds_a, u
                         T::load_sub(raw, c, (kt + (sn == 0 ? 2 : 1)) * BK, sn, nullptr);
                     }
                 }
+                if (s == NS - 1 && slot >= SLOTS - NW) {
+                    const int wi = slot - (SLOTS - NW);
+                    if (wi < PASSES)
+                        lds_a[((kt + 1) & 1) * ABUF + a_lds_unit<BK>(ar + RPP * wi, ac)] = areg[wi];
+                    else if (wi == PASSES)
+                        T::stage_store(btile(kt + 2), bstore, c);
+                }
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
-        store_a((kt + 1) & 1);
-        if (STAGED) T::stage_store(btile(kt + 2), bstore, c);
         __syncthreads();
     };
     if (STAGED) {
