@@ -196,14 +196,14 @@ def run_extra(torch, mg, gen, iters, warmup):
 
 def cpu_baseline(torch, seed):
     """The CPU oracle on a bounded sample of the headline workload: the gate_up GEMM
-    (K=7168, N=4096, int4, group 128) for 4 experts' worth of rows."""
+    (K=7168, N=4096, int4, group 128) of 64 of the 256 experts (a quarter of the rows)."""
     import numpy as np
 
     import oracle
 
     rng = np.random.default_rng(seed)
-    G, K, N = 4, 7168, 4096
-    counts = rng.multinomial(512, np.full(G, 1.0 / G))
+    G, K, N = 64, 7168, 4096
+    counts = rng.multinomial(128 * G, np.full(G, 1.0 / G))
     gl = np.cumsum(counts).astype(np.int64)
     M = int(gl[-1])
     x = torch.from_numpy(rng.standard_normal((M, K)).astype(np.float32)).to(torch.bfloat16)
@@ -229,6 +229,8 @@ def main():
     ap.add_argument("--workload", default="dsv3_int4_prefill")
     ap.add_argument("--no-extra", action="store_true", help="skip the other benchmark configurations")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU oracle baseline")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run one plain 1 GiB device copy (known traffic) to scale FETCH_SIZE / WRITE_SIZE")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.exit("bench.py: this build runs on one GPU only (--gpus 1); the ops shard by expert across GPUs, "
@@ -245,6 +247,13 @@ def main():
     torch.cuda.set_device(0)
     gen = torch.Generator().manual_seed(0)
     torch.manual_seed(0)
+
+    if args.copy_calibration:
+        src = torch.empty(1 << 30, dtype=torch.uint8, device="cuda").fill_(1)
+        dst = torch.empty_like(src)
+        dst.copy_(src)   # reads 1 GiB, writes 1 GiB
+        torch.cuda.synchronize()
+        del src, dst
 
     wl = build_dsv3_int4_prefill(torch, mg, gen)
     ops = wl["ops"]
