@@ -30,6 +30,11 @@ sys.path.insert(0, ROOT)
 
 PEAK_HBM_GBS = 8000.0        # MI355X HBM3E, 8 TB/s
 PEAK_BF16_TFLOPS = 2500.0    # MI355X dense bf16 MFMA, 2.5 PFLOP/s
+# HBM bytes per launch of the int4 grouped GEMM on this workload (mean of the gate_up and down
+# launches), from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs of this script scaled by the
+# --copy-calibration copy (summary under profiles/): 3.27 GB read + 0.369 GB written.
+# Algorithmic bytes: 3.21 GB + 0.369 GB.
+INT4_GEMM_HBM_BYTES_PER_LAUNCH = 3.64e9
 
 
 def routed_counts(torch, tokens, experts, topk, gen, max_rows=None):
@@ -275,7 +280,7 @@ def main():
     avg_launch = sum(t_each) / len(t_each)
     achieved = (step_flops / len(ops)) / avg_launch / 1e12
     roofline = dict(bound="mfma", achieved=achieved, peak=PEAK_BF16_TFLOPS, unit="TFLOP/s",
-                    frac=achieved / PEAK_BF16_TFLOPS, traffic=None,
+                    frac=achieved / PEAK_BF16_TFLOPS, traffic=INT4_GEMM_HBM_BYTES_PER_LAUNCH,
                     kernel="moe::grouped_gemm_kernel<int4>",
                     per_launch={n: dict(us=t * 1e6, TFLOPs=f / t / 1e12, frac=f / t / 1e12 / PEAK_BF16_TFLOPS)
                                 for n, t, f in zip(wl["names"], t_each, wl["flops"])})
