@@ -28,6 +28,8 @@ namespace moe {
 constexpr int GM_BN = 256;     // columns per workgroup
 constexpr int GM_MT_MAX = 12;  // 16-row blocks per tile the LDS buffers are sized for (192 rows)
 constexpr int GM_THREADS = 256;
+constexpr int GM_SKINNY_BLOCKS = 2;  // decode kernel: tiles of at most 32 rows ...
+constexpr int GM_SKINNY_WAVES = 3;   // ... and at least this many wavefronts per SIMD
 
 struct GemmParams {
     const uint16_t* x;
@@ -407,7 +409,7 @@ __device__ __forceinline__ int a_lds_unit(int row, int c) {
     return row * (BK / 8) + (c ^ (row & 7));
 }
 
-template <int FMT, int MT>
+template <int FMT, int MT, int CAPB>
 __device__ __forceinline__ void gemm_tile(const GemmParams& P, u32x4_t* lds_a, u32x4_t* lds_b, int g, int64_t row0,
                                           int rows, int n0) {
     using T = BTraits<FMT>;
@@ -415,7 +417,7 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& P, u32x4_t* lds_a, u
     constexpr int CPR = BK / 8;               // 16-byte chunks per tile row
     constexpr int RPP = GM_THREADS / CPR;     // rows loaded per pass
     constexpr int PASSES = (16 * MT + RPP - 1) / RPP;
-    constexpr int ABUF = 16 * GM_MT_MAX * CPR;  // units per buffer
+    constexpr int ABUF = 16 * CAPB * CPR;  // units per buffer (CAPB row blocks)
 
     const int tid = threadIdx.x, lane = tid & 63;
     BCtx c;
@@ -480,9 +482,9 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& P, u32x4_t* lds_a, u
     const int nk = P.K / BK;
 
     // Every pass is done by all threads: rows past the tile read as zeros (they lie beyond the
-    // buffer resource) and land in LDS rows that exist (the buffers hold 16 * GM_MT_MAX rows)
+    // buffer resource) and land in LDS rows that exist (the buffers hold 16 * CAPB rows)
     // but are never read.  No divergent branch, so the loop body stays one scheduling region.
-    static_assert(PASSES * RPP <= 16 * GM_MT_MAX, "x tile passes overrun the LDS buffer");
+    static_assert(PASSES * RPP <= 16 * CAPB, "x tile passes overrun the LDS buffer");
     auto load_a = [&](int kt) {
 #pragma unroll
         for (int p = 0; p < PASSES; ++p) areg[p] = ldg_b128(rx, vx, (p * RPP * P.K + kt * BK) * 2);
@@ -667,12 +669,17 @@ __device__ __forceinline__ void expert_chunks(int m, int& chunks, int& bpc) {
     bpc = chunks ? (nblk + chunks - 1) / chunks : 0;
 }
 
-template <int FMT>
-__global__ __launch_bounds__(GM_THREADS) void grouped_gemm_kernel(GemmParams P) {
+// CAPB = row blocks the LDS x buffers hold.  CAPB = GM_MT_MAX is the prefill kernel (tiles up
+// to the format's MT_MAX blocks, one workgroup per CU).  CAPB = GM_SKINNY_BLOCKS is the decode
+// kernel: tiles of at most 32 rows, a fraction of the registers and LDS, several workgroups
+// per CU to keep enough weight bytes in flight when the op is HBM bound.
+template <int FMT, int CAPB>
+__global__ __launch_bounds__(GM_THREADS, CAPB == GM_MT_MAX ? 1 : GM_SKINNY_WAVES) void grouped_gemm_kernel(GemmParams P) {
     extern __shared__ u32x4_t smem[];
     constexpr int BK = BTraits<FMT>::BK;
+    constexpr int MTM = CAPB < BTraits<FMT>::MT_MAX ? CAPB : BTraits<FMT>::MT_MAX;   // row blocks per tile
     u32x4_t* lds_a = smem;                                                         // 2 buffers
-    u32x4_t* lds_b = smem + 2 * 16 * GM_MT_MAX * (BK / 8);                         // 2 packed weight tiles
+    u32x4_t* lds_b = smem + 2 * 16 * CAPB * (BK / 8);                              // 2 packed weight tiles
     int* prefix = reinterpret_cast<int*>(lds_b + 2 * BTraits<FMT>::B_LDS_UNITS);   // [G + 1]
     const int tid = threadIdx.x;
     const int ntile_n = P.N / GM_BN;
@@ -687,7 +694,7 @@ __global__ __launch_bounds__(GM_THREADS) void grouped_gemm_kernel(GemmParams P) 
             int64_t s = g ? P.gl[g - 1] : 0, e = P.gl[g];
             s = max((int64_t)0, s); e = min(e, P.M);
             int chunks, bpc;
-            expert_chunks<BTraits<FMT>::MT_MAX>(e > s ? (int)(e - s) : 0, chunks, bpc);
+            expert_chunks<MTM>(e > s ? (int)(e - s) : 0, chunks, bpc);
             sum += chunks * ntile_n;
         }
         part[tid] = sum;
@@ -703,7 +710,7 @@ __global__ __launch_bounds__(GM_THREADS) void grouped_gemm_kernel(GemmParams P) 
             int64_t s = g ? P.gl[g - 1] : 0, e = P.gl[g];
             s = max((int64_t)0, s); e = min(e, P.M);
             int chunks, bpc;
-            expert_chunks<BTraits<FMT>::MT_MAX>(e > s ? (int)(e - s) : 0, chunks, bpc);
+            expert_chunks<MTM>(e > s ? (int)(e - s) : 0, chunks, bpc);
             prefix[g] = run;
             run += chunks * ntile_n;
         }
@@ -730,7 +737,7 @@ __global__ __launch_bounds__(GM_THREADS) void grouped_gemm_kernel(GemmParams P) 
         const int64_t gbeg = g ? max((int64_t)0, P.gl[g - 1]) : 0, gend = min(P.gl[g], P.M);
         const int m = __builtin_amdgcn_readfirstlane((int)(gend - gbeg));
         int chunks, bpc;
-        expert_chunks<BTraits<FMT>::MT_MAX>(m, chunks, bpc);
+        expert_chunks<MTM>(m, chunks, bpc);
         const int local = __builtin_amdgcn_readfirstlane(T - prefix[g]);
         const int chunk = local / ntile_n, nt = local % ntile_n;
         const int rbeg = chunk * bpc * 16;
@@ -741,29 +748,79 @@ __global__ __launch_bounds__(GM_THREADS) void grouped_gemm_kernel(GemmParams P) 
         const int64_t row0 = (((int64_t)rhi << 32) | (uint32_t)rlo) + rbeg;
         const int n0 = nt * GM_BN;
         switch (mt) {
-            case 1: gemm_tile<FMT, 1>(P, lds_a, lds_b, g, row0, rows, n0); break;
-            case 2: gemm_tile<FMT, 2>(P, lds_a, lds_b, g, row0, rows, n0); break;
-            case 3: gemm_tile<FMT, 3>(P, lds_a, lds_b, g, row0, rows, n0); break;
-            case 4: gemm_tile<FMT, 4>(P, lds_a, lds_b, g, row0, rows, n0); break;
-            case 5: gemm_tile<FMT, 5>(P, lds_a, lds_b, g, row0, rows, n0); break;
-            case 6: gemm_tile<FMT, 6>(P, lds_a, lds_b, g, row0, rows, n0); break;
-            case 7: gemm_tile<FMT, 7>(P, lds_a, lds_b, g, row0, rows, n0); break;
-            case 8: gemm_tile<FMT, 8>(P, lds_a, lds_b, g, row0, rows, n0); break;
-            case 9: gemm_tile<FMT, 9>(P, lds_a, lds_b, g, row0, rows, n0); break;
-            case 10: gemm_tile<FMT, 10>(P, lds_a, lds_b, g, row0, rows, n0); break;
+            case 1:
+                if constexpr (MTM >= 1) gemm_tile<FMT, 1, CAPB>(P, lds_a, lds_b, g, row0, rows, n0);
+                break;
+            case 2:
+                if constexpr (MTM >= 2) gemm_tile<FMT, 2, CAPB>(P, lds_a, lds_b, g, row0, rows, n0);
+                break;
+            case 3:
+                if constexpr (MTM >= 3) gemm_tile<FMT, 3, CAPB>(P, lds_a, lds_b, g, row0, rows, n0);
+                break;
+            case 4:
+                if constexpr (MTM >= 4) gemm_tile<FMT, 4, CAPB>(P, lds_a, lds_b, g, row0, rows, n0);
+                break;
+            case 5:
+                if constexpr (MTM >= 5) gemm_tile<FMT, 5, CAPB>(P, lds_a, lds_b, g, row0, rows, n0);
+                break;
+            case 6:
+                if constexpr (MTM >= 6) gemm_tile<FMT, 6, CAPB>(P, lds_a, lds_b, g, row0, rows, n0);
+                break;
+            case 7:
+                if constexpr (MTM >= 7) gemm_tile<FMT, 7, CAPB>(P, lds_a, lds_b, g, row0, rows, n0);
+                break;
+            case 8:
+                if constexpr (MTM >= 8) gemm_tile<FMT, 8, CAPB>(P, lds_a, lds_b, g, row0, rows, n0);
+                break;
+            case 9:
+                if constexpr (MTM >= 9) gemm_tile<FMT, 9, CAPB>(P, lds_a, lds_b, g, row0, rows, n0);
+                break;
+            case 10:
+                if constexpr (MTM >= 10) gemm_tile<FMT, 10, CAPB>(P, lds_a, lds_b, g, row0, rows, n0);
+                break;
             case 11:
-                if constexpr (BTraits<FMT>::MT_MAX >= 11) gemm_tile<FMT, 11>(P, lds_a, lds_b, g, row0, rows, n0);
+                if constexpr (MTM >= 11) gemm_tile<FMT, 11, CAPB>(P, lds_a, lds_b, g, row0, rows, n0);
                 break;
-            default:
-                if constexpr (BTraits<FMT>::MT_MAX >= 12) gemm_tile<FMT, 12>(P, lds_a, lds_b, g, row0, rows, n0);
+            case 12:
+                if constexpr (MTM >= 12) gemm_tile<FMT, 12, CAPB>(P, lds_a, lds_b, g, row0, rows, n0);
                 break;
+            default: break;
         }
     }
 }
 
+template <int FMT, int CAPB>
+static int launch_gemm_cap(const GemmParams& P, const moe_grouped_args* a, hipStream_t stream) {
+    constexpr int BK = BTraits<FMT>::BK;
+    constexpr int MTM = CAPB < BTraits<FMT>::MT_MAX ? CAPB : BTraits<FMT>::MT_MAX;
+    const size_t lds = (size_t)2 * 16 * CAPB * (BK / 8) * 16 + (size_t)2 * BTraits<FMT>::B_LDS_UNITS * 16 +
+                       ((size_t)a->G + 1) * sizeof(int);
+    if (lds > 160 * 1024 - 2048) return MOE_ERR_TOO_LARGE;
+    static bool attr_set = false;  // idempotent; a race only repeats the same call
+    if (!attr_set) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(&grouped_gemm_kernel<FMT, CAPB>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 2048) != hipSuccess)
+            return MOE_ERR_LAUNCH;
+        attr_set = true;
+    }
+    int dev = 0, cus = 256;
+    if (hipGetDevice(&dev) != hipSuccess) return MOE_ERR_NO_DEVICE;
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return MOE_ERR_NO_DEVICE;
+    // persistent grid: one workgroup per CU (prefill) or as many as fit (decode), but no more than
+    // an upper bound on the tile count that needs no look at group_list (every expert adds at most
+    // one partly filled chunk)
+    const int64_t per_cu = CAPB == GM_MT_MAX ? 1 : GM_SKINNY_WAVES;
+    const int64_t max_chunks = a->M / (16 * MTM) + a->G;
+    const int64_t max_tiles = max_chunks * (a->N / GM_BN);
+    const int64_t want = max_tiles < cus * per_cu ? max_tiles : cus * per_cu;
+    // a multiple of 8 so that the XCD-aware order covers every tile index
+    const int64_t grid = want > 0 ? (want + 7) / 8 * 8 : 8;
+    hipLaunchKernelGGL((grouped_gemm_kernel<FMT, CAPB>), dim3((unsigned)grid), dim3(GM_THREADS), lds, stream, P);
+    return hipGetLastError() == hipSuccess ? MOE_OK : MOE_ERR_LAUNCH;
+}
+
 template <int FMT>
 static int launch_gemm_fmt(const moe_grouped_args* a, hipStream_t stream) {
-    constexpr int BK = BTraits<FMT>::BK;
     GemmParams P;
     P.x = static_cast<const uint16_t*>(a->x);
     P.w = static_cast<const uint8_t*>(a->weight);
@@ -772,32 +829,20 @@ static int launch_gemm_fmt(const moe_grouped_args* a, hipStream_t stream) {
     P.gl = a->group_list;
     P.y = static_cast<uint16_t*>(a->y);
     P.M = a->M; P.K = (int)a->K; P.N = (int)a->N; P.G = (int)a->G; P.scale_rows = (int)a->scale_rows;
-
-    const size_t lds = (size_t)2 * 16 * GM_MT_MAX * (BK / 8) * 16 + (size_t)2 * BTraits<FMT>::B_LDS_UNITS * 16 +
-                       ((size_t)a->G + 1) * sizeof(int);
-    if (lds > 160 * 1024 - 2048) return MOE_ERR_TOO_LARGE;
-    static bool attr_set = false;  // idempotent; a race only repeats the same call
-    if (!attr_set) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void*>(&grouped_gemm_kernel<FMT>),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 2048) != hipSuccess)
-            return MOE_ERR_LAUNCH;
-        attr_set = true;
-    }
-    int dev = 0, cus = 256;
-    if (hipGetDevice(&dev) != hipSuccess) return MOE_ERR_NO_DEVICE;
-    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return MOE_ERR_NO_DEVICE;
-    // upper bound on the tile count without reading group_list: every expert adds at most
-    // one partly filled chunk
-    const int64_t max_chunks = a->M / (16 * BTraits<FMT>::MT_MAX) + a->G;
-    const int64_t max_tiles = max_chunks * (a->N / GM_BN);
-    // a multiple of 8 so that the XCD-aware order covers every tile index
-    const int64_t want = max_tiles < cus ? max_tiles : cus;
-    const int64_t grid = want > 0 ? (want + 7) / 8 * 8 : 8;
-    hipLaunchKernelGGL((grouped_gemm_kernel<FMT>), dim3((unsigned)grid), dim3(GM_THREADS), lds, stream, P);
-    return hipGetLastError() == hipSuccess ? MOE_OK : MOE_ERR_LAUNCH;
+    // Decode-like batches (on average at most 24 rows per expert; group_list itself stays on the
+    // device) are HBM bound: use the small-tile kernel.  An expert with more than 32 rows then
+    // costs one pass over its weights per 32 rows.
+    if (a->M <= 24 * a->G) return launch_gemm_cap<FMT, GM_SKINNY_BLOCKS>(P, a, stream);
+    return launch_gemm_cap<FMT, GM_MT_MAX>(P, a, stream);
 }
 
 int launch_grouped_gemm(const moe_grouped_args* a, hipStream_t stream) {
+    // Decode-sized batches on the K-contiguous containers (on average at most 4 rows per
+    // expert) are pure weight streaming: the GEMV kernel reads every weight row as one
+    // contiguous run and is the faster of the two there.  It keeps the dequantized weights in
+    // fp32 instead of rounding them to bf16 first, which stays inside the op's tolerance.
+    if ((a->format == MOE_FMT_FP4_B32 || a->format == MOE_FMT_BF16) && a->M <= 4 * a->G)
+        return launch_grouped_gemv(a, stream);
     switch (a->format) {
         case MOE_FMT_FP4_REF: return launch_gemm_fmt<MOE_FMT_FP4_REF>(a, stream);
         case MOE_FMT_FP8_REF: return launch_gemm_fmt<MOE_FMT_FP8_REF>(a, stream);
