@@ -30,23 +30,25 @@ __device__ __forceinline__ void group_rows(const int64_t* gl, int g, int64_t M, 
 
 // ---------------------------------------------------------------------------------
 // K-contiguous containers: MOE_FMT_BF16 [G,N,K] and MOE_FMT_FP4_B32 [G,N,K/2].
-// A workgroup owns 64 weight rows (n) of one expert; each wavefront takes 8 rows at
+// A workgroup owns NR_WG weight rows (n) of one expert; each wavefront takes 8 rows at
 // a time and all of K: a lane reads CH consecutive k (16 bytes) of each of the 8
 // rows per step, so a step has 8 independent 1 KiB loads in flight per wavefront.
 // x (<= 4 rows) is staged once in LDS.
 // ---------------------------------------------------------------------------------
-constexpr int GVK_NR_WG = 64;
-constexpr int GVK_NRW = 8;
+constexpr int GVK_NRW = 8;  // weight rows per wavefront step
 
 template <int FMT>
 struct KMajor;
 template <>
 struct KMajor<MOE_FMT_BF16> {
-    static constexpr int CH = 8;  // k per lane per step (16 B of weights)
+    static constexpr int CH = 8;      // k per lane per step (16 B of weights)
+    static constexpr int NR_WG = 32;  // weight rows per workgroup: small enough that the last
+                                      // round of workgroups does not leave CUs idle for long
 };
 template <>
 struct KMajor<MOE_FMT_FP4_B32> {
-    static constexpr int CH = 32;  // one scale block (16 B of codes)
+    static constexpr int CH = 32;     // one scale block (16 B of codes)
+    static constexpr int NR_WG = 64;  // decode-bound: fewer x refills per weight byte pay more
 };
 
 // LDS position (in 16-byte units) of the 8 k starting at k8*8, laid out so that the
@@ -69,7 +71,7 @@ __device__ __forceinline__ void gemv_kmajor_rows(const uint8_t* __restrict__ wg,
     const int nchunks = (K + GV_KC - 1) / GV_KC;
     const int64_t wrow_bytes = FMT == MOE_FMT_BF16 ? (int64_t)K * 2 : (int64_t)K / 2;
 
-    for (int it = 0; it < GVK_NR_WG / (4 * GVK_NRW); ++it) {
+    for (int it = 0; it < KMajor<FMT>::NR_WG / (4 * GVK_NRW); ++it) {
         const int n = n0 + (it * 4 + wave) * GVK_NRW;
         float acc[GVK_NRW][MG];
 #pragma unroll
@@ -158,7 +160,7 @@ __global__ __launch_bounds__(256) void gemv_kmajor_kernel(const uint16_t* __rest
                                                           const int64_t* __restrict__ gl, uint16_t* __restrict__ y,
                                                           int64_t M, int K, int N) {
     extern __shared__ u32x4_t xs[];
-    const int g = blockIdx.y, n0 = blockIdx.x * GVK_NR_WG;
+    const int g = blockIdx.y, n0 = blockIdx.x * KMajor<FMT>::NR_WG;
     int64_t start, end;
     group_rows(gl, g, M, start, end);
     if (end <= start) return;
@@ -377,7 +379,7 @@ static int launch_kmajor(const moe_grouped_args* a, hipStream_t stream) {
     const int kc = (int)(a->K < GV_KC ? a->K : GV_KC);
     const size_t lds = (size_t)GV_ROWS * GV_KC / 8 * 16;
     (void)kc;
-    dim3 grid((unsigned)((a->N + GVK_NR_WG - 1) / GVK_NR_WG), (unsigned)a->G);
+    dim3 grid((unsigned)((a->N + KMajor<FMT>::NR_WG - 1) / KMajor<FMT>::NR_WG), (unsigned)a->G);
     hipLaunchKernelGGL((gemv_kmajor_kernel<FMT>), grid, dim3(256), lds, stream,
                        static_cast<const uint16_t*>(a->x), static_cast<const uint8_t*>(a->weight),
                        static_cast<const uint16_t*>(a->scale), a->group_list, static_cast<uint16_t*>(a->y), a->M,
