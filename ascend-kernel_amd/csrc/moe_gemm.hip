@@ -167,6 +167,24 @@ struct BTraits<MOE_FMT_INT4> {
         const int grow = c.gmul ? (int)__umulhi(sub, c.gmul) : (int)sub;
         raw.sc[s] = ldg_b64(c.rs, c.vs, (grow * c.N + c.n0) * 2);
     }
+    // LDS-direct loads of the packed tile: instruction j (8 per k step) brings rows 8j + (lane >> 3)
+    // of the tile into the 1 KB block j of the stage, lane l landing at byte 16 l.  Position
+    // lane & 7 of a row holds the chunk that stage_store would put there; 8j + a has the
+    // (row >> 3) parity of j, and a wavefront only issues instructions with j = w (mod 4).
+    __device__ static __forceinline__ int dma_voff(const BCtx& c, int lane) {
+        return (lane >> 3) * (c.N >> 1) + (((lane & 7) ^ (4 * (c.w & 1))) * 16);
+    }
+    __device__ static __forceinline__ int dma_soff(const BCtx& c, int k0, int j) {
+        return (k0 + 8 * j) * (c.N >> 1) + (c.n0 >> 1);
+    }
+    // scale row of 32-k sub-step `sub` of the expert
+    __device__ static __forceinline__ int scale_row(const BCtx& c, uint32_t sub) {
+        return c.gmul ? (int)__umulhi(sub, c.gmul) : (int)sub;
+    }
+    // this lane's 4 scales of sub-step s from the stage's scale block (2 rows of 256 bf16)
+    __device__ static __forceinline__ void load_scale_lds(Raw& raw, const BCtx& c, int s, const u32x4_t* stile) {
+        raw.sc[s] = *reinterpret_cast<const u32x2_t*>(reinterpret_cast<const uint16_t*>(stile) + 256 * s + col(c, 0));
+    }
     // The nibble masks come from BCtx as values the compiler cannot see through; with literal
     // masks it folds them into every extraction and spends an extra instruction per element
     // instead of using v_cvt_f32_ubyte0 / ubyte1 directly.
@@ -409,18 +427,10 @@ __device__ __forceinline__ int a_lds_unit(int row, int c) {
     return row * (BK / 8) + (c ^ (row & 7));
 }
 
-template <int FMT, int MT, int CAPB>
-__device__ __forceinline__ void gemm_tile(const GemmParams& P, u32x4_t* lds_a, u32x4_t* lds_b, int g, int64_t row0,
-                                          int rows, int n0) {
-    using T = BTraits<FMT>;
-    constexpr int BK = T::BK, NS = T::NS;
-    constexpr int CPR = BK / 8;               // 16-byte chunks per tile row
-    constexpr int RPP = GM_THREADS / CPR;     // rows loaded per pass
-    constexpr int PASSES = (16 * MT + RPP - 1) / RPP;
-    constexpr int ABUF = 16 * CAPB * CPR;  // units per buffer (CAPB row blocks)
-
+// Per-tile context: lane coordinates and the buffer resources of expert g.
+template <int FMT>
+__device__ __forceinline__ void make_ctx(BCtx& c, const GemmParams& P, int g, int n0) {
     const int tid = threadIdx.x, lane = tid & 63;
-    BCtx c;
     c.K = P.K; c.N = P.N; c.n0 = n0;
     c.i = lane & 15; c.q = lane >> 4; c.w = __builtin_amdgcn_readfirstlane(tid >> 6);
     c.gmul = 0; c.sg = nullptr; c.og = nullptr; c.s8 = nullptr;
@@ -461,6 +471,49 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& P, u32x4_t* lds_a, u
             c.rs = c.rw;
             break;
     }
+}
+
+// Epilogue: fp32 -> bf16 (RNE), rows beyond the chunk are dropped.
+template <int FMT, int MT>
+__device__ __forceinline__ void store_tile(const GemmParams& P, const BCtx& c, f32x4_t (&acc)[MT][4], int64_t row0, int rows,
+                                           int n0) {
+    using T = BTraits<FMT>;
+    constexpr bool N_CONTIG = (FMT == MOE_FMT_INT4 || FMT == MOE_FMT_FP4_REF || FMT == MOE_FMT_INT8 ||
+                               FMT == MOE_FMT_FP8_REF);
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int row = 16 * mt + 4 * c.q + r;
+            if (row < rows) {
+                uint16_t* yp = P.y + (row0 + row) * (int64_t)P.N + n0;
+                if (N_CONTIG) {
+                    u32x2_t v;
+                    v[0] = pack_bf16_rne(acc[mt][0][r], acc[mt][1][r]);
+                    v[1] = pack_bf16_rne(acc[mt][2][r], acc[mt][3][r]);
+                    *reinterpret_cast<u32x2_t*>(yp + T::col(c, 0)) = v;
+                } else {
+#pragma unroll
+                    for (int t = 0; t < 4; ++t)
+                        yp[T::col(c, t)] = (uint16_t)(pack_bf16_rne(acc[mt][t][r], 0.f) & 0xffffu);
+                }
+            }
+        }
+}
+
+template <int FMT, int MT, int CAPB>
+__device__ __forceinline__ void gemm_tile(const GemmParams& P, u32x4_t* lds_a, u32x4_t* lds_b, int g, int64_t row0,
+                                          int rows, int n0) {
+    using T = BTraits<FMT>;
+    constexpr int BK = T::BK, NS = T::NS;
+    constexpr int CPR = BK / 8;               // 16-byte chunks per tile row
+    constexpr int RPP = GM_THREADS / CPR;     // rows loaded per pass
+    constexpr int PASSES = (16 * MT + RPP - 1) / RPP;
+    constexpr int ABUF = 16 * CAPB * CPR;  // units per buffer (CAPB row blocks)
+
+    const int tid = threadIdx.x;
+    BCtx c;
+    make_ctx<FMT>(c, P, g, n0);
     T::init(c);
     typename T::Dq dq;
     dq.init_tile(c);
@@ -631,28 +684,190 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& P, u32x4_t* lds_a, u
     // the accumulators were last written by MFMAs the compiler cannot see: wait out their latency
     asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
 
-    // epilogue: fp32 -> bf16 (RNE), rows beyond the chunk are dropped
-    constexpr bool N_CONTIG = (FMT == MOE_FMT_INT4 || FMT == MOE_FMT_FP4_REF || FMT == MOE_FMT_INT8 ||
-                               FMT == MOE_FMT_FP8_REF);
+    store_tile<FMT, MT>(P, c, acc, row0, rows, n0);
+}
+
+// ---------------------------------------------------------------------------------
+// Tile routine for the containers whose packed tile is staged in LDS (int4).  Everything the
+// k loop consumes -- x tile, packed weight tile, scales -- is brought in by loads that write
+// LDS directly (buffer_load_dwordx4 ... lds: lane l of the wavefront writes bytes
+// [16 l, 16 l + 16) after the instruction's LDS base).  No staging registers and no LDS
+// store instructions, so the loads can run far ahead: a ring of GM_STAGES stages per
+// operand, filled about three k steps (several microseconds of HBM latency) before use.
+//
+// Schedule of k step kt (two 32-k sub-steps, 8 MT MFMAs per wavefront):
+//   first MFMA slots   issue the loads of x stage kt+3 and of weight/scale stage kt+4
+//                      (weights run one stage ahead of x because their dwords are pulled
+//                      into registers a step before they are decoded);
+//   whole step         MFMAs on x stage kt, decode of the next sub-step between them,
+//                      this lane's packed dwords of stage kt+1 read from LDS as soon as the
+//                      registers holding stage kt's have been decoded;
+//   R fragments before the end   wait until this wavefront's own loads issued two steps ago
+//                      (x stage kt+1, weight stage kt+2) have landed, then the step's only
+//                      barrier; the x fragment reads that follow already belong to step kt+1,
+//                      so no LDS latency is exposed at the step boundary.
+// A stage is overwritten by loads issued after the barrier that follows its last read.
+// vmcnt counts this wavefront's loads in order; every wavefront issues the same number NI
+// of them per step (waves without a row block of their own repeat one), so "at most 2 NI
+// outstanding" means exactly "the group issued two steps ago has landed".
+// ---------------------------------------------------------------------------------
+constexpr int GM_STAGES = 4;
+constexpr int GM_SC_UNITS = 64;   // 16-byte units of one scale stage: 2 rows of 256 bf16
+
+#define MOE_LDS_PTR(p) ((__attribute__((address_space(3))) void*)(p))
+__device__ __forceinline__ void lds_load16(rsrc_t r, const u32x4_t* dst, int voff, int soff) {
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(r, MOE_LDS_PTR(const_cast<u32x4_t*>(dst)), 16, voff, soff, 0, 0);
+}
+
+template <int N>
+struct IntC { static constexpr int value = N; };
+
+template <int FMT, int MT, int CAPB>
+__device__ __forceinline__ void gemm_tile_dma(const GemmParams& P, u32x4_t* smem, int g, int64_t row0, int rows, int n0) {
+    using T = BTraits<FMT>;
+    static_assert(T::BK == 64 && T::NS == 2 && GM_STAGES == 4, "the schedule below is written for two sub-steps and four stages");
+    constexpr int BK = 64, NS = 2, S = GM_STAGES;
+    constexpr int A_UNITS = 16 * CAPB * 8, B_UNITS = T::B_LDS_UNITS;
+    u32x4_t* lds_a = smem;
+    u32x4_t* lds_b = lds_a + S * A_UNITS;
+    u32x4_t* lds_s = lds_b + S * B_UNITS;
+
+    const int lane = threadIdx.x & 63;
+    BCtx c;
+    make_ctx<FMT>(c, P, g, n0);
+    T::init(c);
+    typename T::Dq dq;
+    dq.init_tile(c);
+
+    // x rows through a buffer resource that ends after the last valid row (padded rows read as
+    // zeros).  Load instruction j covers rows 8j + (lane >> 3); position lane & 7 of a row
+    // holds chunk (lane & 7) ^ (row & 7), the swizzle a_lds_unit expects.
+    const rsrc_t rx = make_rsrc(P.x + row0 * (int64_t)P.K, (int64_t)rows * P.K * 2);
+    const int va = ((lane >> 3) * P.K + (((lane & 7) ^ (lane >> 3)) * 8)) * 2;
+    const int vb = T::dma_voff(c, lane);
+    const int vs_lo = (lane & 31) * 16;
+    const int hi_mask = lane >= 32 ? -1 : 0;
+
+    constexpr int NA = (2 * MT + 3) / 4;          // x load instructions per wavefront per step
+    constexpr int NB = B_UNITS / 64 / 4;          // packed-tile instructions per wavefront per step
+    constexpr int NI = NA + NB + 1;               // + the scale block
+    static_assert(NI <= 4 * MT, "not enough MFMA slots for the loads of one step");
+    static_assert(2 * NI <= 63, "vmcnt range");
+
+    // m-th load of the group issued during step kt (kt may be negative in the prologue)
+    auto issue = [&](int m, int kt) {
+        if (m < NA) {
+            int j = c.w + 4 * m;
+            if (4 * NA > 2 * MT) j = j >= 2 * MT ? j - 2 * MT : j;   // repeat a block rather than issue fewer loads
+            lds_load16(rx, lds_a + ((kt + 3) & (S - 1)) * A_UNITS + j * 64, va, (8 * j * P.K + (kt + 3) * BK) * 2);
+        } else if (m < NA + NB) {
+            const int j = c.w + 4 * (m - NA);
+            lds_load16(c.rw, lds_b + ((kt + 4) & (S - 1)) * B_UNITS + j * 64, vb, T::dma_soff(c, (kt + 4) * BK, j));
+        } else {
+            const uint32_t sub = (uint32_t)((kt + 4) * NS);
+            const int g0 = T::scale_row(c, sub), g1 = T::scale_row(c, sub + 1);
+            const int vs = vs_lo + (hi_mask & ((g1 - g0) * P.N * 2));   // lanes 32..63 fetch the row of sub-step 1
+            lds_load16(c.rs, lds_s + ((kt + 4) & (S - 1)) * GM_SC_UNITS, vs, (g0 * P.N + n0) * 2);
+        }
+    };
+
+    f32x4_t acc[MT][4];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const int row = 16 * mt + 4 * c.q + r;
-            if (row < rows) {
-                uint16_t* yp = P.y + (row0 + row) * (int64_t)P.N + n0;
-                if (N_CONTIG) {
-                    u32x2_t v;
-                    v[0] = pack_bf16_rne(acc[mt][0][r], acc[mt][1][r]);
-                    v[1] = pack_bf16_rne(acc[mt][2][r], acc[mt][3][r]);
-                    *reinterpret_cast<u32x2_t*>(yp + T::col(c, 0)) = v;
-                } else {
+        for (int t = 0; t < 4; ++t) acc[mt][t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+
+    typename T::Raw raw;
+    const int nk = P.K / BK;
+    constexpr int RING = 3, F = NS * MT;
+    constexpr int R = RING < MT ? RING : MT;   // x fragments read ahead of their MFMAs
+    constexpr int SLOTS = 4 * MT, UNITS = 17;
+
+    __syncthreads();  // every wavefront is done with the previous tile (its loads have been drained)
+    // weight stage 0 first, then the three groups the steady state would have issued before step 0
 #pragma unroll
-                    for (int t = 0; t < 4; ++t)
-                        yp[T::col(c, t)] = (uint16_t)(pack_bf16_rne(acc[mt][t][r], 0.f) & 0xffffu);
+    for (int m = NA; m < NI; ++m) issue(m, -4);
+#pragma unroll
+    for (int kt = -3; kt < 0; ++kt)
+#pragma unroll
+        for (int m = 0; m < NI; ++m) issue(m, kt);
+    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(2 * NI) : "memory");   // x 0, weights 0 and 1 are in LDS
+
+#pragma unroll
+    for (int s = 0; s < NS; ++s) {
+        T::load_sub(raw, c, 0, s, lds_b);
+        T::load_scale_lds(raw, c, s, lds_s);
+    }
+    u32x4_t bf[2][4];
+    dq.prep(raw, c, 0);
+#pragma unroll
+    for (int p = 0; p < 4; ++p)
+#pragma unroll
+        for (int t = 0; t < 4; ++t) dq.unit(raw, c, 0, p, t, bf[0]);
+
+    // ring of 4 x fragments; fragment f of step kt lives in afr[(kt F + f) & 3], F is even
+    u32x4_t afr[4];
+    auto read_a = [&](const u32x4_t* la, int f, int ring) {
+        afr[ring & 3] = la[a_lds_unit<BK>(16 * (f % MT) + c.i, T::a_chunk(f / MT, c.q))];
+    };
+#pragma unroll
+    for (int f = 0; f < R; ++f) read_a(lds_a, f, f);
+
+    auto step = [&](int kt, auto parity) {
+        constexpr int base = (F & 3) ? 2 * decltype(parity)::value : 0;   // (kt F) & 3
+        const u32x4_t* la = lds_a + (kt & (S - 1)) * A_UNITS;
+        const u32x4_t* la_next = lds_a + ((kt + 1) & (S - 1)) * A_UNITS;
+        const u32x4_t* btile = lds_b + ((kt + 1) & (S - 1)) * B_UNITS;
+        const u32x4_t* stile = lds_s + ((kt + 1) & (S - 1)) * GM_SC_UNITS;
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int s = 0; s < NS; ++s) {
+            const int sn = (s + 1) % NS;                 // sub-step being decoded
+            u32x4_t* bcur = bf[s & 1];
+            u32x4_t* bnxt = bf[(s + 1) & 1];
+#pragma unroll
+            for (int slot = 0; slot < SLOTS; ++slot) {
+                const int mt = slot >> 2, t = slot & 3, f = s * MT + mt;
+                if (s == NS - 1 && slot == 4 * (MT - R))
+                    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(2 * NI) : "memory");
+                if (t == 0) {
+                    const int fr = f + R;
+                    if (fr < F) read_a(la, fr, base + fr); else read_a(la_next, fr - F, base + fr);
                 }
+                mfma_16x16x32(acc[mt][t], afr[(base + f) & 3], bcur[t]);
+                if (s == 0) {
+                    if (slot < NI) issue(slot, kt);
+                    if (slot == (NI < SLOTS ? NI : SLOTS - 1)) {
+                        // sub-step 0 of step kt+1: its registers were decoded during the previous step
+                        T::load_sub(raw, c, 0, 0, btile);
+                        T::load_scale_lds(raw, c, 0, stile);
+                    }
+                }
+#pragma unroll
+                for (int u = (slot * UNITS + SLOTS - 1) / SLOTS; u < ((slot + 1) * UNITS + SLOTS - 1) / SLOTS; ++u) {
+                    if (u == 0)
+                        dq.prep(raw, c, sn);
+                    else
+                        dq.unit(raw, c, sn, (u - 1) >> 2, (u - 1) & 3, bnxt);
+                }
+                if (slot == ((UNITS - 1) * SLOTS) / UNITS && sn != 0) {
+                    // sub-step sn of this step has been decoded: refill its registers from step kt+1
+                    T::load_sub(raw, c, 0, sn, btile);
+                    T::load_scale_lds(raw, c, sn, stile);
+                }
+                __builtin_amdgcn_sched_barrier(0);
             }
         }
+    };
+    for (int kt = 0; kt < nk; kt += 2) {
+        step(kt, IntC<0>{});
+        if (kt + 1 < nk) step(kt + 1, IntC<1>{});
+    }
+    // drain this wavefront's loads (they target stages past K and are never read) before the next
+    // tile reuses the ring; the accumulators were last written by MFMAs the compiler cannot see
+    asm volatile("s_waitcnt vmcnt(0)\n\ts_nop 15\n\ts_nop 15" ::: "memory");
+
+    store_tile<FMT, MT>(P, c, acc, row0, rows, n0);
 }
 
 // ---------------------------------------------------------------------------------
@@ -669,6 +884,25 @@ __device__ __forceinline__ void expert_chunks(int m, int& chunks, int& bpc) {
     bpc = chunks ? (nblk + chunks - 1) / chunks : 0;
 }
 
+// The prefill kernel of the staged containers uses the LDS-direct tile routine.
+template <int FMT, int CAPB>
+constexpr bool uses_lds_loads() { return BTraits<FMT>::B_LDS_UNITS > 0 && CAPB == GM_MT_MAX; }
+// 16-byte LDS units the tile routine needs (the tile prefix array follows them)
+template <int FMT, int CAPB>
+constexpr int tile_lds_units() {
+    return uses_lds_loads<FMT, CAPB>()
+               ? GM_STAGES * (16 * CAPB * 8 + BTraits<FMT>::B_LDS_UNITS + GM_SC_UNITS)
+               : 2 * 16 * CAPB * (BTraits<FMT>::BK / 8) + 2 * BTraits<FMT>::B_LDS_UNITS;
+}
+
+template <int FMT, int MT, int CAPB>
+__device__ __forceinline__ void run_tile(const GemmParams& P, u32x4_t* smem, int g, int64_t row0, int rows, int n0) {
+    if constexpr (uses_lds_loads<FMT, CAPB>())
+        gemm_tile_dma<FMT, MT, CAPB>(P, smem, g, row0, rows, n0);
+    else
+        gemm_tile<FMT, MT, CAPB>(P, smem, smem + 2 * 16 * CAPB * (BTraits<FMT>::BK / 8), g, row0, rows, n0);
+}
+
 // CAPB = row blocks the LDS x buffers hold.  CAPB = GM_MT_MAX is the prefill kernel (tiles up
 // to the format's MT_MAX blocks, one workgroup per CU).  CAPB = GM_SKINNY_BLOCKS is the decode
 // kernel: tiles of at most 32 rows, a fraction of the registers and LDS, several workgroups
@@ -678,9 +912,7 @@ __global__ __launch_bounds__(GM_THREADS, CAPB == GM_MT_MAX ? 1 : GM_SKINNY_WAVES
     extern __shared__ u32x4_t smem[];
     constexpr int BK = BTraits<FMT>::BK;
     constexpr int MTM = CAPB < BTraits<FMT>::MT_MAX ? CAPB : BTraits<FMT>::MT_MAX;   // row blocks per tile
-    u32x4_t* lds_a = smem;                                                         // 2 buffers
-    u32x4_t* lds_b = smem + 2 * 16 * CAPB * (BK / 8);                              // 2 packed weight tiles
-    int* prefix = reinterpret_cast<int*>(lds_b + 2 * BTraits<FMT>::B_LDS_UNITS);   // [G + 1]
+    int* prefix = reinterpret_cast<int*>(smem + tile_lds_units<FMT, CAPB>());      // [G + 1]
     const int tid = threadIdx.x;
     const int ntile_n = P.N / GM_BN;
 
@@ -749,40 +981,40 @@ __global__ __launch_bounds__(GM_THREADS, CAPB == GM_MT_MAX ? 1 : GM_SKINNY_WAVES
         const int n0 = nt * GM_BN;
         switch (mt) {
             case 1:
-                if constexpr (MTM >= 1) gemm_tile<FMT, 1, CAPB>(P, lds_a, lds_b, g, row0, rows, n0);
+                if constexpr (MTM >= 1) run_tile<FMT, 1, CAPB>(P, smem, g, row0, rows, n0);
                 break;
             case 2:
-                if constexpr (MTM >= 2) gemm_tile<FMT, 2, CAPB>(P, lds_a, lds_b, g, row0, rows, n0);
+                if constexpr (MTM >= 2) run_tile<FMT, 2, CAPB>(P, smem, g, row0, rows, n0);
                 break;
             case 3:
-                if constexpr (MTM >= 3) gemm_tile<FMT, 3, CAPB>(P, lds_a, lds_b, g, row0, rows, n0);
+                if constexpr (MTM >= 3) run_tile<FMT, 3, CAPB>(P, smem, g, row0, rows, n0);
                 break;
             case 4:
-                if constexpr (MTM >= 4) gemm_tile<FMT, 4, CAPB>(P, lds_a, lds_b, g, row0, rows, n0);
+                if constexpr (MTM >= 4) run_tile<FMT, 4, CAPB>(P, smem, g, row0, rows, n0);
                 break;
             case 5:
-                if constexpr (MTM >= 5) gemm_tile<FMT, 5, CAPB>(P, lds_a, lds_b, g, row0, rows, n0);
+                if constexpr (MTM >= 5) run_tile<FMT, 5, CAPB>(P, smem, g, row0, rows, n0);
                 break;
             case 6:
-                if constexpr (MTM >= 6) gemm_tile<FMT, 6, CAPB>(P, lds_a, lds_b, g, row0, rows, n0);
+                if constexpr (MTM >= 6) run_tile<FMT, 6, CAPB>(P, smem, g, row0, rows, n0);
                 break;
             case 7:
-                if constexpr (MTM >= 7) gemm_tile<FMT, 7, CAPB>(P, lds_a, lds_b, g, row0, rows, n0);
+                if constexpr (MTM >= 7) run_tile<FMT, 7, CAPB>(P, smem, g, row0, rows, n0);
                 break;
             case 8:
-                if constexpr (MTM >= 8) gemm_tile<FMT, 8, CAPB>(P, lds_a, lds_b, g, row0, rows, n0);
+                if constexpr (MTM >= 8) run_tile<FMT, 8, CAPB>(P, smem, g, row0, rows, n0);
                 break;
             case 9:
-                if constexpr (MTM >= 9) gemm_tile<FMT, 9, CAPB>(P, lds_a, lds_b, g, row0, rows, n0);
+                if constexpr (MTM >= 9) run_tile<FMT, 9, CAPB>(P, smem, g, row0, rows, n0);
                 break;
             case 10:
-                if constexpr (MTM >= 10) gemm_tile<FMT, 10, CAPB>(P, lds_a, lds_b, g, row0, rows, n0);
+                if constexpr (MTM >= 10) run_tile<FMT, 10, CAPB>(P, smem, g, row0, rows, n0);
                 break;
             case 11:
-                if constexpr (MTM >= 11) gemm_tile<FMT, 11, CAPB>(P, lds_a, lds_b, g, row0, rows, n0);
+                if constexpr (MTM >= 11) run_tile<FMT, 11, CAPB>(P, smem, g, row0, rows, n0);
                 break;
             case 12:
-                if constexpr (MTM >= 12) gemm_tile<FMT, 12, CAPB>(P, lds_a, lds_b, g, row0, rows, n0);
+                if constexpr (MTM >= 12) run_tile<FMT, 12, CAPB>(P, smem, g, row0, rows, n0);
                 break;
             default: break;
         }
@@ -793,8 +1025,7 @@ template <int FMT, int CAPB>
 static int launch_gemm_cap(const GemmParams& P, const moe_grouped_args* a, hipStream_t stream) {
     constexpr int BK = BTraits<FMT>::BK;
     constexpr int MTM = CAPB < BTraits<FMT>::MT_MAX ? CAPB : BTraits<FMT>::MT_MAX;
-    const size_t lds = (size_t)2 * 16 * CAPB * (BK / 8) * 16 + (size_t)2 * BTraits<FMT>::B_LDS_UNITS * 16 +
-                       ((size_t)a->G + 1) * sizeof(int);
+    const size_t lds = (size_t)tile_lds_units<FMT, CAPB>() * 16 + ((size_t)a->G + 1) * sizeof(int);
     if (lds > 160 * 1024 - 2048) return MOE_ERR_TOO_LARGE;
     static bool attr_set = false;  // idempotent; a race only repeats the same call
     if (!attr_set) {
