@@ -480,23 +480,25 @@ __device__ __forceinline__ void store_tile(const GemmParams& P, const BCtx& c, f
     using T = BTraits<FMT>;
     constexpr bool N_CONTIG = (FMT == MOE_FMT_INT4 || FMT == MOE_FMT_FP4_REF || FMT == MOE_FMT_INT8 ||
                                FMT == MOE_FMT_FP8_REF);
+    // through a buffer resource that ends after the tile's last valid row: stores to padded
+    // rows fall outside it and are dropped
+    const rsrc_t ry = make_rsrc(P.y + row0 * (int64_t)P.N, (int64_t)rows * P.N * 2);
+    const int vy = (4 * c.q * P.N + n0) * 2;
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-            const int row = 16 * mt + 4 * c.q + r;
-            if (row < rows) {
-                uint16_t* yp = P.y + (row0 + row) * (int64_t)P.N + n0;
-                if (N_CONTIG) {
-                    u32x2_t v;
-                    v[0] = pack_bf16_rne(acc[mt][0][r], acc[mt][1][r]);
-                    v[1] = pack_bf16_rne(acc[mt][2][r], acc[mt][3][r]);
-                    *reinterpret_cast<u32x2_t*>(yp + T::col(c, 0)) = v;
-                } else {
+            const int so = (16 * mt + r) * P.N * 2;
+            if (N_CONTIG) {
+                u32x2_t v;
+                v[0] = pack_bf16_rne(acc[mt][0][r], acc[mt][1][r]);
+                v[1] = pack_bf16_rne(acc[mt][2][r], acc[mt][3][r]);
+                __builtin_amdgcn_raw_buffer_store_b64(v, ry, vy + T::col(c, 0) * 2, so, 0);
+            } else {
 #pragma unroll
-                    for (int t = 0; t < 4; ++t)
-                        yp[T::col(c, t)] = (uint16_t)(pack_bf16_rne(acc[mt][t][r], 0.f) & 0xffffu);
-                }
+                for (int t = 0; t < 4; ++t)
+                    __builtin_amdgcn_raw_buffer_store_b16((uint16_t)(pack_bf16_rne(acc[mt][t][r], 0.f) & 0xffffu), ry,
+                                                          vy + T::col(c, t) * 2, so, 0);
             }
         }
 }
@@ -870,6 +872,268 @@ __device__ __forceinline__ void gemm_tile_dma(const GemmParams& P, u32x4_t* smem
     store_tile<FMT, MT>(P, c, acc, row0, rows, n0);
 }
 
+
+// ---------------------------------------------------------------------------------
+// Prefill tile routine with 8 wavefronts (two per SIMD).  A single wavefront issues at most
+// one instruction every ~5 cycles whatever its kind, and an MFMA holds its issue port for
+// 8 of its 16 cycles; with one wavefront per SIMD the decode instructions and the MFMAs of
+// a k step therefore add up instead of overlapping.  Two wavefronts per SIMD let one decode
+// while the other's MFMAs run.  Each wavefront owns 32 of the tile's 256 columns for all rows
+// (two MFMAs per x fragment), so every weight element is still decoded exactly once per
+// tile; the price is that every x fragment is read from LDS by 8 wavefronts instead of 4.
+// Loads, stage ring and barrier placement are those of gemm_tile_dma.
+//
+// int4 layout.  Wavefront wv = 4 dg + np handles, of the tile's 32 dword columns, the 16
+// starting at 16 dg, and of each dword the byte np: lane (i, q) owns columns
+// 8 (16 dg + i) + 2 np + {0, 1} (MFMA t = the nibble of that byte) for its 8 k rows.
+// Decode of a k-row pair (a, b): v_perm gathers the two bytes, the low nibbles (& 0x0f0f)
+// and high nibbles (>> 4 & 0x0f0f) are bytes 0x00..0x0f, which read as OCP e4m3 are
+// exactly q / 512 -- v_cvt_pk_f32_fp8 converts both rows at once -- and one fma per element
+// applies 512 * scale and the zero point: q s - 8 s = (q - 8) s exactly.
+// ---------------------------------------------------------------------------------
+template <int FMT>
+struct W8Traits;
+
+template <>
+struct W8Traits<MOE_FMT_INT4> {
+    static constexpr int MT_MAX = 10;   // 160 rows: the largest tile that keeps every value in registers
+    static constexpr int B_LDS_UNITS = 64 * 8;   // packed tile of one k step: 64 rows of 128 bytes
+    struct Ctx {
+        rsrc_t rw, rs;
+        int N, n0, i, q, wv, dg, np;
+        uint32_t gmul, sel, mask;   // scale-row multiplier (see BCtx), v_perm selector, 0x0f0f
+    };
+    struct Raw {
+        uint32_t r[2][8];
+        uint32_t sc[2];
+    };
+    __device__ static __forceinline__ int col(const Ctx& c, int t) { return 8 * (16 * c.dg + c.i) + 2 * c.np + t; }
+    __device__ static __forceinline__ void init(Ctx& c, const GemmParams& P, int g, int n0) {
+        const int tid = threadIdx.x, lane = tid & 63;
+        c.N = P.N; c.n0 = n0;
+        c.i = lane & 15; c.q = lane >> 4; c.wv = __builtin_amdgcn_readfirstlane(tid >> 6);
+        c.dg = c.wv >> 2; c.np = c.wv & 3;
+        const int64_t KN = (int64_t)P.K * P.N;
+        c.rw = make_rsrc(P.w + g * (KN >> 1), KN >> 1);
+        c.rs = make_rsrc(static_cast<const uint16_t*>(P.scale) + (int64_t)g * P.scale_rows * P.N,
+                         (int64_t)P.scale_rows * P.N * 2);
+        const uint32_t per = (uint32_t)((P.K / P.scale_rows) >> 5);  // sub-steps per scale group
+        c.gmul = per == 1 ? 0u : 0xffffffffu / per + 1u;
+        c.sel = 0x0c0c0000u | ((4u + (uint32_t)c.np) << 8) | (uint32_t)c.np;   // byte np of a, byte np of b, 0, 0
+        c.mask = 0x0f0fu;
+        asm volatile("" : "+s"(c.mask));   // kept opaque so that it stays one SGPR operand
+    }
+    // LDS-direct load of the packed tile: wavefront wv brings rows 8 wv + (lane >> 3) into the 1 KB
+    // block wv of the stage; position lane & 7 of a row holds chunk (lane & 7) ^ 4 (wv & 1), i.e. the
+    // two 64-byte halves of the rows with odd (row >> 3) are swapped, so that the four q groups of a
+    // wavefront read from both halves of the banks.
+    __device__ static __forceinline__ int dma_voff(const Ctx& c, int lane) {
+        return (lane >> 3) * (c.N >> 1) + (((lane & 7) ^ (4 * (c.wv & 1))) * 16);
+    }
+    __device__ static __forceinline__ int dma_soff(const Ctx& c, int k0) { return (k0 + 8 * c.wv) * (c.N >> 1) + (c.n0 >> 1); }
+    __device__ static __forceinline__ int scale_row(const Ctx& c, uint32_t sub) {
+        return c.gmul ? (int)__umulhi(sub, c.gmul) : (int)sub;
+    }
+    __device__ static __forceinline__ void load_sub(Raw& raw, const Ctx& c, int s, const u32x4_t* tile) {
+        const uint32_t* t32 = reinterpret_cast<const uint32_t*>(tile);
+        const int d = 16 * c.dg + c.i;  // dword of the row
+        const int unit = (d >> 2) ^ (4 * (c.q & 1));
+#pragma unroll
+        for (int j = 0; j < 8; ++j) raw.r[s][j] = t32[((32 * s + 8 * c.q + j) * 8 + unit) * 4 + (d & 3)];
+    }
+    __device__ static __forceinline__ void load_scale(Raw& raw, const Ctx& c, int s, const u32x4_t* stile) {
+        raw.sc[s] = *reinterpret_cast<const uint32_t*>(reinterpret_cast<const uint16_t*>(stile) + 256 * s + col(c, 0));
+    }
+    struct Dq {
+        float m[2], z[2];
+        uint32_t pr;   // gathered bytes of the current row pair
+        __device__ __forceinline__ void prep(const Raw& raw, int s) {
+            const uint32_t sc = raw.sc[s];
+            const float s0 = bf16_lo(sc), s1 = bf16_hi(sc);
+            m[0] = s0 * 512.f; m[1] = s1 * 512.f;
+            z[0] = -8.f * s0; z[1] = -8.f * s1;
+        }
+        // half unit: nibble t of row pair p -> dword p of the fragment of MFMA t
+        __device__ __forceinline__ void unit(const Raw& raw, const Ctx& c, int s, int p, int t, u32x4_t out[2]) {
+            if (t == 0) pr = __builtin_amdgcn_perm(raw.r[s][2 * p + 1], raw.r[s][2 * p], c.sel);
+            const uint32_t nib = (t == 0 ? pr : pr >> 4) & c.mask;
+            const f32x2_t f = __builtin_amdgcn_cvt_pk_f32_fp8(nib, false);
+            out[t][p] = pack_bf16_rne(fmaf(f[0], m[t], z[t]), fmaf(f[1], m[t], z[t]));
+        }
+    };
+};
+
+constexpr int GM_W8_THREADS = 512;
+
+template <int FMT, int MT, int CAPB>
+__device__ __forceinline__ void gemm_tile_w8(const GemmParams& P, u32x4_t* smem, int g, int64_t row0, int rows, int n0) {
+    using T = W8Traits<FMT>;
+    constexpr int BK = 64, NS = 2, S = GM_STAGES;
+    static_assert(S == 4, "stage indices below are taken modulo 4");
+    constexpr int A_UNITS = 16 * CAPB * 8, B_UNITS = T::B_LDS_UNITS;
+    u32x4_t* lds_a = smem;
+    u32x4_t* lds_b = lds_a + S * A_UNITS;
+    u32x4_t* lds_s = lds_b + S * B_UNITS;
+
+    const int lane = threadIdx.x & 63;
+    typename T::Ctx c;
+    T::init(c, P, g, n0);
+    typename T::Dq dq;
+
+    // x rows through a buffer resource that ends after the last valid row (padded rows read as
+    // zeros).  Load instruction j covers rows 8j + (lane >> 3); position lane & 7 of a row
+    // holds chunk (lane & 7) ^ (row & 7), the swizzle a_lds_unit expects.
+    const rsrc_t rx = make_rsrc(P.x + row0 * (int64_t)P.K, (int64_t)rows * P.K * 2);
+    const int va = ((lane >> 3) * P.K + (((lane & 7) ^ (lane >> 3)) * 8)) * 2;
+    const int vb = T::dma_voff(c, lane);
+
+    constexpr int NA = (2 * MT + 7) / 8;   // x load instructions per wavefront per step
+    constexpr int NI = NA + 2;             // + one packed-tile instruction + this wavefront's eighth of the scales
+    constexpr int SLOTS = 2 * MT;          // MFMAs per sub-step
+    constexpr int UNITS = 9;               // prep + 8 half units per sub-step
+
+    // Loads.  Everything that does not change from step to step is computed here; per load the
+    // loop only adds a running k offset to a per-tile constant.  Stage numbers are compile-time
+    // constants (the k loop is unrolled four times).
+    int ja[NA], ca[NA];                    // x block of the m-th x load: LDS unit offset and byte offset of its rows
+#pragma unroll
+    for (int m = 0; m < NA; ++m) {
+        int j = c.wv + 8 * m;
+        if (8 * NA > 2 * MT) j = j % (2 * MT);   // repeat a block rather than issue fewer loads
+        ja[m] = j * 64;
+        ca[m] = 8 * j * P.K * 2;
+    }
+    const int cb = T::dma_soff(c, 0);                      // packed tile: rows 8 wv + [0,8) of the step
+    const int kb_step = BK * (P.N >> 1);
+    const int cs = n0 * 2 + (c.wv & 3) * 128;              // scales: bytes [128 (wv & 3), +128) of row wv >> 2
+    const int lane16 = lane * 16;
+    const bool s_lane = lane < 8;
+    // m-th load of the group issued during step kt: x stage kt+3 (LDS stage SA), weight and scale
+    // stage kt+4 (LDS stage SB)
+    auto issue = [&](int m, int kt, int SA, int SB) {
+        if (m < NA) {
+            lds_load16(rx, lds_a + SA * A_UNITS + ja[m], va, ca[m] + (kt + 3) * (BK * 2));
+        } else if (m == NA) {
+            lds_load16(c.rw, lds_b + SB * B_UNITS + c.wv * 64, vb, cb + (kt + 4) * kb_step);
+        } else {
+            const int grow = T::scale_row(c, (uint32_t)((kt + 4) * NS + (c.wv >> 2)));
+            if (s_lane) lds_load16(c.rs, lds_s + SB * GM_SC_UNITS + c.wv * 8, lane16, grow * (P.N * 2) + cs);
+        }
+    };
+
+    f32x4_t acc[MT][2];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int t = 0; t < 2; ++t) acc[mt][t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+
+    typename T::Raw raw;
+    const int nk = P.K / BK;
+    constexpr int RING = 3, F = NS * MT;
+    constexpr int R = RING < MT ? RING : MT;   // x fragments read ahead of their MFMAs
+
+    __syncthreads();  // every wavefront is done with the previous tile (its loads have been drained)
+    // weight stage 0 first, then the three groups the steady state would have issued before step 0
+#pragma unroll
+    for (int m = NA; m < NI; ++m) issue(m, -4, 0, 0);
+#pragma unroll
+    for (int kt = -3; kt < 0; ++kt)
+#pragma unroll
+        for (int m = 0; m < NI; ++m) issue(m, kt, kt + 3, (kt + 4) & 3);
+    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(2 * NI) : "memory");   // x 0, weights 0 and 1 are in LDS
+
+#pragma unroll
+    for (int s = 0; s < NS; ++s) {
+        T::load_sub(raw, c, s, lds_b);
+        T::load_scale(raw, c, s, lds_s);
+    }
+    u32x4_t bf[2][2];
+    dq.prep(raw, 0);
+#pragma unroll
+    for (int p = 0; p < 4; ++p)
+#pragma unroll
+        for (int t = 0; t < 2; ++t) dq.unit(raw, c, 0, p, t, bf[0]);
+
+    // ring of 4 x fragments; fragment f of step kt lives in afr[(kt F + f) & 3], F is even
+    u32x4_t afr[4];
+    auto read_a = [&](const u32x4_t* la, int f, int ring) {
+        afr[ring & 3] = la[a_lds_unit<BK>(16 * (f % MT) + c.i, 4 * (f / MT) + c.q)];
+    };
+#pragma unroll
+    for (int f = 0; f < R; ++f) read_a(lds_a, f, f);
+
+    // one k step; Q = kt & 3 as a compile-time constant
+    auto step = [&](int kt, auto q4) {
+        constexpr int Q = decltype(q4)::value;
+        constexpr int base = (F & 3) ? 2 * (Q & 1) : 0;   // (kt F) & 3
+        const u32x4_t* la = lds_a + Q * A_UNITS;
+        const u32x4_t* la_next = lds_a + ((Q + 1) & 3) * A_UNITS;
+        const u32x4_t* btile = lds_b + ((Q + 1) & 3) * B_UNITS;
+        const u32x4_t* stile = lds_s + ((Q + 1) & 3) * GM_SC_UNITS;
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int s = 0; s < NS; ++s) {
+            const int sn = (s + 1) % NS;                 // sub-step being decoded
+            u32x4_t* bcur = bf[s & 1];
+            u32x4_t* bnxt = bf[(s + 1) & 1];
+#pragma unroll
+            for (int slot = 0; slot < SLOTS; ++slot) {
+                const int mt = slot >> 1, t = slot & 1, f = s * MT + mt;
+                if (s == NS - 1 && slot == 2 * (MT - R))
+                    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(2 * NI) : "memory");
+                if (t == 0) {
+                    const int fr = f + R;
+                    if (fr < F) read_a(la, fr, base + fr); else read_a(la_next, fr - F, base + fr);
+                }
+                mfma_16x16x32(acc[mt][t], afr[(base + f) & 3], bcur[t]);
+                if (s == 0) {
+                    // this step's loads, spread over the first slots
+#pragma unroll
+                    for (int m = (slot * NI + SLOTS - 1) / SLOTS; m < ((slot + 1) * NI + SLOTS - 1) / SLOTS; ++m)
+                        issue(m, kt, (Q + 3) & 3, Q);
+                    if (slot == 0) {
+                        // sub-step 0 of step kt+1: its registers were decoded during the previous step
+                        T::load_sub(raw, c, 0, btile);
+                        T::load_scale(raw, c, 0, stile);
+                    }
+                }
+#pragma unroll
+                for (int u = (slot * UNITS + SLOTS - 1) / SLOTS; u < ((slot + 1) * UNITS + SLOTS - 1) / SLOTS; ++u) {
+                    if (u == 0)
+                        dq.prep(raw, sn);
+                    else
+                        dq.unit(raw, c, sn, (u - 1) >> 1, (u - 1) & 1, bnxt);
+                }
+                if (slot == SLOTS - 1 && sn != 0) {
+                    // sub-step sn of this step has been decoded: refill its registers from step kt+1
+                    T::load_sub(raw, c, sn, btile);
+                    T::load_scale(raw, c, sn, stile);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+    };
+    for (int kt = 0; kt < nk; kt += 4) {
+        step(kt, IntC<0>{});
+        if (kt + 1 < nk) step(kt + 1, IntC<1>{});
+        if (kt + 2 < nk) step(kt + 2, IntC<2>{});
+        if (kt + 3 < nk) step(kt + 3, IntC<3>{});
+    }
+    // drain this wavefront's loads (they target stages past K and are never read) before the next
+    // tile reuses the ring; the accumulators were last written by MFMAs the compiler cannot see
+    asm volatile("s_waitcnt vmcnt(0)\n\ts_nop 15\n\ts_nop 15" ::: "memory");
+
+    // epilogue through a buffer resource that ends after the tile's last valid row: stores to
+    // padded rows fall outside it and are dropped
+    const rsrc_t ry = make_rsrc(P.y + row0 * (int64_t)P.N, (int64_t)rows * P.N * 2);
+    const int vy = (4 * c.q * P.N + n0 + T::col(c, 0)) * 2;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+            __builtin_amdgcn_raw_buffer_store_b32(pack_bf16_rne(acc[mt][0][r], acc[mt][1][r]), ry, vy, (16 * mt + r) * P.N * 2, 0);
+}
+
 // ---------------------------------------------------------------------------------
 // Tile scheduler (role of GMMAntiquantProcess::Process,
 // grouped_gemm/op_kernel/grouped_matmul_antiquant.h:241-288).  Expert g with m_g rows
@@ -884,21 +1148,25 @@ __device__ __forceinline__ void expert_chunks(int m, int& chunks, int& bpc) {
     bpc = chunks ? (nblk + chunks - 1) / chunks : 0;
 }
 
-// The prefill kernel of the staged containers uses the LDS-direct tile routine.
-template <int FMT, int CAPB>
-constexpr bool uses_lds_loads() { return BTraits<FMT>::B_LDS_UNITS > 0 && CAPB == GM_MT_MAX; }
+// Kernel variants: WAVES = 4 is the general kernel (CAPB = GM_MT_MAX: prefill, one workgroup per
+// CU; CAPB = GM_SKINNY_BLOCKS: decode-sized tiles, several workgroups per CU); WAVES = 8 is the
+// prefill kernel with two wavefronts per SIMD, for the containers that have W8Traits.
+template <int FMT, int CAPB, int WAVES>
+constexpr int tile_mt_max() {
+    if constexpr (WAVES == 8) return W8Traits<FMT>::MT_MAX < CAPB ? W8Traits<FMT>::MT_MAX : CAPB;
+    else return CAPB < BTraits<FMT>::MT_MAX ? CAPB : BTraits<FMT>::MT_MAX;
+}
 // 16-byte LDS units the tile routine needs (the tile prefix array follows them)
-template <int FMT, int CAPB>
+template <int FMT, int CAPB, int WAVES>
 constexpr int tile_lds_units() {
-    return uses_lds_loads<FMT, CAPB>()
-               ? GM_STAGES * (16 * CAPB * 8 + BTraits<FMT>::B_LDS_UNITS + GM_SC_UNITS)
-               : 2 * 16 * CAPB * (BTraits<FMT>::BK / 8) + 2 * BTraits<FMT>::B_LDS_UNITS;
+    if constexpr (WAVES == 8) return GM_STAGES * (16 * CAPB * 8 + W8Traits<FMT>::B_LDS_UNITS + GM_SC_UNITS);
+    else return 2 * 16 * CAPB * (BTraits<FMT>::BK / 8) + 2 * BTraits<FMT>::B_LDS_UNITS;
 }
 
-template <int FMT, int MT, int CAPB>
+template <int FMT, int MT, int CAPB, int WAVES>
 __device__ __forceinline__ void run_tile(const GemmParams& P, u32x4_t* smem, int g, int64_t row0, int rows, int n0) {
-    if constexpr (uses_lds_loads<FMT, CAPB>())
-        gemm_tile_dma<FMT, MT, CAPB>(P, smem, g, row0, rows, n0);
+    if constexpr (WAVES == 8)
+        gemm_tile_w8<FMT, MT, CAPB>(P, smem, g, row0, rows, n0);
     else
         gemm_tile<FMT, MT, CAPB>(P, smem, smem + 2 * 16 * CAPB * (BTraits<FMT>::BK / 8), g, row0, rows, n0);
 }
@@ -907,19 +1175,19 @@ __device__ __forceinline__ void run_tile(const GemmParams& P, u32x4_t* smem, int
 // to the format's MT_MAX blocks, one workgroup per CU).  CAPB = GM_SKINNY_BLOCKS is the decode
 // kernel: tiles of at most 32 rows, a fraction of the registers and LDS, several workgroups
 // per CU to keep enough weight bytes in flight when the op is HBM bound.
-template <int FMT, int CAPB>
-__global__ __launch_bounds__(GM_THREADS, CAPB == GM_MT_MAX ? 1 : GM_SKINNY_WAVES) void grouped_gemm_kernel(GemmParams P) {
+template <int FMT, int CAPB, int WAVES>
+__global__ __launch_bounds__(64 * WAVES, CAPB == GM_MT_MAX ? 1 : GM_SKINNY_WAVES) void grouped_gemm_kernel(GemmParams P) {
     extern __shared__ u32x4_t smem[];
-    constexpr int BK = BTraits<FMT>::BK;
-    constexpr int MTM = CAPB < BTraits<FMT>::MT_MAX ? CAPB : BTraits<FMT>::MT_MAX;   // row blocks per tile
-    int* prefix = reinterpret_cast<int*>(smem + tile_lds_units<FMT, CAPB>());      // [G + 1]
+    constexpr int THREADS = 64 * WAVES;
+    constexpr int MTM = tile_mt_max<FMT, CAPB, WAVES>();                                  // row blocks per tile
+    int* prefix = reinterpret_cast<int*>(smem + tile_lds_units<FMT, CAPB, WAVES>());      // [G + 1]
     const int tid = threadIdx.x;
     const int ntile_n = P.N / GM_BN;
 
     // exclusive scan of tiles per expert: each thread takes a contiguous run of experts
     {
-        __shared__ int part[GM_THREADS];
-        const int per = (P.G + GM_THREADS - 1) / GM_THREADS;
+        __shared__ int part[THREADS];
+        const int per = (P.G + THREADS - 1) / THREADS;
         const int g0 = tid * per, g1 = min(P.G, g0 + per);
         int sum = 0;
         for (int g = g0; g < g1; ++g) {
@@ -933,7 +1201,7 @@ __global__ __launch_bounds__(GM_THREADS, CAPB == GM_MT_MAX ? 1 : GM_SKINNY_WAVES
         __syncthreads();
         if (tid == 0) {
             int run = 0;
-            for (int t = 0; t < GM_THREADS; ++t) { const int v = part[t]; part[t] = run; run += v; }
+            for (int t = 0; t < THREADS; ++t) { const int v = part[t]; part[t] = run; run += v; }
             prefix[P.G] = run;
         }
         __syncthreads();
@@ -981,55 +1249,54 @@ __global__ __launch_bounds__(GM_THREADS, CAPB == GM_MT_MAX ? 1 : GM_SKINNY_WAVES
         const int n0 = nt * GM_BN;
         switch (mt) {
             case 1:
-                if constexpr (MTM >= 1) run_tile<FMT, 1, CAPB>(P, smem, g, row0, rows, n0);
+                if constexpr (MTM >= 1) run_tile<FMT, 1, CAPB, WAVES>(P, smem, g, row0, rows, n0);
                 break;
             case 2:
-                if constexpr (MTM >= 2) run_tile<FMT, 2, CAPB>(P, smem, g, row0, rows, n0);
+                if constexpr (MTM >= 2) run_tile<FMT, 2, CAPB, WAVES>(P, smem, g, row0, rows, n0);
                 break;
             case 3:
-                if constexpr (MTM >= 3) run_tile<FMT, 3, CAPB>(P, smem, g, row0, rows, n0);
+                if constexpr (MTM >= 3) run_tile<FMT, 3, CAPB, WAVES>(P, smem, g, row0, rows, n0);
                 break;
             case 4:
-                if constexpr (MTM >= 4) run_tile<FMT, 4, CAPB>(P, smem, g, row0, rows, n0);
+                if constexpr (MTM >= 4) run_tile<FMT, 4, CAPB, WAVES>(P, smem, g, row0, rows, n0);
                 break;
             case 5:
-                if constexpr (MTM >= 5) run_tile<FMT, 5, CAPB>(P, smem, g, row0, rows, n0);
+                if constexpr (MTM >= 5) run_tile<FMT, 5, CAPB, WAVES>(P, smem, g, row0, rows, n0);
                 break;
             case 6:
-                if constexpr (MTM >= 6) run_tile<FMT, 6, CAPB>(P, smem, g, row0, rows, n0);
+                if constexpr (MTM >= 6) run_tile<FMT, 6, CAPB, WAVES>(P, smem, g, row0, rows, n0);
                 break;
             case 7:
-                if constexpr (MTM >= 7) run_tile<FMT, 7, CAPB>(P, smem, g, row0, rows, n0);
+                if constexpr (MTM >= 7) run_tile<FMT, 7, CAPB, WAVES>(P, smem, g, row0, rows, n0);
                 break;
             case 8:
-                if constexpr (MTM >= 8) run_tile<FMT, 8, CAPB>(P, smem, g, row0, rows, n0);
+                if constexpr (MTM >= 8) run_tile<FMT, 8, CAPB, WAVES>(P, smem, g, row0, rows, n0);
                 break;
             case 9:
-                if constexpr (MTM >= 9) run_tile<FMT, 9, CAPB>(P, smem, g, row0, rows, n0);
+                if constexpr (MTM >= 9) run_tile<FMT, 9, CAPB, WAVES>(P, smem, g, row0, rows, n0);
                 break;
             case 10:
-                if constexpr (MTM >= 10) run_tile<FMT, 10, CAPB>(P, smem, g, row0, rows, n0);
+                if constexpr (MTM >= 10) run_tile<FMT, 10, CAPB, WAVES>(P, smem, g, row0, rows, n0);
                 break;
             case 11:
-                if constexpr (MTM >= 11) run_tile<FMT, 11, CAPB>(P, smem, g, row0, rows, n0);
+                if constexpr (MTM >= 11) run_tile<FMT, 11, CAPB, WAVES>(P, smem, g, row0, rows, n0);
                 break;
             case 12:
-                if constexpr (MTM >= 12) run_tile<FMT, 12, CAPB>(P, smem, g, row0, rows, n0);
+                if constexpr (MTM >= 12) run_tile<FMT, 12, CAPB, WAVES>(P, smem, g, row0, rows, n0);
                 break;
             default: break;
         }
     }
 }
 
-template <int FMT, int CAPB>
+template <int FMT, int CAPB, int WAVES>
 static int launch_gemm_cap(const GemmParams& P, const moe_grouped_args* a, hipStream_t stream) {
-    constexpr int BK = BTraits<FMT>::BK;
-    constexpr int MTM = CAPB < BTraits<FMT>::MT_MAX ? CAPB : BTraits<FMT>::MT_MAX;
-    const size_t lds = (size_t)tile_lds_units<FMT, CAPB>() * 16 + ((size_t)a->G + 1) * sizeof(int);
+    constexpr int MTM = tile_mt_max<FMT, CAPB, WAVES>();
+    const size_t lds = (size_t)tile_lds_units<FMT, CAPB, WAVES>() * 16 + ((size_t)a->G + 1) * sizeof(int);
     if (lds > 160 * 1024 - 2048) return MOE_ERR_TOO_LARGE;
     static bool attr_set = false;  // idempotent; a race only repeats the same call
     if (!attr_set) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void*>(&grouped_gemm_kernel<FMT, CAPB>),
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(&grouped_gemm_kernel<FMT, CAPB, WAVES>),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 2048) != hipSuccess)
             return MOE_ERR_LAUNCH;
         attr_set = true;
@@ -1046,7 +1313,7 @@ static int launch_gemm_cap(const GemmParams& P, const moe_grouped_args* a, hipSt
     const int64_t want = max_tiles < cus * per_cu ? max_tiles : cus * per_cu;
     // a multiple of 8 so that the XCD-aware order covers every tile index
     const int64_t grid = want > 0 ? (want + 7) / 8 * 8 : 8;
-    hipLaunchKernelGGL((grouped_gemm_kernel<FMT, CAPB>), dim3((unsigned)grid), dim3(GM_THREADS), lds, stream, P);
+    hipLaunchKernelGGL((grouped_gemm_kernel<FMT, CAPB, WAVES>), dim3((unsigned)grid), dim3(64 * WAVES), lds, stream, P);
     return hipGetLastError() == hipSuccess ? MOE_OK : MOE_ERR_LAUNCH;
 }
 
@@ -1063,8 +1330,9 @@ static int launch_gemm_fmt(const moe_grouped_args* a, hipStream_t stream) {
     // Decode-like batches (on average at most 24 rows per expert; group_list itself stays on the
     // device) are HBM bound: use the small-tile kernel.  An expert with more than 32 rows then
     // costs one pass over its weights per 32 rows.
-    if (a->M <= 24 * a->G) return launch_gemm_cap<FMT, GM_SKINNY_BLOCKS>(P, a, stream);
-    return launch_gemm_cap<FMT, GM_MT_MAX>(P, a, stream);
+    if (a->M <= 24 * a->G) return launch_gemm_cap<FMT, GM_SKINNY_BLOCKS, 4>(P, a, stream);
+    if constexpr (FMT == MOE_FMT_INT4) return launch_gemm_cap<FMT, GM_MT_MAX, 8>(P, a, stream);
+    else return launch_gemm_cap<FMT, GM_MT_MAX, 4>(P, a, stream);
 }
 
 int launch_grouped_gemm(const moe_grouped_args* a, hipStream_t stream) {
