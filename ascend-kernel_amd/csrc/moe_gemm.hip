@@ -167,24 +167,6 @@ struct BTraits<MOE_FMT_INT4> {
         const int grow = c.gmul ? (int)__umulhi(sub, c.gmul) : (int)sub;
         raw.sc[s] = ldg_b64(c.rs, c.vs, (grow * c.N + c.n0) * 2);
     }
-    // LDS-direct loads of the packed tile: instruction j (8 per k step) brings rows 8j + (lane >> 3)
-    // of the tile into the 1 KB block j of the stage, lane l landing at byte 16 l.  Position
-    // lane & 7 of a row holds the chunk that stage_store would put there; 8j + a has the
-    // (row >> 3) parity of j, and a wavefront only issues instructions with j = w (mod 4).
-    __device__ static __forceinline__ int dma_voff(const BCtx& c, int lane) {
-        return (lane >> 3) * (c.N >> 1) + (((lane & 7) ^ (4 * (c.w & 1))) * 16);
-    }
-    __device__ static __forceinline__ int dma_soff(const BCtx& c, int k0, int j) {
-        return (k0 + 8 * j) * (c.N >> 1) + (c.n0 >> 1);
-    }
-    // scale row of 32-k sub-step `sub` of the expert
-    __device__ static __forceinline__ int scale_row(const BCtx& c, uint32_t sub) {
-        return c.gmul ? (int)__umulhi(sub, c.gmul) : (int)sub;
-    }
-    // this lane's 4 scales of sub-step s from the stage's scale block (2 rows of 256 bf16)
-    __device__ static __forceinline__ void load_scale_lds(Raw& raw, const BCtx& c, int s, const u32x4_t* stile) {
-        raw.sc[s] = *reinterpret_cast<const u32x2_t*>(reinterpret_cast<const uint16_t*>(stile) + 256 * s + col(c, 0));
-    }
     // The nibble masks come from BCtx as values the compiler cannot see through; with literal
     // masks it folds them into every extraction and spends an extra instruction per element
     // instead of using v_cvt_f32_ubyte0 / ubyte1 directly.
@@ -690,32 +672,11 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& P, u32x4_t* lds_a, u
 }
 
 // ---------------------------------------------------------------------------------
-// Tile routine for the containers whose packed tile is staged in LDS (int4).  Everything the
-// k loop consumes -- x tile, packed weight tile, scales -- is brought in by loads that write
-// LDS directly (buffer_load_dwordx4 ... lds: lane l of the wavefront writes bytes
-// [16 l, 16 l + 16) after the instruction's LDS base).  No staging registers and no LDS
-// store instructions, so the loads can run far ahead: a ring of GM_STAGES stages per
-// operand, filled about three k steps (several microseconds of HBM latency) before use.
-//
-// Schedule of k step kt (two 32-k sub-steps, 8 MT MFMAs per wavefront):
-//   first MFMA slots   issue the loads of x stage kt+3 and of weight/scale stage kt+4
-//                      (weights run one stage ahead of x because their dwords are pulled
-//                      into registers a step before they are decoded);
-//   whole step         MFMAs on x stage kt, decode of the next sub-step between them,
-//                      this lane's packed dwords of stage kt+1 read from LDS as soon as the
-//                      registers holding stage kt's have been decoded;
-//   R fragments before the end   wait until this wavefront's own loads issued two steps ago
-//                      (x stage kt+1, weight stage kt+2) have landed, then the step's only
-//                      barrier; the x fragment reads that follow already belong to step kt+1,
-//                      so no LDS latency is exposed at the step boundary.
-// A stage is overwritten by loads issued after the barrier that follows its last read.
-// vmcnt counts this wavefront's loads in order; every wavefront issues the same number NI
-// of them per step (waves without a row block of their own repeat one), so "at most 2 NI
-// outstanding" means exactly "the group issued two steps ago has landed".
+// LDS-direct loads (buffer_load_dwordx4 ... lds): lane l of the wavefront writes bytes
+// [16 l, 16 l + 16) after the instruction's LDS base.  No staging registers and no LDS store
+// instructions, so a tile routine can keep a ring of stages filled several k steps (a few
+// microseconds of HBM latency) ahead of their use.
 // ---------------------------------------------------------------------------------
-constexpr int GM_STAGES = 4;
-constexpr int GM_SC_UNITS = 64;   // 16-byte units of one scale stage: 2 rows of 256 bf16
-
 #define MOE_LDS_PTR(p) ((__attribute__((address_space(3))) void*)(p))
 __device__ __forceinline__ void lds_load16(rsrc_t r, const u32x4_t* dst, int voff, int soff) {
     __builtin_amdgcn_raw_ptr_buffer_load_lds(r, MOE_LDS_PTR(const_cast<u32x4_t*>(dst)), 16, voff, soff, 0, 0);
@@ -724,180 +685,53 @@ __device__ __forceinline__ void lds_load16(rsrc_t r, const u32x4_t* dst, int vof
 template <int N>
 struct IntC { static constexpr int value = N; };
 
-template <int FMT, int MT, int CAPB>
-__device__ __forceinline__ void gemm_tile_dma(const GemmParams& P, u32x4_t* smem, int g, int64_t row0, int rows, int n0) {
-    using T = BTraits<FMT>;
-    static_assert(T::BK == 64 && T::NS == 2 && GM_STAGES == 4, "the schedule below is written for two sub-steps and four stages");
-    constexpr int BK = 64, NS = 2, S = GM_STAGES;
-    constexpr int A_UNITS = 16 * CAPB * 8, B_UNITS = T::B_LDS_UNITS;
-    u32x4_t* lds_a = smem;
-    u32x4_t* lds_b = lds_a + S * A_UNITS;
-    u32x4_t* lds_s = lds_b + S * B_UNITS;
-
-    const int lane = threadIdx.x & 63;
-    BCtx c;
-    make_ctx<FMT>(c, P, g, n0);
-    T::init(c);
-    typename T::Dq dq;
-    dq.init_tile(c);
-
-    // x rows through a buffer resource that ends after the last valid row (padded rows read as
-    // zeros).  Load instruction j covers rows 8j + (lane >> 3); position lane & 7 of a row
-    // holds chunk (lane & 7) ^ (row & 7), the swizzle a_lds_unit expects.
-    const rsrc_t rx = make_rsrc(P.x + row0 * (int64_t)P.K, (int64_t)rows * P.K * 2);
-    const int va = ((lane >> 3) * P.K + (((lane & 7) ^ (lane >> 3)) * 8)) * 2;
-    const int vb = T::dma_voff(c, lane);
-    const int vs_lo = (lane & 31) * 16;
-    const int hi_mask = lane >= 32 ? -1 : 0;
-
-    constexpr int NA = (2 * MT + 3) / 4;          // x load instructions per wavefront per step
-    constexpr int NB = B_UNITS / 64 / 4;          // packed-tile instructions per wavefront per step
-    constexpr int NI = NA + NB + 1;               // + the scale block
-    static_assert(NI <= 4 * MT, "not enough MFMA slots for the loads of one step");
-    static_assert(2 * NI <= 63, "vmcnt range");
-
-    // m-th load of the group issued during step kt (kt may be negative in the prologue)
-    auto issue = [&](int m, int kt) {
-        if (m < NA) {
-            int j = c.w + 4 * m;
-            if (4 * NA > 2 * MT) j = j >= 2 * MT ? j - 2 * MT : j;   // repeat a block rather than issue fewer loads
-            lds_load16(rx, lds_a + ((kt + 3) & (S - 1)) * A_UNITS + j * 64, va, (8 * j * P.K + (kt + 3) * BK) * 2);
-        } else if (m < NA + NB) {
-            const int j = c.w + 4 * (m - NA);
-            lds_load16(c.rw, lds_b + ((kt + 4) & (S - 1)) * B_UNITS + j * 64, vb, T::dma_soff(c, (kt + 4) * BK, j));
-        } else {
-            const uint32_t sub = (uint32_t)((kt + 4) * NS);
-            const int g0 = T::scale_row(c, sub), g1 = T::scale_row(c, sub + 1);
-            const int vs = vs_lo + (hi_mask & ((g1 - g0) * P.N * 2));   // lanes 32..63 fetch the row of sub-step 1
-            lds_load16(c.rs, lds_s + ((kt + 4) & (S - 1)) * GM_SC_UNITS, vs, (g0 * P.N + n0) * 2);
-        }
-    };
-
-    f32x4_t acc[MT][4];
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-        for (int t = 0; t < 4; ++t) acc[mt][t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-
-    typename T::Raw raw;
-    const int nk = P.K / BK;
-    constexpr int RING = 3, F = NS * MT;
-    constexpr int R = RING < MT ? RING : MT;   // x fragments read ahead of their MFMAs
-    constexpr int SLOTS = 4 * MT, UNITS = 17;
-
-    __syncthreads();  // every wavefront is done with the previous tile (its loads have been drained)
-    // weight stage 0 first, then the three groups the steady state would have issued before step 0
-#pragma unroll
-    for (int m = NA; m < NI; ++m) issue(m, -4);
-#pragma unroll
-    for (int kt = -3; kt < 0; ++kt)
-#pragma unroll
-        for (int m = 0; m < NI; ++m) issue(m, kt);
-    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(2 * NI) : "memory");   // x 0, weights 0 and 1 are in LDS
-
-#pragma unroll
-    for (int s = 0; s < NS; ++s) {
-        T::load_sub(raw, c, 0, s, lds_b);
-        T::load_scale_lds(raw, c, s, lds_s);
-    }
-    u32x4_t bf[2][4];
-    dq.prep(raw, c, 0);
-#pragma unroll
-    for (int p = 0; p < 4; ++p)
-#pragma unroll
-        for (int t = 0; t < 4; ++t) dq.unit(raw, c, 0, p, t, bf[0]);
-
-    // ring of 4 x fragments; fragment f of step kt lives in afr[(kt F + f) & 3], F is even
-    u32x4_t afr[4];
-    auto read_a = [&](const u32x4_t* la, int f, int ring) {
-        afr[ring & 3] = la[a_lds_unit<BK>(16 * (f % MT) + c.i, T::a_chunk(f / MT, c.q))];
-    };
-#pragma unroll
-    for (int f = 0; f < R; ++f) read_a(lds_a, f, f);
-
-    auto step = [&](int kt, auto parity) {
-        constexpr int base = (F & 3) ? 2 * decltype(parity)::value : 0;   // (kt F) & 3
-        const u32x4_t* la = lds_a + (kt & (S - 1)) * A_UNITS;
-        const u32x4_t* la_next = lds_a + ((kt + 1) & (S - 1)) * A_UNITS;
-        const u32x4_t* btile = lds_b + ((kt + 1) & (S - 1)) * B_UNITS;
-        const u32x4_t* stile = lds_s + ((kt + 1) & (S - 1)) * GM_SC_UNITS;
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int s = 0; s < NS; ++s) {
-            const int sn = (s + 1) % NS;                 // sub-step being decoded
-            u32x4_t* bcur = bf[s & 1];
-            u32x4_t* bnxt = bf[(s + 1) & 1];
-#pragma unroll
-            for (int slot = 0; slot < SLOTS; ++slot) {
-                const int mt = slot >> 2, t = slot & 3, f = s * MT + mt;
-                if (s == NS - 1 && slot == 4 * (MT - R))
-                    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(2 * NI) : "memory");
-                if (t == 0) {
-                    const int fr = f + R;
-                    if (fr < F) read_a(la, fr, base + fr); else read_a(la_next, fr - F, base + fr);
-                }
-                mfma_16x16x32(acc[mt][t], afr[(base + f) & 3], bcur[t]);
-                if (s == 0) {
-                    if (slot < NI) issue(slot, kt);
-                    if (slot == (NI < SLOTS ? NI : SLOTS - 1)) {
-                        // sub-step 0 of step kt+1: its registers were decoded during the previous step
-                        T::load_sub(raw, c, 0, 0, btile);
-                        T::load_scale_lds(raw, c, 0, stile);
-                    }
-                }
-#pragma unroll
-                for (int u = (slot * UNITS + SLOTS - 1) / SLOTS; u < ((slot + 1) * UNITS + SLOTS - 1) / SLOTS; ++u) {
-                    if (u == 0)
-                        dq.prep(raw, c, sn);
-                    else
-                        dq.unit(raw, c, sn, (u - 1) >> 2, (u - 1) & 3, bnxt);
-                }
-                if (slot == ((UNITS - 1) * SLOTS) / UNITS && sn != 0) {
-                    // sub-step sn of this step has been decoded: refill its registers from step kt+1
-                    T::load_sub(raw, c, 0, sn, btile);
-                    T::load_scale_lds(raw, c, sn, stile);
-                }
-                __builtin_amdgcn_sched_barrier(0);
-            }
-        }
-    };
-    for (int kt = 0; kt < nk; kt += 2) {
-        step(kt, IntC<0>{});
-        if (kt + 1 < nk) step(kt + 1, IntC<1>{});
-    }
-    // drain this wavefront's loads (they target stages past K and are never read) before the next
-    // tile reuses the ring; the accumulators were last written by MFMAs the compiler cannot see
-    asm volatile("s_waitcnt vmcnt(0)\n\ts_nop 15\n\ts_nop 15" ::: "memory");
-
-    store_tile<FMT, MT>(P, c, acc, row0, rows, n0);
-}
-
-
 // ---------------------------------------------------------------------------------
-// Prefill tile routine with 8 wavefronts (two per SIMD).  A single wavefront issues at most
-// one instruction every ~5 cycles whatever its kind, and an MFMA holds its issue port for
-// 8 of its 16 cycles; with one wavefront per SIMD the decode instructions and the MFMAs of
-// a k step therefore add up instead of overlapping.  Two wavefronts per SIMD let one decode
-// while the other's MFMAs run.  Each wavefront owns 32 of the tile's 256 columns for all rows
-// (two MFMAs per x fragment), so every weight element is still decoded exactly once per
-// tile; the price is that every x fragment is read from LDS by 8 wavefronts instead of 4.
-// Loads, stage ring and barrier placement are those of gemm_tile_dma.
+// Prefill tile routine with two wavefronts per SIMD ("narrow" wavefronts: 32 columns each).
 //
-// int4 layout.  Wavefront wv = 4 dg + np handles, of the tile's 32 dword columns, the 16
-// starting at 16 dg, and of each dword the byte np: lane (i, q) owns columns
-// 8 (16 dg + i) + 2 np + {0, 1} (MFMA t = the nibble of that byte) for its 8 k rows.
+// A single wavefront issues at most one instruction every ~5 cycles whatever its kind, and an
+// MFMA holds the SIMD's vector issue port for about 8 of its 16 cycles; with one wavefront
+// per SIMD the decode instructions and the MFMAs of a k step add up instead of overlapping.
+// Here each wavefront owns 32 columns for all rows of the tile (two MFMAs per x fragment), so
+// that a CU holds 8 of them and every weight element is still decoded exactly once per tile.
+// NW wavefronts form a workgroup with a tile of 32 NW columns: NW = 8 is one workgroup per CU,
+// NW = 4 two independent workgroups per CU, each with its own barrier.
+//
+// Everything the k loop consumes -- x tile, packed weight tile, scales -- is brought in by
+// LDS-direct loads into a ring of S stages per operand.  Schedule of k step kt (two 32-k
+// sub-steps, 4 MT MFMAs per wavefront):
+//   first MFMA slots   issue the loads of x stage kt+S-1 and of weight/scale stage kt+S
+//                      (weights run one stage ahead of x because their dwords are pulled
+//                      into registers a step before they are decoded);
+//   whole step         MFMAs on x stage kt, decode of the next sub-step, this lane's packed
+//                      dwords of stage kt+1 read from LDS as soon as the registers holding
+//                      stage kt's have been decoded;
+//   R fragments before the end   wait until this wavefront's own loads issued S-2 steps ago
+//                      (x stage kt+1, weight stage kt+2) have landed, then the step's only
+//                      barrier; the x fragment reads that follow already belong to step kt+1,
+//                      so no LDS latency is exposed at the step boundary.
+// A stage is overwritten by loads issued after the barrier that follows its last read.
+// vmcnt counts this wavefront's loads in order; every wavefront issues the same number NI
+// of them per step (waves without a row block of their own repeat one), so "at most
+// (S-2) NI outstanding" means exactly "the group issued S-2 steps ago has landed".
+//
+// int4 layout.  Wavefront wv handles, of the tile's dword columns, the 16 starting at
+// 16 (wv >> 2), and of each dword the byte np = wv & 3: lane (i, q) owns columns
+// 8 (16 (wv >> 2) + i) + 2 np + {0, 1} (MFMA t = the nibble of that byte) for its 8 k rows.
 // Decode of a k-row pair (a, b): v_perm gathers the two bytes, the low nibbles (& 0x0f0f)
 // and high nibbles (>> 4 & 0x0f0f) are bytes 0x00..0x0f, which read as OCP e4m3 are
 // exactly q / 512 -- v_cvt_pk_f32_fp8 converts both rows at once -- and one fma per element
 // applies 512 * scale and the zero point: q s - 8 s = (q - 8) s exactly.
 // ---------------------------------------------------------------------------------
-template <int FMT>
-struct W8Traits;
+template <int FMT, int NW>
+struct NarrowTraits;
 
-template <>
-struct W8Traits<MOE_FMT_INT4> {
-    static constexpr int MT_MAX = 10;   // 160 rows: the largest tile that keeps every value in registers
-    static constexpr int B_LDS_UNITS = 64 * 8;   // packed tile of one k step: 64 rows of 128 bytes
+template <int NW>
+struct NarrowTraits<MOE_FMT_INT4, NW> {
+    static_assert(NW == 4 || NW == 8, "4 or 8 wavefronts per workgroup");
+    static constexpr int MT_MAX = 10;            // 160 rows: the largest tile that keeps every value in registers
+    static constexpr int ROW_UNITS = NW;         // 16-byte chunks of one packed row of the tile (32 NW columns)
+    static constexpr int B_LDS_UNITS = 64 * ROW_UNITS;   // packed tile of one k step: 64 rows
+    static constexpr int SC_UNITS = 8 * NW;      // scale block of one k step: 2 rows (one per sub-step) of 32 NW bf16
     struct Ctx {
         rsrc_t rw, rs;
         int N, n0, i, q, wv, dg, np;
@@ -923,26 +757,39 @@ struct W8Traits<MOE_FMT_INT4> {
         c.mask = 0x0f0fu;
         asm volatile("" : "+s"(c.mask));   // kept opaque so that it stays one SGPR operand
     }
-    // LDS-direct load of the packed tile: wavefront wv brings rows 8 wv + (lane >> 3) into the 1 KB
-    // block wv of the stage; position lane & 7 of a row holds chunk (lane & 7) ^ 4 (wv & 1), i.e. the
-    // two 64-byte halves of the rows with odd (row >> 3) are swapped, so that the four q groups of a
-    // wavefront read from both halves of the banks.
+    // LDS-direct load of the packed tile, one instruction per wavefront and k step: 64 / NW
+    // consecutive LDS rows starting at row (64 / NW) wv, lane l at byte 16 l of that block.
+    // The four q groups of a wavefront read the same dword columns of four different rows at
+    // once; the LDS placement spreads them over the banks:
+    //   NW = 8 (128-byte rows): the two 64-byte halves of the rows with odd (row >> 3) are swapped;
+    //   NW = 4 (64-byte rows):  LDS row rho holds tile row rho ^ ((rho >> 3) & 3).
     __device__ static __forceinline__ int dma_voff(const Ctx& c, int lane) {
-        return (lane >> 3) * (c.N >> 1) + (((lane & 7) ^ (4 * (c.wv & 1))) * 16);
+        if constexpr (NW == 8) {
+            return (lane >> 3) * (c.N >> 1) + (((lane & 7) ^ (4 * (c.wv & 1))) * 16);
+        } else {
+            const int rl = lane >> 2;                                   // LDS row within this wavefront's 16
+            const int row = rl ^ ((2 * c.wv + (rl >> 3)) & 3);          // tile row within the same 16
+            return row * (c.N >> 1) + (lane & 3) * 16;
+        }
     }
-    __device__ static __forceinline__ int dma_soff(const Ctx& c, int k0) { return (k0 + 8 * c.wv) * (c.N >> 1) + (c.n0 >> 1); }
+    __device__ static __forceinline__ int dma_soff(const Ctx& c) { return (64 / NW) * c.wv * (c.N >> 1) + (c.n0 >> 1); }
     __device__ static __forceinline__ int scale_row(const Ctx& c, uint32_t sub) {
         return c.gmul ? (int)__umulhi(sub, c.gmul) : (int)sub;
     }
     __device__ static __forceinline__ void load_sub(Raw& raw, const Ctx& c, int s, const u32x4_t* tile) {
         const uint32_t* t32 = reinterpret_cast<const uint32_t*>(tile);
         const int d = 16 * c.dg + c.i;  // dword of the row
-        const int unit = (d >> 2) ^ (4 * (c.q & 1));
+        if constexpr (NW == 8) {
+            const int unit = (d >> 2) ^ (4 * (c.q & 1));
 #pragma unroll
-        for (int j = 0; j < 8; ++j) raw.r[s][j] = t32[((32 * s + 8 * c.q + j) * 8 + unit) * 4 + (d & 3)];
+            for (int j = 0; j < 8; ++j) raw.r[s][j] = t32[((32 * s + 8 * c.q + j) * 8 + unit) * 4 + (d & 3)];
+        } else {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) raw.r[s][j] = t32[((32 * s + 8 * c.q + j) ^ c.q) * 16 + d];
+        }
     }
     __device__ static __forceinline__ void load_scale(Raw& raw, const Ctx& c, int s, const u32x4_t* stile) {
-        raw.sc[s] = *reinterpret_cast<const uint32_t*>(reinterpret_cast<const uint16_t*>(stile) + 256 * s + col(c, 0));
+        raw.sc[s] = *reinterpret_cast<const uint32_t*>(reinterpret_cast<const uint16_t*>(stile) + 32 * NW * s + col(c, 0));
     }
     struct Dq {
         float m[2], z[2];
@@ -963,14 +810,13 @@ struct W8Traits<MOE_FMT_INT4> {
     };
 };
 
-constexpr int GM_W8_THREADS = 512;
-
-template <int FMT, int MT, int CAPB>
-__device__ __forceinline__ void gemm_tile_w8(const GemmParams& P, u32x4_t* smem, int g, int64_t row0, int rows, int n0) {
-    using T = W8Traits<FMT>;
-    constexpr int BK = 64, NS = 2, S = GM_STAGES;
-    static_assert(S == 4, "stage indices below are taken modulo 4");
-    constexpr int A_UNITS = 16 * CAPB * 8, B_UNITS = T::B_LDS_UNITS;
+// NW wavefronts per workgroup, S stages, x buffers for CAPB row blocks.
+template <int FMT, int MT, int CAPB, int NW, int S>
+__device__ __forceinline__ void gemm_tile_narrow(const GemmParams& P, u32x4_t* smem, int g, int64_t row0, int rows, int n0) {
+    using T = NarrowTraits<FMT, NW>;
+    constexpr int BK = 64, NS = 2;
+    static_assert(S == 3 || S == 4, "ring of 3 or 4 stages");
+    constexpr int A_UNITS = 16 * CAPB * 8, B_UNITS = T::B_LDS_UNITS, SC_UNITS = T::SC_UNITS;
     u32x4_t* lds_a = smem;
     u32x4_t* lds_b = lds_a + S * A_UNITS;
     u32x4_t* lds_s = lds_b + S * B_UNITS;
@@ -987,37 +833,42 @@ __device__ __forceinline__ void gemm_tile_w8(const GemmParams& P, u32x4_t* smem,
     const int va = ((lane >> 3) * P.K + (((lane & 7) ^ (lane >> 3)) * 8)) * 2;
     const int vb = T::dma_voff(c, lane);
 
-    constexpr int NA = (2 * MT + 7) / 8;   // x load instructions per wavefront per step
-    constexpr int NI = NA + 2;             // + one packed-tile instruction + this wavefront's eighth of the scales
-    constexpr int SLOTS = 2 * MT;          // MFMAs per sub-step
-    constexpr int UNITS = 9;               // prep + 8 half units per sub-step
+    constexpr int NA = (2 * MT + NW - 1) / NW;   // x load instructions per wavefront per step
+    constexpr int NI = NA + 2;                   // + one packed-tile instruction + this wavefront's share of the scales
+    constexpr int SLOTS = 2 * MT;                // MFMAs per sub-step
+    constexpr int LEAD = S - 1;                  // x stage loaded during step kt: kt + LEAD; weights: kt + LEAD + 1
+    static_assert((S - 2) * NI <= 63, "vmcnt range");
 
     // Loads.  Everything that does not change from step to step is computed here; per load the
     // loop only adds a running k offset to a per-tile constant.  Stage numbers are compile-time
-    // constants (the k loop is unrolled four times).
+    // constants (the k loop is unrolled).
     int ja[NA], ca[NA];                    // x block of the m-th x load: LDS unit offset and byte offset of its rows
 #pragma unroll
     for (int m = 0; m < NA; ++m) {
-        int j = c.wv + 8 * m;
-        if (8 * NA > 2 * MT) j = j % (2 * MT);   // repeat a block rather than issue fewer loads
+        int j = c.wv + NW * m;
+        if (NW * NA > 2 * MT) j = j % (2 * MT);   // repeat a block rather than issue fewer loads
         ja[m] = j * 64;
         ca[m] = 8 * j * P.K * 2;
     }
-    const int cb = T::dma_soff(c, 0);                      // packed tile: rows 8 wv + [0,8) of the step
+    const int cb = T::dma_soff(c);
     const int kb_step = BK * (P.N >> 1);
-    const int cs = n0 * 2 + (c.wv & 3) * 128;              // scales: bytes [128 (wv & 3), +128) of row wv >> 2
+    // scales: the stage's block is 2 rows of 64 NW bytes; wavefront wv fetches 128 bytes of it with
+    // its first 8 lanes
+    constexpr int SEGS = NW / 2;                           // 128-byte segments per scale row of the tile
+    const int srow = c.wv / SEGS;
+    const int cs = n0 * 2 + (c.wv % SEGS) * 128;
     const int lane16 = lane * 16;
     const bool s_lane = lane < 8;
-    // m-th load of the group issued during step kt: x stage kt+3 (LDS stage SA), weight and scale
-    // stage kt+4 (LDS stage SB)
+    // m-th load of the group issued during step kt: x stage kt+LEAD (LDS stage SA), weight and
+    // scale stage kt+LEAD+1 (LDS stage SB)
     auto issue = [&](int m, int kt, int SA, int SB) {
         if (m < NA) {
-            lds_load16(rx, lds_a + SA * A_UNITS + ja[m], va, ca[m] + (kt + 3) * (BK * 2));
+            lds_load16(rx, lds_a + SA * A_UNITS + ja[m], va, ca[m] + (kt + LEAD) * (BK * 2));
         } else if (m == NA) {
-            lds_load16(c.rw, lds_b + SB * B_UNITS + c.wv * 64, vb, cb + (kt + 4) * kb_step);
+            lds_load16(c.rw, lds_b + SB * B_UNITS + c.wv * 64, vb, cb + (kt + LEAD + 1) * kb_step);
         } else {
-            const int grow = T::scale_row(c, (uint32_t)((kt + 4) * NS + (c.wv >> 2)));
-            if (s_lane) lds_load16(c.rs, lds_s + SB * GM_SC_UNITS + c.wv * 8, lane16, grow * (P.N * 2) + cs);
+            const int grow = T::scale_row(c, (uint32_t)((kt + LEAD + 1) * NS + srow));
+            if (s_lane) lds_load16(c.rs, lds_s + SB * SC_UNITS + c.wv * 8, lane16, grow * (P.N * 2) + cs);
         }
     };
 
@@ -1033,14 +884,14 @@ __device__ __forceinline__ void gemm_tile_w8(const GemmParams& P, u32x4_t* smem,
     constexpr int R = RING < MT ? RING : MT;   // x fragments read ahead of their MFMAs
 
     __syncthreads();  // every wavefront is done with the previous tile (its loads have been drained)
-    // weight stage 0 first, then the three groups the steady state would have issued before step 0
+    // weight stage 0 first, then the groups the steady state would have issued before step 0
 #pragma unroll
-    for (int m = NA; m < NI; ++m) issue(m, -4, 0, 0);
+    for (int m = NA; m < NI; ++m) issue(m, -LEAD - 1, 0, 0);
 #pragma unroll
-    for (int kt = -3; kt < 0; ++kt)
+    for (int kt = -LEAD; kt < 0; ++kt)
 #pragma unroll
-        for (int m = 0; m < NI; ++m) issue(m, kt, kt + 3, (kt + 4) & 3);
-    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(2 * NI) : "memory");   // x 0, weights 0 and 1 are in LDS
+        for (int m = 0; m < NI; ++m) issue(m, kt, (kt + LEAD) % S, (kt + LEAD + 1) % S);
+    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"((S - 2) * NI) : "memory");   // x 0, weights 0 and 1 are in LDS
 
 #pragma unroll
     for (int s = 0; s < NS; ++s) {
@@ -1062,14 +913,14 @@ __device__ __forceinline__ void gemm_tile_w8(const GemmParams& P, u32x4_t* smem,
 #pragma unroll
     for (int f = 0; f < R; ++f) read_a(lds_a, f, f);
 
-    // one k step; Q = kt & 3 as a compile-time constant
-    auto step = [&](int kt, auto q4) {
-        constexpr int Q = decltype(q4)::value;
-        constexpr int base = (F & 3) ? 2 * (Q & 1) : 0;   // (kt F) & 3
-        const u32x4_t* la = lds_a + Q * A_UNITS;
-        const u32x4_t* la_next = lds_a + ((Q + 1) & 3) * A_UNITS;
-        const u32x4_t* btile = lds_b + ((Q + 1) & 3) * B_UNITS;
-        const u32x4_t* stile = lds_s + ((Q + 1) & 3) * GM_SC_UNITS;
+    // one k step; Q = kt mod (unroll factor) as a compile-time constant
+    auto step = [&](int kt, auto qc) {
+        constexpr int Q = decltype(qc)::value;
+        constexpr int base = (F & 3) ? 2 * (Q & 1) : 0;   // (kt F) & 3; the unroll factor is even
+        const u32x4_t* la = lds_a + (Q % S) * A_UNITS;
+        const u32x4_t* la_next = lds_a + ((Q + 1) % S) * A_UNITS;
+        const u32x4_t* btile = lds_b + ((Q + 1) % S) * B_UNITS;
+        const u32x4_t* stile = lds_s + ((Q + 1) % S) * SC_UNITS;
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int s = 0; s < NS; ++s) {
@@ -1080,44 +931,48 @@ __device__ __forceinline__ void gemm_tile_w8(const GemmParams& P, u32x4_t* smem,
             for (int slot = 0; slot < SLOTS; ++slot) {
                 const int mt = slot >> 1, t = slot & 1, f = s * MT + mt;
                 if (s == NS - 1 && slot == 2 * (MT - R))
-                    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(2 * NI) : "memory");
+                    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"((S - 2) * NI) : "memory");
                 if (t == 0) {
                     const int fr = f + R;
                     if (fr < F) read_a(la, fr, base + fr); else read_a(la_next, fr - F, base + fr);
                 }
                 mfma_16x16x32(acc[mt][t], afr[(base + f) & 3], bcur[t]);
                 if (s == 0) {
-                    // this step's loads, spread over the first slots
+                    // this step's loads, spread over the slots of the first sub-step
 #pragma unroll
                     for (int m = (slot * NI + SLOTS - 1) / SLOTS; m < ((slot + 1) * NI + SLOTS - 1) / SLOTS; ++m)
-                        issue(m, kt, (Q + 3) & 3, Q);
+                        issue(m, kt, (Q + LEAD) % S, (Q + LEAD + 1) % S);
                     if (slot == 0) {
                         // sub-step 0 of step kt+1: its registers were decoded during the previous step
                         T::load_sub(raw, c, 0, btile);
                         T::load_scale(raw, c, 0, stile);
                     }
                 }
+                if (slot == SLOTS - 1) {
+                    // decode of the next sub-step (the compiler places it; the other wavefront of
+                    // the SIMD runs MFMAs meanwhile), then refill of the registers just decoded
+                    dq.prep(raw, sn);
 #pragma unroll
-                for (int u = (slot * UNITS + SLOTS - 1) / SLOTS; u < ((slot + 1) * UNITS + SLOTS - 1) / SLOTS; ++u) {
-                    if (u == 0)
-                        dq.prep(raw, sn);
-                    else
-                        dq.unit(raw, c, sn, (u - 1) >> 1, (u - 1) & 1, bnxt);
-                }
-                if (slot == SLOTS - 1 && sn != 0) {
-                    // sub-step sn of this step has been decoded: refill its registers from step kt+1
-                    T::load_sub(raw, c, sn, btile);
-                    T::load_scale(raw, c, sn, stile);
+                    for (int u = 0; u < 8; ++u) dq.unit(raw, c, sn, u >> 1, u & 1, bnxt);
+                    if (sn != 0) {
+                        T::load_sub(raw, c, sn, btile);
+                        T::load_scale(raw, c, sn, stile);
+                    }
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
     };
-    for (int kt = 0; kt < nk; kt += 4) {
+    constexpr int U = S == 4 ? 4 : 6;   // multiple of S (stage numbers) and of 2 (fragment ring)
+    for (int kt = 0; kt < nk; kt += U) {
         step(kt, IntC<0>{});
         if (kt + 1 < nk) step(kt + 1, IntC<1>{});
         if (kt + 2 < nk) step(kt + 2, IntC<2>{});
         if (kt + 3 < nk) step(kt + 3, IntC<3>{});
+        if constexpr (U == 6) {
+            if (kt + 4 < nk) step(kt + 4, IntC<4>{});
+            if (kt + 5 < nk) step(kt + 5, IntC<5>{});
+        }
     }
     // drain this wavefront's loads (they target stages past K and are never read) before the next
     // tile reuses the ring; the accumulators were last written by MFMAs the compiler cannot see
@@ -1148,41 +1003,58 @@ __device__ __forceinline__ void expert_chunks(int m, int& chunks, int& bpc) {
     bpc = chunks ? (nblk + chunks - 1) / chunks : 0;
 }
 
-// Kernel variants: WAVES = 4 is the general kernel (CAPB = GM_MT_MAX: prefill, one workgroup per
-// CU; CAPB = GM_SKINNY_BLOCKS: decode-sized tiles, several workgroups per CU); WAVES = 8 is the
-// prefill kernel with two wavefronts per SIMD, for the containers that have W8Traits.
-template <int FMT, int CAPB, int WAVES>
-constexpr int tile_mt_max() {
-    if constexpr (WAVES == 8) return W8Traits<FMT>::MT_MAX < CAPB ? W8Traits<FMT>::MT_MAX : CAPB;
-    else return CAPB < BTraits<FMT>::MT_MAX ? CAPB : BTraits<FMT>::MT_MAX;
-}
-// 16-byte LDS units the tile routine needs (the tile prefix array follows them)
-template <int FMT, int CAPB, int WAVES>
-constexpr int tile_lds_units() {
-    if constexpr (WAVES == 8) return GM_STAGES * (16 * CAPB * 8 + W8Traits<FMT>::B_LDS_UNITS + GM_SC_UNITS);
-    else return 2 * 16 * CAPB * (BTraits<FMT>::BK / 8) + 2 * BTraits<FMT>::B_LDS_UNITS;
-}
+// Kernel variants.
+//   GK_GENERAL  4 wavefronts of 64 columns, one workgroup per CU, tiles of up to 192 rows
+//   GK_SKINNY   the same tile routine with tiles of at most 32 rows and several workgroups per CU
+//               (decode-sized batches are HBM bound: more weight bytes in flight)
+//   GK_NARROW8  8 wavefronts of 32 columns, one workgroup per CU       } containers with
+//   GK_NARROW4  4 wavefronts of 32 columns, two workgroups per CU      } NarrowTraits
+enum { GK_GENERAL = 0, GK_SKINNY = 1, GK_NARROW8 = 2, GK_NARROW4 = 3 };
+#ifndef MOE_INT4_PREFILL_KIND
+#define MOE_INT4_PREFILL_KIND GK_NARROW8
+#endif
 
-template <int FMT, int MT, int CAPB, int WAVES>
+template <int FMT, int KIND>
+struct KernelCfg {
+    static constexpr bool NARROW = KIND == GK_NARROW8 || KIND == GK_NARROW4;
+    static constexpr int WAVES = KIND == GK_NARROW8 ? 8 : 4;
+    static constexpr int BN = NARROW ? 32 * WAVES : GM_BN;                       // columns per tile
+    static constexpr int WG_PER_CU = KIND == GK_SKINNY ? GM_SKINNY_WAVES : KIND == GK_NARROW4 ? 2 : 1;
+    static constexpr int STAGES = KIND == GK_NARROW4 ? 3 : 4;                    // narrow kernels only
+    static constexpr int CAPB = KIND == GK_SKINNY ? GM_SKINNY_BLOCKS : KIND == GK_NARROW4 ? 10 : GM_MT_MAX;
+    static constexpr int fmt_mt_max() {
+        if constexpr (NARROW) return NarrowTraits<FMT, WAVES>::MT_MAX;
+        else return BTraits<FMT>::MT_MAX;
+    }
+    static constexpr int MTM = CAPB < fmt_mt_max() ? CAPB : fmt_mt_max();        // row blocks per tile
+    // 16-byte LDS units of the tile routine (the tile prefix array follows them)
+    static constexpr int lds_units() {
+        if constexpr (NARROW)
+            return STAGES * (16 * CAPB * 8 + NarrowTraits<FMT, WAVES>::B_LDS_UNITS + NarrowTraits<FMT, WAVES>::SC_UNITS);
+        else
+            return 2 * 16 * CAPB * (BTraits<FMT>::BK / 8) + 2 * BTraits<FMT>::B_LDS_UNITS;
+    }
+};
+
+template <int FMT, int MT, int KIND>
 __device__ __forceinline__ void run_tile(const GemmParams& P, u32x4_t* smem, int g, int64_t row0, int rows, int n0) {
-    if constexpr (WAVES == 8)
-        gemm_tile_w8<FMT, MT, CAPB>(P, smem, g, row0, rows, n0);
+    using C = KernelCfg<FMT, KIND>;
+    if constexpr (C::NARROW)
+        gemm_tile_narrow<FMT, MT, C::CAPB, C::WAVES, C::STAGES>(P, smem, g, row0, rows, n0);
     else
-        gemm_tile<FMT, MT, CAPB>(P, smem, smem + 2 * 16 * CAPB * (BTraits<FMT>::BK / 8), g, row0, rows, n0);
+        gemm_tile<FMT, MT, C::CAPB>(P, smem, smem + 2 * 16 * C::CAPB * (BTraits<FMT>::BK / 8), g, row0, rows, n0);
 }
 
-// CAPB = row blocks the LDS x buffers hold.  CAPB = GM_MT_MAX is the prefill kernel (tiles up
-// to the format's MT_MAX blocks, one workgroup per CU).  CAPB = GM_SKINNY_BLOCKS is the decode
-// kernel: tiles of at most 32 rows, a fraction of the registers and LDS, several workgroups
-// per CU to keep enough weight bytes in flight when the op is HBM bound.
-template <int FMT, int CAPB, int WAVES>
-__global__ __launch_bounds__(64 * WAVES, CAPB == GM_MT_MAX ? 1 : GM_SKINNY_WAVES) void grouped_gemm_kernel(GemmParams P) {
+template <int FMT, int KIND>
+__global__ __launch_bounds__((64 * KernelCfg<FMT, KIND>::WAVES), (KernelCfg<FMT, KIND>::WG_PER_CU)) void grouped_gemm_kernel(GemmParams P) {
+    using C = KernelCfg<FMT, KIND>;
+    constexpr int WAVES = C::WAVES;
     extern __shared__ u32x4_t smem[];
     constexpr int THREADS = 64 * WAVES;
-    constexpr int MTM = tile_mt_max<FMT, CAPB, WAVES>();                                  // row blocks per tile
-    int* prefix = reinterpret_cast<int*>(smem + tile_lds_units<FMT, CAPB, WAVES>());      // [G + 1]
+    constexpr int MTM = C::MTM;
+    int* prefix = reinterpret_cast<int*>(smem + C::lds_units());      // [G + 1]
     const int tid = threadIdx.x;
-    const int ntile_n = P.N / GM_BN;
+    const int ntile_n = P.N / C::BN;
 
     // exclusive scan of tiles per expert: each thread takes a contiguous run of experts
     {
@@ -1246,74 +1118,73 @@ __global__ __launch_bounds__(64 * WAVES, CAPB == GM_MT_MAX ? 1 : GM_SKINNY_WAVES
         const int rlo = __builtin_amdgcn_readfirstlane((int)(uint32_t)(gbeg & 0xffffffffLL));
         const int rhi = __builtin_amdgcn_readfirstlane((int)(gbeg >> 32));
         const int64_t row0 = (((int64_t)rhi << 32) | (uint32_t)rlo) + rbeg;
-        const int n0 = nt * GM_BN;
+        const int n0 = nt * C::BN;
         switch (mt) {
             case 1:
-                if constexpr (MTM >= 1) run_tile<FMT, 1, CAPB, WAVES>(P, smem, g, row0, rows, n0);
+                if constexpr (MTM >= 1) run_tile<FMT, 1, KIND>(P, smem, g, row0, rows, n0);
                 break;
             case 2:
-                if constexpr (MTM >= 2) run_tile<FMT, 2, CAPB, WAVES>(P, smem, g, row0, rows, n0);
+                if constexpr (MTM >= 2) run_tile<FMT, 2, KIND>(P, smem, g, row0, rows, n0);
                 break;
             case 3:
-                if constexpr (MTM >= 3) run_tile<FMT, 3, CAPB, WAVES>(P, smem, g, row0, rows, n0);
+                if constexpr (MTM >= 3) run_tile<FMT, 3, KIND>(P, smem, g, row0, rows, n0);
                 break;
             case 4:
-                if constexpr (MTM >= 4) run_tile<FMT, 4, CAPB, WAVES>(P, smem, g, row0, rows, n0);
+                if constexpr (MTM >= 4) run_tile<FMT, 4, KIND>(P, smem, g, row0, rows, n0);
                 break;
             case 5:
-                if constexpr (MTM >= 5) run_tile<FMT, 5, CAPB, WAVES>(P, smem, g, row0, rows, n0);
+                if constexpr (MTM >= 5) run_tile<FMT, 5, KIND>(P, smem, g, row0, rows, n0);
                 break;
             case 6:
-                if constexpr (MTM >= 6) run_tile<FMT, 6, CAPB, WAVES>(P, smem, g, row0, rows, n0);
+                if constexpr (MTM >= 6) run_tile<FMT, 6, KIND>(P, smem, g, row0, rows, n0);
                 break;
             case 7:
-                if constexpr (MTM >= 7) run_tile<FMT, 7, CAPB, WAVES>(P, smem, g, row0, rows, n0);
+                if constexpr (MTM >= 7) run_tile<FMT, 7, KIND>(P, smem, g, row0, rows, n0);
                 break;
             case 8:
-                if constexpr (MTM >= 8) run_tile<FMT, 8, CAPB, WAVES>(P, smem, g, row0, rows, n0);
+                if constexpr (MTM >= 8) run_tile<FMT, 8, KIND>(P, smem, g, row0, rows, n0);
                 break;
             case 9:
-                if constexpr (MTM >= 9) run_tile<FMT, 9, CAPB, WAVES>(P, smem, g, row0, rows, n0);
+                if constexpr (MTM >= 9) run_tile<FMT, 9, KIND>(P, smem, g, row0, rows, n0);
                 break;
             case 10:
-                if constexpr (MTM >= 10) run_tile<FMT, 10, CAPB, WAVES>(P, smem, g, row0, rows, n0);
+                if constexpr (MTM >= 10) run_tile<FMT, 10, KIND>(P, smem, g, row0, rows, n0);
                 break;
             case 11:
-                if constexpr (MTM >= 11) run_tile<FMT, 11, CAPB, WAVES>(P, smem, g, row0, rows, n0);
+                if constexpr (MTM >= 11) run_tile<FMT, 11, KIND>(P, smem, g, row0, rows, n0);
                 break;
             case 12:
-                if constexpr (MTM >= 12) run_tile<FMT, 12, CAPB, WAVES>(P, smem, g, row0, rows, n0);
+                if constexpr (MTM >= 12) run_tile<FMT, 12, KIND>(P, smem, g, row0, rows, n0);
                 break;
             default: break;
         }
     }
 }
 
-template <int FMT, int CAPB, int WAVES>
-static int launch_gemm_cap(const GemmParams& P, const moe_grouped_args* a, hipStream_t stream) {
-    constexpr int MTM = tile_mt_max<FMT, CAPB, WAVES>();
-    const size_t lds = (size_t)tile_lds_units<FMT, CAPB, WAVES>() * 16 + ((size_t)a->G + 1) * sizeof(int);
-    if (lds > 160 * 1024 - 2048) return MOE_ERR_TOO_LARGE;
+template <int FMT, int KIND>
+static int launch_gemm_kind(const GemmParams& P, const moe_grouped_args* a, hipStream_t stream) {
+    using C = KernelCfg<FMT, KIND>;
+    const size_t lds = (size_t)C::lds_units() * 16 + ((size_t)a->G + 1) * sizeof(int);
+    const size_t lds_max = (160 * 1024 - 2048) / C::WG_PER_CU;
+    if (lds > lds_max) return MOE_ERR_TOO_LARGE;
     static bool attr_set = false;  // idempotent; a race only repeats the same call
     if (!attr_set) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void*>(&grouped_gemm_kernel<FMT, CAPB, WAVES>),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 2048) != hipSuccess)
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(&grouped_gemm_kernel<FMT, KIND>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_max) != hipSuccess)
             return MOE_ERR_LAUNCH;
         attr_set = true;
     }
     int dev = 0, cus = 256;
     if (hipGetDevice(&dev) != hipSuccess) return MOE_ERR_NO_DEVICE;
     if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return MOE_ERR_NO_DEVICE;
-    // persistent grid: one workgroup per CU (prefill) or as many as fit (decode), but no more than
-    // an upper bound on the tile count that needs no look at group_list (every expert adds at most
-    // one partly filled chunk)
-    const int64_t per_cu = CAPB == GM_MT_MAX ? 1 : GM_SKINNY_WAVES;
-    const int64_t max_chunks = a->M / (16 * MTM) + a->G;
-    const int64_t max_tiles = max_chunks * (a->N / GM_BN);
-    const int64_t want = max_tiles < cus * per_cu ? max_tiles : cus * per_cu;
+    // persistent grid: as many workgroups as the CUs hold, but no more than an upper bound on the
+    // tile count that needs no look at group_list (every expert adds at most one partly filled chunk)
+    const int64_t max_chunks = a->M / (16 * C::MTM) + a->G;
+    const int64_t max_tiles = max_chunks * (a->N / C::BN);
+    const int64_t want = max_tiles < (int64_t)cus * C::WG_PER_CU ? max_tiles : (int64_t)cus * C::WG_PER_CU;
     // a multiple of 8 so that the XCD-aware order covers every tile index
     const int64_t grid = want > 0 ? (want + 7) / 8 * 8 : 8;
-    hipLaunchKernelGGL((grouped_gemm_kernel<FMT, CAPB, WAVES>), dim3((unsigned)grid), dim3(64 * WAVES), lds, stream, P);
+    hipLaunchKernelGGL((grouped_gemm_kernel<FMT, KIND>), dim3((unsigned)grid), dim3(64 * C::WAVES), lds, stream, P);
     return hipGetLastError() == hipSuccess ? MOE_OK : MOE_ERR_LAUNCH;
 }
 
@@ -1330,9 +1201,9 @@ static int launch_gemm_fmt(const moe_grouped_args* a, hipStream_t stream) {
     // Decode-like batches (on average at most 24 rows per expert; group_list itself stays on the
     // device) are HBM bound: use the small-tile kernel.  An expert with more than 32 rows then
     // costs one pass over its weights per 32 rows.
-    if (a->M <= 24 * a->G) return launch_gemm_cap<FMT, GM_SKINNY_BLOCKS, 4>(P, a, stream);
-    if constexpr (FMT == MOE_FMT_INT4) return launch_gemm_cap<FMT, GM_MT_MAX, 8>(P, a, stream);
-    else return launch_gemm_cap<FMT, GM_MT_MAX, 4>(P, a, stream);
+    if (a->M <= 24 * a->G) return launch_gemm_kind<FMT, GK_SKINNY>(P, a, stream);
+    if constexpr (FMT == MOE_FMT_INT4) return launch_gemm_kind<FMT, MOE_INT4_PREFILL_KIND>(P, a, stream);
+    else return launch_gemm_kind<FMT, GK_GENERAL>(P, a, stream);
 }
 
 int launch_grouped_gemm(const moe_grouped_args* a, hipStream_t stream) {
