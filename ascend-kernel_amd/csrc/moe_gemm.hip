@@ -69,12 +69,6 @@ __device__ __forceinline__ void mfma_16x16x32(f32x4_t& acc, const u32x4_t& a, co
     asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
 }
 
-// Same with the accumulator in ordinary VGPRs.  A kernel that uses no AGPRs at all may use
-// the whole unified register file as VGPRs (otherwise the compiler splits it in two halves).
-__device__ __forceinline__ void mfma_16x16x32_v(f32x4_t& acc, const u32x4_t& a, const u32x4_t& b) {
-    asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+v"(acc) : "v"(a), "v"(b));
-}
-
 // Ties a value to the chain of volatile asm statements (the MFMAs): whatever is computed
 // from the returned value is emitted after every earlier volatile asm, whatever produced the
 // argument before every later one.  Emits no instruction.  Used to pin each decode unit
@@ -699,8 +693,7 @@ struct IntC { static constexpr int value = N; };
 // per SIMD the decode instructions and the MFMAs of a k step add up instead of overlapping.
 // Here each wavefront owns 32 columns for all rows of the tile (two MFMAs per x fragment), so
 // that a CU holds 8 of them and every weight element is still decoded exactly once per tile.
-// NW wavefronts form a workgroup with a tile of 32 NW columns: NW = 8 is one workgroup per CU,
-// NW = 4 two independent workgroups per CU, each with its own barrier.
+// The NW = 8 wavefronts of the workgroup share a tile of 256 columns.
 //
 // Everything the k loop consumes -- x tile, packed weight tile, scales -- is brought in by
 // LDS-direct loads into a ring of S stages per operand.  Schedule of k step kt (two 32-k
@@ -733,7 +726,7 @@ struct NarrowTraits;
 
 template <int NW>
 struct NarrowTraits<MOE_FMT_INT4, NW> {
-    static_assert(NW == 4 || NW == 8, "4 or 8 wavefronts per workgroup");
+    static_assert(NW == 8, "the LDS layout of the packed tile is written for 8 wavefronts (128-byte rows)");
     static constexpr int MT_MAX = 10;            // 160 rows: the largest tile that keeps every value in registers
     static constexpr int ROW_UNITS = NW;         // 16-byte chunks of one packed row of the tile (32 NW columns)
     static constexpr int B_LDS_UNITS = 64 * ROW_UNITS;   // packed tile of one k step: 64 rows
@@ -763,20 +756,12 @@ struct NarrowTraits<MOE_FMT_INT4, NW> {
         c.mask = 0x0f0fu;
         asm volatile("" : "+s"(c.mask));   // kept opaque so that it stays one SGPR operand
     }
-    // LDS-direct load of the packed tile, one instruction per wavefront and k step: 64 / NW
-    // consecutive LDS rows starting at row (64 / NW) wv, lane l at byte 16 l of that block.
-    // The four q groups of a wavefront read the same dword columns of four different rows at
-    // once; the LDS placement spreads them over the banks:
-    //   NW = 8 (128-byte rows): the two 64-byte halves of the rows with odd (row >> 3) are swapped;
-    //   NW = 4 (64-byte rows):  LDS row rho holds tile row rho ^ ((rho >> 3) & 3).
+    // LDS-direct load of the packed tile, one instruction per wavefront and k step: 8 consecutive
+    // LDS rows starting at row 8 wv, lane l at byte 16 l of that block.  The four q groups of a
+    // wavefront read the same dword columns of four different rows at once; the two 64-byte
+    // halves of the rows with odd (row >> 3) are swapped to spread them over the banks.
     __device__ static __forceinline__ int dma_voff(const Ctx& c, int lane) {
-        if constexpr (NW == 8) {
-            return (lane >> 3) * (c.N >> 1) + (((lane & 7) ^ (4 * (c.wv & 1))) * 16);
-        } else {
-            const int rl = lane >> 2;                                   // LDS row within this wavefront's 16
-            const int row = rl ^ ((2 * c.wv + (rl >> 3)) & 3);          // tile row within the same 16
-            return row * (c.N >> 1) + (lane & 3) * 16;
-        }
+        return (lane >> 3) * (c.N >> 1) + (((lane & 7) ^ (4 * (c.wv & 1))) * 16);
     }
     __device__ static __forceinline__ int dma_soff(const Ctx& c) { return (64 / NW) * c.wv * (c.N >> 1) + (c.n0 >> 1); }
     __device__ static __forceinline__ int scale_row(const Ctx& c, uint32_t sub) {
@@ -785,14 +770,9 @@ struct NarrowTraits<MOE_FMT_INT4, NW> {
     __device__ static __forceinline__ void load_sub(Raw& raw, const Ctx& c, int s, const u32x4_t* tile) {
         const uint32_t* t32 = reinterpret_cast<const uint32_t*>(tile);
         const int d = 16 * c.dg + c.i;  // dword of the row
-        if constexpr (NW == 8) {
-            const int unit = (d >> 2) ^ (4 * (c.q & 1));
+        const int unit = (d >> 2) ^ (4 * (c.q & 1));
 #pragma unroll
-            for (int j = 0; j < 8; ++j) raw.r[s][j] = t32[((32 * s + 8 * c.q + j) * 8 + unit) * 4 + (d & 3)];
-        } else {
-#pragma unroll
-            for (int j = 0; j < 8; ++j) raw.r[s][j] = t32[((32 * s + 8 * c.q + j) ^ c.q) * 16 + d];
-        }
+        for (int j = 0; j < 8; ++j) raw.r[s][j] = t32[((32 * s + 8 * c.q + j) * 8 + unit) * 4 + (d & 3)];
     }
     __device__ static __forceinline__ void load_scale(Raw& raw, const Ctx& c, int s, const u32x4_t* stile) {
         raw.sc[s] = *reinterpret_cast<const uint32_t*>(reinterpret_cast<const uint16_t*>(stile) + 32 * NW * s + col(c, 0));
@@ -996,278 +976,6 @@ __device__ __forceinline__ void gemm_tile_narrow(const GemmParams& P, u32x4_t* s
 }
 
 // ---------------------------------------------------------------------------------
-// Prefill tile routine with specialized wavefronts (int4).
-//
-// Wavefronts issue in order.  When one wavefront both decodes and multiplies, its decode
-// instructions queue up behind MFMAs that wait for the matrix pipe, and its MFMAs behind
-// decode chains; measured, two such wavefronts per SIMD keep the pipe barely half busy.  Here
-// the 8 wavefronts of the workgroup split the work by kind, one of each kind per SIMD:
-//   consumers (wavefronts 0-3)  64 columns each for all rows of the tile: x fragments and
-//                               ready-made bf16 weight fragments from LDS, MFMAs, nothing else;
-//   producers (wavefronts 4-7)  issue all LDS-direct loads (x tile, packed tile, scales), decode
-//                               the packed tile of their consumer's 64 columns and write the
-//                               bf16 fragments to LDS, lane-linear: lane l of MFMA t at
-//                               16-byte unit 64 t + l, so writes and reads are conflict-free.
-// Producers run one k step ahead: during consumer step kt they decode the packed stage kt+1
-// into fragment buffer (kt+1) & 1 and issue the loads of x stage kt+2 and packed stage kt+3
-// (rings of 3 stages).  One barrier per step: producers call it at the end of their step,
-// after their own loads of the previous step have landed (vmcnt) and their fragment writes
-// are done (lgkmcnt); consumers call it R x fragments before the end of theirs, after the
-// last LDS read of the current step, and prefetch the next step's first fragments behind it.
-// Everything a wavefront overwrites after a barrier was last read before that barrier.
-//
-// Decode (producer lane (i, q) of column group cw: the 4 columns of half cw & 1 of dword
-// column 16 (cw >> 1) + i, 8 k rows per sub-step): per k-row pair (a, b) v_perm gathers the
-// lane's two bytes of both rows; low nibbles (& 0x0f0f0f0f) and high nibbles (>> 4 &
-// 0x0f0f0f0f) are bytes 0x00..0x0f, which read as OCP e4m3 are exactly q / 512;
-// v_cvt_pk_f32_fp8 converts two at a time and one fma per element applies 512 * scale and
-// the zero point: q s - 8 s = (q - 8) s exactly.  2.5 VALU instructions per element.
-// ---------------------------------------------------------------------------------
-constexpr int PC_STAGES = 3;
-constexpr int PC_CAPB = 10;                        // x stages hold 160 rows
-constexpr int PC_A_UNITS = 16 * PC_CAPB * 8;       // 16-byte units of one x stage (rows of 64 bf16)
-constexpr int PC_B_UNITS = 64 * 8;                 // packed int4 tile of one k step: 64 rows of 128 bytes
-constexpr int PC_SC_UNITS = 64;                    // 2 scale rows (one per sub-step) of 256 bf16
-constexpr int PC_F_UNITS = 2 * 4 * 4 * 64;         // fragments of one k step: [sub-step][column group][t][lane]
-constexpr int PC_LDS_UNITS = PC_STAGES * (PC_A_UNITS + PC_B_UNITS + PC_SC_UNITS) + 2 * PC_F_UNITS;
-
-template <int MT>
-__device__ __forceinline__ void gemm_tile_pc_int4(const GemmParams& P, u32x4_t* smem, int g, int64_t row0, int rows, int n0) {
-    constexpr int BK = 64, NS = 2, S = PC_STAGES;
-    u32x4_t* lds_a = smem;
-    u32x4_t* lds_b = lds_a + S * PC_A_UNITS;
-    u32x4_t* lds_s = lds_b + S * PC_B_UNITS;
-    u32x4_t* lds_f = lds_s + S * PC_SC_UNITS;
-
-    const int tid = threadIdx.x, lane = tid & 63;
-    const int i = lane & 15, q = lane >> 4;
-    const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int cw = wv & 3;                                   // column group: 64 columns
-    const int col0 = 128 * (cw >> 1) + 8 * i + 4 * (cw & 1);  // this lane's 4 columns (MFMA t = column col0 + t)
-    const int nk = P.K / BK;
-
-    if (wv < 4) {
-        // ------------------------------------------------------------------ consumer
-        f32x4_t acc[MT][4];
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-            for (int t = 0; t < 4; ++t) acc[mt][t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-        constexpr int RING = 3, F = NS * MT, SLOTS = 4 * MT;
-        constexpr int R = RING < MT ? RING : MT;   // x fragments read ahead of their MFMAs
-        u32x4_t afr[4], bf[2][4];
-        auto read_a = [&](const u32x4_t* la, int f, int ring) {
-            afr[ring & 3] = la[a_lds_unit<BK>(16 * (f % MT) + i, 4 * (f / MT) + q)];
-        };
-        // fragments of sub-step s of the step whose buffer is fb
-        auto read_b = [&](u32x4_t dst[4], const u32x4_t* fb, int s) {
-#pragma unroll
-            for (int t = 0; t < 4; ++t) dst[t] = fb[((s * 4 + cw) * 4 + t) * 64 + lane];
-        };
-        asm volatile("s_barrier" ::: "memory");   // #0: the producers' first loads have landed
-        asm volatile("s_barrier" ::: "memory");   // #1: fragments of step 0 and x stage 0 are in LDS
-        read_b(bf[0], lds_f, 0);
-#pragma unroll
-        for (int f = 0; f < R; ++f) read_a(lds_a, f, f);
-
-        // one k step; Q = kt mod 6 as a compile-time constant (stage kt % 3, buffer kt & 1)
-        auto step = [&](auto qc) {
-            constexpr int Q = decltype(qc)::value;
-            constexpr int base = (F & 3) ? 2 * (Q & 1) : 0;   // (kt F) & 3, F is even
-            const u32x4_t* la = lds_a + (Q % S) * PC_A_UNITS;
-            const u32x4_t* la_next = lds_a + ((Q + 1) % S) * PC_A_UNITS;
-            const u32x4_t* fcur = lds_f + (Q & 1) * PC_F_UNITS;
-            const u32x4_t* fnext = lds_f + ((Q + 1) & 1) * PC_F_UNITS;
-            __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for (int s = 0; s < NS; ++s) {
-#pragma unroll
-                for (int slot = 0; slot < SLOTS; ++slot) {
-                    const int mt = slot >> 2, t = slot & 3, f = s * MT + mt;
-                    if (s == NS - 1 && slot == 4 * (MT - R)) {
-                        asm volatile("s_barrier" ::: "memory");
-                        read_b(bf[0], fnext, 0);            // first sub-step of the next step
-                    }
-                    if (t == 0) {
-                        const int fr = f + R;
-                        if (fr < F) read_a(la, fr, base + fr); else read_a(la_next, fr - F, base + fr);
-                    }
-                    mfma_16x16x32_v(acc[mt][t], afr[(base + f) & 3], bf[s][t]);
-                    if (s == 0 && slot == 0) read_b(bf[1], fcur, 1);   // second sub-step of this step
-                    __builtin_amdgcn_sched_barrier(0);
-                }
-            }
-        };
-        for (int kt = 0; kt < nk; kt += 6) {
-            step(IntC<0>{});
-            if (kt + 1 < nk) step(IntC<1>{});
-            if (kt + 2 < nk) step(IntC<2>{});
-            if (kt + 3 < nk) step(IntC<3>{});
-            if (kt + 4 < nk) step(IntC<4>{});
-            if (kt + 5 < nk) step(IntC<5>{});
-        }
-        // the accumulators were last written by MFMAs the compiler cannot see: wait out their latency
-        asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
-        // the tile's last LDS reads are done: the producers may start the next tile
-        asm volatile("s_barrier" ::: "memory");
-
-        // epilogue through a buffer resource that ends after the tile's last valid row: stores to
-        // padded rows fall outside it and are dropped
-        const rsrc_t ry = make_rsrc(P.y + row0 * (int64_t)P.N, (int64_t)rows * P.N * 2);
-        const int vy = (4 * q * P.N + n0 + col0) * 2;
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                u32x2_t v;
-                v[0] = pack_bf16_rne(acc[mt][0][r], acc[mt][1][r]);
-                v[1] = pack_bf16_rne(acc[mt][2][r], acc[mt][3][r]);
-                __builtin_amdgcn_raw_buffer_store_b64(v, ry, vy, (16 * mt + r) * P.N * 2, 0);
-            }
-    } else {
-        // ------------------------------------------------------------------ producer
-        const int64_t KN = (int64_t)P.K * P.N;
-        const rsrc_t rw = make_rsrc(P.w + g * (KN >> 1), KN >> 1);
-        const rsrc_t rs = make_rsrc(static_cast<const uint16_t*>(P.scale) + (int64_t)g * P.scale_rows * P.N,
-                                    (int64_t)P.scale_rows * P.N * 2);
-        const uint32_t per = (uint32_t)((P.K / P.scale_rows) >> 5);  // 32-k sub-steps per scale group
-        const uint32_t gmul = per == 1 ? 0u : 0xffffffffu / per + 1u;   // sub-step -> scale row as a multiply
-        auto scale_row = [&](uint32_t sub) { return gmul ? (int)__umulhi(sub, gmul) : (int)sub; };
-        // x rows through a buffer resource that ends after the last valid row (padded rows read as
-        // zeros).  Load instruction j covers rows 8j + (lane >> 3); position lane & 7 of a row
-        // holds chunk (lane & 7) ^ (row & 7), the swizzle a_lds_unit expects.
-        const rsrc_t rx = make_rsrc(P.x + row0 * (int64_t)P.K, (int64_t)rows * P.K * 2);
-        const int va = ((lane >> 3) * P.K + (((lane & 7) ^ (lane >> 3)) * 8)) * 2;
-        // packed tile: instruction j (8 per k step, this producer issues j = cw and cw + 4) brings rows
-        // 8j + (lane >> 3) into the 1 KB block j of the stage; the two 64-byte halves of the rows
-        // with odd (row >> 3) are swapped, so that the four q groups of a wavefront read from both
-        // halves of the banks
-        const int vb = (lane >> 3) * (P.N >> 1) + (((lane & 7) ^ (4 * (cw & 1))) * 16);
-        constexpr int NA = (2 * MT + 3) / 4;   // x load instructions per producer per step
-        constexpr int NI = NA + 3;             // + two packed-tile instructions + a quarter of the scales
-        static_assert(NI <= 63, "vmcnt range");
-        int ja[NA], ca[NA];
-#pragma unroll
-        for (int m = 0; m < NA; ++m) {
-            int j = cw + 4 * m;
-            if (4 * NA > 2 * MT) j = j % (2 * MT);   // repeat a block rather than issue fewer loads
-            ja[m] = j * 64;
-            ca[m] = 8 * j * P.K * 2;
-        }
-        const int cb = 8 * cw * (P.N >> 1) + (n0 >> 1);
-        const int kb_step = BK * (P.N >> 1);
-        const int cs = n0 * 2 + (cw & 1) * 256;    // scales: bytes [256 (cw & 1), +256) of row cw >> 1, 16 lanes
-        const int lane16 = lane * 16;
-        const bool s_lane = lane < 16;
-        // group kt: x stage kt+2 (LDS stage SA), packed and scale stage kt+3 (LDS stage SB)
-        auto issue_group = [&](int kt, int SA, int SB) {
-#pragma unroll
-            for (int m = 0; m < NA; ++m)
-                lds_load16(rx, lds_a + SA * PC_A_UNITS + ja[m], va, ca[m] + (kt + 2) * (BK * 2));
-#pragma unroll
-            for (int m = 0; m < 2; ++m)
-                lds_load16(rw, lds_b + SB * PC_B_UNITS + (cw + 4 * m) * 64, vb, cb + 32 * m * (P.N >> 1) + (kt + 3) * kb_step);
-            const int grow = scale_row((uint32_t)((kt + 3) * NS + (cw >> 1)));
-            if (s_lane) lds_load16(rs, lds_s + SB * PC_SC_UNITS + cw * 16, lane16, grow * (P.N * 2) + cs);
-        };
-        // perm selector: bytes 2h, 2h+1 of row a, then of row b (h = half of the dword this lane owns)
-        const uint32_t h2 = 2u * (uint32_t)(cw & 1);
-        uint32_t sel = h2 | ((h2 + 1u) << 8) | ((4u + h2) << 16) | ((5u + h2) << 24);
-        uint32_t mask = 0x0f0f0f0fu;
-        asm volatile("" : "+s"(mask), "+s"(sel));   // kept opaque so that each stays one SGPR operand
-        const int d = 16 * (cw >> 1) + i;            // dword column of this lane
-        const int unit = (d >> 2) ^ (4 * (q & 1));
-        // decode packed stage SB into fragment buffer fb
-        auto produce = [&](int SB, u32x4_t* fb) {
-            const uint32_t* t32 = reinterpret_cast<const uint32_t*>(lds_b + SB * PC_B_UNITS);
-            const uint16_t* sc16 = reinterpret_cast<const uint16_t*>(lds_s + SB * PC_SC_UNITS);
-#pragma unroll
-            for (int s = 0; s < NS; ++s) {
-                uint32_t r[8];
-#pragma unroll
-                for (int j = 0; j < 8; ++j) r[j] = t32[((32 * s + 8 * q + j) * 8 + unit) * 4 + (d & 3)];
-                const u32x2_t sc = *reinterpret_cast<const u32x2_t*>(sc16 + 256 * s + col0);
-                float m[4], z[4];
-                const float s0 = bf16_lo(sc[0]), s1 = bf16_hi(sc[0]), s2 = bf16_lo(sc[1]), s3 = bf16_hi(sc[1]);
-                m[0] = s0 * 512.f; m[1] = s1 * 512.f; m[2] = s2 * 512.f; m[3] = s3 * 512.f;
-                z[0] = -8.f * s0; z[1] = -8.f * s1; z[2] = -8.f * s2; z[3] = -8.f * s3;
-                // Written stage by stage over the four row pairs so that consecutive instructions are
-                // independent (a VALU result is not available to the very next instruction); the fences
-                // keep the scheduler from folding the stages back into per-element chains.
-                u32x4_t out[4];
-                uint32_t pr[4], lo[4], hi[4];
-                f32x2_t a02[4], b02[4], a13[4], b13[4];
-#pragma unroll
-                for (int p = 0; p < 4; ++p) pr[p] = __builtin_amdgcn_perm(r[2 * p + 1], r[2 * p], sel);   // a.b0 a.b1 b.b0 b.b1
-                __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                for (int p = 0; p < 4; ++p) lo[p] = pr[p] & mask;
-#pragma unroll
-                for (int p = 0; p < 4; ++p) hi[p] = pr[p] >> 4;
-                __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                for (int p = 0; p < 4; ++p) hi[p] &= mask;
-                __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                for (int p = 0; p < 4; ++p) {
-                    a02[p] = __builtin_amdgcn_cvt_pk_f32_fp8(lo[p], false);
-                    b02[p] = __builtin_amdgcn_cvt_pk_f32_fp8(lo[p], true);
-                }
-#pragma unroll
-                for (int p = 0; p < 4; ++p) {
-                    a13[p] = __builtin_amdgcn_cvt_pk_f32_fp8(hi[p], false);
-                    b13[p] = __builtin_amdgcn_cvt_pk_f32_fp8(hi[p], true);
-                }
-                __builtin_amdgcn_sched_barrier(0);
-                float wa[4][4], wb[4][4];
-#pragma unroll
-                for (int p = 0; p < 4; ++p) {
-                    wa[p][0] = fmaf(a02[p][0], m[0], z[0]); wb[p][0] = fmaf(b02[p][0], m[0], z[0]);
-                    wa[p][1] = fmaf(a13[p][0], m[1], z[1]); wb[p][1] = fmaf(b13[p][0], m[1], z[1]);
-                    wa[p][2] = fmaf(a02[p][1], m[2], z[2]); wb[p][2] = fmaf(b02[p][1], m[2], z[2]);
-                    wa[p][3] = fmaf(a13[p][1], m[3], z[3]); wb[p][3] = fmaf(b13[p][1], m[3], z[3]);
-                }
-                __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                for (int p = 0; p < 4; ++p)
-#pragma unroll
-                    for (int t = 0; t < 4; ++t) out[t][p] = pack_bf16_rne(wa[p][t], wb[p][t]);
-                __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                for (int t = 0; t < 4; ++t) fb[((s * 4 + cw) * 4 + t) * 64 + lane] = out[t];
-            }
-        };
-
-        // packed stage 0 and group -2 (x stage 0, packed stage 1)
-#pragma unroll
-        for (int m = 0; m < 2; ++m) lds_load16(rw, lds_b + (cw + 4 * m) * 64, vb, cb + 32 * m * (P.N >> 1));
-        if (s_lane) lds_load16(rs, lds_s + cw * 16, lane16, scale_row((uint32_t)(cw >> 1)) * (P.N * 2) + cs);
-        issue_group(-2, 0, 1);
-        asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");                  // #0
-        issue_group(-1, 1, 2);
-        produce(0, lds_f);
-        asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(NI) : "memory");   // #1
-        // producer step kt (alongside consumer step kt): group kt, fragments of step kt+1
-        auto pstep = [&](int kt, auto qc) {
-            constexpr int Q = decltype(qc)::value;
-            issue_group(kt, (Q + 2) % S, Q % S);
-            produce((Q + 1) % S, lds_f + ((Q + 1) & 1) * PC_F_UNITS);
-            asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(NI) : "memory");
-        };
-        for (int kt = 0; kt < nk; kt += 6) {
-            pstep(kt, IntC<0>{});
-            if (kt + 1 < nk) pstep(kt + 1, IntC<1>{});
-            if (kt + 2 < nk) pstep(kt + 2, IntC<2>{});
-            if (kt + 3 < nk) pstep(kt + 3, IntC<3>{});
-            if (kt + 4 < nk) pstep(kt + 4, IntC<4>{});
-            if (kt + 5 < nk) pstep(kt + 5, IntC<5>{});
-        }
-        // drain the loads that target stages past K (never read), then the tile-end barrier
-        asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
-    }
-}
-
-// ---------------------------------------------------------------------------------
 // Tile scheduler (role of GMMAntiquantProcess::Process,
 // grouped_gemm/op_kernel/grouped_matmul_antiquant.h:241-288).  Expert g with m_g rows
 // has ceil(m_g/16) row blocks, cut into the fewest chunks of <= MT_MAX blocks, as
@@ -1285,33 +993,25 @@ __device__ __forceinline__ void expert_chunks(int m, int& chunks, int& bpc) {
 //   GK_GENERAL  4 wavefronts of 64 columns, one workgroup per CU, tiles of up to 192 rows
 //   GK_SKINNY   the same tile routine with tiles of at most 32 rows and several workgroups per CU
 //               (decode-sized batches are HBM bound: more weight bytes in flight)
-//   GK_NARROW8  8 wavefronts of 32 columns, one workgroup per CU       } containers with
-//   GK_NARROW4  4 wavefronts of 32 columns, two workgroups per CU      } NarrowTraits
-//   GK_SPLIT    8 wavefronts, 4 that multiply and 4 that load and decode (int4)
-enum { GK_GENERAL = 0, GK_SKINNY = 1, GK_NARROW8 = 2, GK_NARROW4 = 3, GK_SPLIT = 4 };
-#ifndef MOE_INT4_PREFILL_KIND
-#define MOE_INT4_PREFILL_KIND GK_SPLIT
-#endif
+//   GK_NARROW8  8 wavefronts of 32 columns, one workgroup per CU (containers with NarrowTraits)
+enum { GK_GENERAL = 0, GK_SKINNY = 1, GK_NARROW8 = 2 };
 
 template <int FMT, int KIND>
 struct KernelCfg {
-    static constexpr bool NARROW = KIND == GK_NARROW8 || KIND == GK_NARROW4;
-    static constexpr int WAVES = (KIND == GK_NARROW8 || KIND == GK_SPLIT) ? 8 : 4;
+    static constexpr bool NARROW = KIND == GK_NARROW8;
+    static constexpr int WAVES = KIND == GK_NARROW8 ? 8 : 4;
     static constexpr int BN = NARROW ? 32 * WAVES : GM_BN;                       // columns per tile
-    static constexpr int WG_PER_CU = KIND == GK_SKINNY ? GM_SKINNY_WAVES : KIND == GK_NARROW4 ? 2 : 1;
-    static constexpr int STAGES = KIND == GK_NARROW4 ? 3 : 4;                    // narrow kernels only
-    static constexpr int CAPB = KIND == GK_SKINNY ? GM_SKINNY_BLOCKS : (KIND == GK_NARROW4 || KIND == GK_SPLIT) ? 10 : GM_MT_MAX;
+    static constexpr int WG_PER_CU = KIND == GK_SKINNY ? GM_SKINNY_WAVES : 1;
+    static constexpr int STAGES = 4;                                             // narrow kernel only
+    static constexpr int CAPB = KIND == GK_SKINNY ? GM_SKINNY_BLOCKS : GM_MT_MAX;
     static constexpr int fmt_mt_max() {
-        if constexpr (KIND == GK_SPLIT) return PC_CAPB;
-        else if constexpr (NARROW) return NarrowTraits<FMT, WAVES>::MT_MAX;
+        if constexpr (NARROW) return NarrowTraits<FMT, WAVES>::MT_MAX;
         else return BTraits<FMT>::MT_MAX;
     }
     static constexpr int MTM = CAPB < fmt_mt_max() ? CAPB : fmt_mt_max();        // row blocks per tile
     // 16-byte LDS units of the tile routine (the tile prefix array follows them)
     static constexpr int lds_units() {
-        if constexpr (KIND == GK_SPLIT)
-            return PC_LDS_UNITS;
-        else if constexpr (NARROW)
+        if constexpr (NARROW)
             return STAGES * (16 * CAPB * 8 + NarrowTraits<FMT, WAVES>::B_LDS_UNITS + NarrowTraits<FMT, WAVES>::SC_UNITS);
         else
             return 2 * 16 * CAPB * (BTraits<FMT>::BK / 8) + 2 * BTraits<FMT>::B_LDS_UNITS;
@@ -1321,9 +1021,7 @@ struct KernelCfg {
 template <int FMT, int MT, int KIND>
 __device__ __forceinline__ void run_tile(const GemmParams& P, u32x4_t* smem, int g, int64_t row0, int rows, int n0) {
     using C = KernelCfg<FMT, KIND>;
-    if constexpr (KIND == GK_SPLIT)
-        gemm_tile_pc_int4<MT>(P, smem, g, row0, rows, n0);
-    else if constexpr (C::NARROW)
+    if constexpr (C::NARROW)
         gemm_tile_narrow<FMT, MT, C::CAPB, C::WAVES, C::STAGES>(P, smem, g, row0, rows, n0);
     else
         gemm_tile<FMT, MT, C::CAPB>(P, smem, smem + 2 * 16 * C::CAPB * (BTraits<FMT>::BK / 8), g, row0, rows, n0);
@@ -1486,7 +1184,7 @@ static int launch_gemm_fmt(const moe_grouped_args* a, hipStream_t stream) {
     // device) are HBM bound: use the small-tile kernel.  An expert with more than 32 rows then
     // costs one pass over its weights per 32 rows.
     if (a->M <= 24 * a->G) return launch_gemm_kind<FMT, GK_SKINNY>(P, a, stream);
-    if constexpr (FMT == MOE_FMT_INT4) return launch_gemm_kind<FMT, MOE_INT4_PREFILL_KIND>(P, a, stream);
+    if constexpr (FMT == MOE_FMT_INT4) return launch_gemm_kind<FMT, GK_NARROW8>(P, a, stream);
     else return launch_gemm_kind<FMT, GK_GENERAL>(P, a, stream);
 }
 
