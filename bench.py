@@ -34,7 +34,7 @@ PEAK_BF16_TFLOPS = 2500.0    # MI355X dense bf16 MFMA, 2.5 PFLOP/s
 # launches), from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs of this script scaled by the
 # --copy-calibration copy (summary under profiles/): 3.27 GB read + 0.369 GB written.
 # Algorithmic bytes: 3.21 GB + 0.369 GB.
-INT4_GEMM_HBM_BYTES_PER_LAUNCH = 3.64e9
+INT4_GEMM_HBM_BYTES_PER_LAUNCH = 3.65e9
 
 
 def routed_counts(torch, tokens, experts, topk, gen, max_rows=None):
