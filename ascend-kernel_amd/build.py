@@ -47,6 +47,7 @@ def build_kernels(jobs: int = 4) -> str:
         if len(procs) >= jobs:
             _wait(procs)
     _wait(procs)
+    _check_accumulator_moves("moe_gemm.hip")
     _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", LIB])
     return LIB
 
@@ -63,6 +64,49 @@ def _check_resources(src: str, remarks: list) -> None:
             scratch = int(line.split("ScratchSize [bytes/lane]:")[1].split()[0])
             if scratch:
                 raise RuntimeError(f"{src}: {name} uses {scratch} bytes of scratch per lane")
+
+
+def _check_accumulator_moves(src: str) -> None:
+    """Second guard for the inline-asm MFMAs of the GEMM: inside the k loops nothing but MFMAs may
+    touch an accumulator register.  The compiler does not know the latency of the asm MFMAs, so a
+    copy it inserted there (live-range split, spill to another register) would read a value that
+    is not written yet.  Compiles the source to assembly and scans every innermost loop that
+    contains MFMAs for v_accvgpr_read/write of a register one of those MFMAs accumulates into."""
+    import re
+    import tempfile
+
+    with tempfile.TemporaryDirectory() as tmp:
+        asm = os.path.join(tmp, src + ".s")
+        cmd = [HIPCC, *HIP_FLAGS, "-x", "hip", "-I", os.path.join(ROOT, "include"), "-I", CSRC, "-S",
+               "--cuda-device-only", os.path.join(CSRC, src), "-o", asm]
+        print("+", " ".join(cmd), flush=True)
+        subprocess.run(cmd, check=True, stderr=subprocess.DEVNULL)
+        text = open(asm).read()
+    for m in re.finditer(r"^(\w*grouped_gemm_kernel\w*):", text, re.M):
+        lines = text[m.end():text.index("s_endpgm", m.end())].split("\n")
+        labels = {mm.group(1): i for i, l in enumerate(lines) if (mm := re.match(r"^(\.LBB\d+_\d+):", l))}
+        loops = []
+        for i, l in enumerate(lines):
+            mm = re.search(r"s_cbranch_\w+ (\.LBB\d+_\d+)", l)
+            if mm and labels.get(mm.group(1), i) < i:
+                loops.append((labels[mm.group(1)], i))
+        for s0, e0 in loops:
+            if any(s1 >= s0 and e1 <= e0 and (s1, e1) != (s0, e0) for s1, e1 in loops):
+                continue  # not innermost
+            body = lines[s0:e0 + 1]
+            accs = set()
+            for l in body:
+                mm = re.search(r"v_mfma\S+ ([av])\[(\d+):(\d+)\]", l)
+                if mm:
+                    if mm.group(1) == "v":
+                        raise RuntimeError(f"{src}: {m.group(1)} accumulates in VGPRs; moves cannot be checked")
+                    accs.update(range(int(mm.group(2)), int(mm.group(3)) + 1))
+            for l in body:
+                mm = re.search(r"v_accvgpr_(read|write)_b32 (\S+), (\S+)", l)
+                if mm and accs:
+                    reg = mm.group(3) if mm.group(1) == "read" else mm.group(2)
+                    if int(reg.strip("a,")) in accs:
+                        raise RuntimeError(f"{src}: {m.group(1)} moves accumulator {reg} inside a k loop: {l.strip()}")
 
 
 def _wait(procs):
