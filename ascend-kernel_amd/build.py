@@ -66,12 +66,17 @@ def _check_resources(src: str, remarks: list) -> None:
                 raise RuntimeError(f"{src}: {name} uses {scratch} bytes of scratch per lane")
 
 
+# instructions that must separate an ordinary write of an accumulator register from an MFMA on it
+ACC_WRITE_GAP = 8
+
+
 def _check_accumulator_moves(src: str) -> None:
     """Second guard for the inline-asm MFMAs of the GEMM: inside the k loops nothing but MFMAs may
     touch an accumulator register.  The compiler does not know the latency of the asm MFMAs, so a
     copy it inserted there (live-range split, spill to another register) would read a value that
     is not written yet.  Compiles the source to assembly and scans every innermost loop that
-    contains MFMAs for v_accvgpr_read/write of a register one of those MFMAs accumulates into."""
+    contains MFMAs for any other instruction that names a register one of those MFMAs accumulates
+    into (accumulators may be AGPRs or VGPRs)."""
     import re
     import tempfile
 
@@ -82,6 +87,15 @@ def _check_accumulator_moves(src: str) -> None:
         print("+", " ".join(cmd), flush=True)
         subprocess.run(cmd, check=True, stderr=subprocess.DEVNULL)
         text = open(asm).read()
+    def regs(tok):
+        out = []
+        for mm in re.finditer(r"\b([av])\[(\d+):(\d+)\]|\b([av])(\d+)\b", tok):
+            if mm.group(1):
+                out += [(mm.group(1), r) for r in range(int(mm.group(2)), int(mm.group(3)) + 1)]
+            else:
+                out.append((mm.group(4), int(mm.group(5))))
+        return out
+
     for m in re.finditer(r"^(\w*grouped_gemm_kernel\w*):", text, re.M):
         lines = text[m.end():text.index("s_endpgm", m.end())].split("\n")
         labels = {mm.group(1): i for i, l in enumerate(lines) if (mm := re.match(r"^(\.LBB\d+_\d+):", l))}
@@ -93,20 +107,32 @@ def _check_accumulator_moves(src: str) -> None:
         for s0, e0 in loops:
             if any(s1 >= s0 and e1 <= e0 and (s1, e1) != (s0, e0) for s1, e1 in loops):
                 continue  # not innermost
-            body = lines[s0:e0 + 1]
+            body = [l.split(";")[0].strip() for l in lines[s0:e0 + 1]]
             accs = set()
             for l in body:
-                mm = re.search(r"v_mfma\S+ ([av])\[(\d+):(\d+)\]", l)
-                if mm:
-                    if mm.group(1) == "v":
-                        raise RuntimeError(f"{src}: {m.group(1)} accumulates in VGPRs; moves cannot be checked")
-                    accs.update(range(int(mm.group(2)), int(mm.group(3)) + 1))
+                if l.startswith("v_mfma"):
+                    accs.update(regs(l.split(None, 1)[1].split(",")[0]))
             for l in body:
-                mm = re.search(r"v_accvgpr_(read|write)_b32 (\S+), (\S+)", l)
-                if mm and accs:
-                    reg = mm.group(3) if mm.group(1) == "read" else mm.group(2)
-                    if int(reg.strip("a,")) in accs:
-                        raise RuntimeError(f"{src}: {m.group(1)} moves accumulator {reg} inside a k loop: {l.strip()}")
+                if not accs or not l or l.startswith("v_mfma") or l.endswith(":") or l.startswith("."):
+                    continue
+                parts = l.split(None, 1)
+                if len(parts) == 2 and any(r in accs for r in regs(parts[1])):
+                    raise RuntimeError(f"{src}: {m.group(1)} touches an accumulator inside a k loop: {l}")
+        # Outside the loops too: an ordinary write of an MFMA's accumulator input needs wait states
+        # before that MFMA (the compiler inserts them only for MFMAs it can see), e.g. zeros
+        # re-materialized right in front of a peeled first k step.
+        code = [l.split(";")[0].strip() for l in lines]
+        code = [l for l in code if l and not l.endswith(":") and not l.startswith(".")]
+        for i, l in enumerate(code):
+            if not l.startswith("v_mfma"):
+                continue
+            accs = set(regs(l.split(None, 1)[1].split(",")[0]))
+            for prev in code[max(0, i - ACC_WRITE_GAP):i]:
+                parts = prev.split(None, 1)
+                if prev.startswith("v_mfma") or prev.startswith("s_") or len(parts) < 2:
+                    continue
+                if any(r in accs for r in regs(parts[1].split(",")[0])):
+                    raise RuntimeError(f"{src}: {m.group(1)} writes an accumulator right before its MFMA: {prev}")
 
 
 def _wait(procs):

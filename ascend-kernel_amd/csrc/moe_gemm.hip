@@ -14,6 +14,8 @@
 // L2.  A workgroup has 4 wavefronts; every wavefront owns 64 of the 256 columns for
 // ALL rows of the tile, so each weight element is dequantized exactly once per tile.
 // x tiles go through a double-buffered, XOR-swizzled LDS tile shared by the 4 waves.
+// (Prefill on the int4 container uses a variant with 8 wavefronts and LDS-direct loads, see
+// gemm_tile_pair_int4.)
 //
 // MFMA: v_mfma_f32_16x16x32_bf16.  Lane l = 16*q + i holds, for A, row i and
 // k = 8q..8q+7 of the 16x32 block; for B, column i and the same k; for the result,
@@ -67,6 +69,12 @@ __device__ __forceinline__ u32x4_t ldg_b128(rsrc_t r, int voff, int soff) {
 // which waits out the MFMA latency first.
 __device__ __forceinline__ void mfma_16x16x32(f32x4_t& acc, const u32x4_t& a, const u32x4_t& b) {
     asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
+}
+
+// Same with the accumulator in ordinary VGPRs.  A kernel that uses no AGPRs at all may use
+// the whole unified register file as VGPRs (otherwise the compiler splits it in two halves).
+__device__ __forceinline__ void mfma_16x16x32_v(f32x4_t& acc, const u32x4_t& a, const u32x4_t& b) {
+    asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+v"(acc) : "v"(a), "v"(b));
 }
 
 // Ties a value to the chain of volatile asm statements (the MFMAs): whatever is computed
@@ -682,297 +690,294 @@ __device__ __forceinline__ void lds_load16(rsrc_t r, const u32x4_t* dst, int vof
     __builtin_amdgcn_raw_ptr_buffer_load_lds(r, MOE_LDS_PTR(const_cast<u32x4_t*>(dst)), 16, voff, soff, 0, 0);
 }
 
-template <int N>
-struct IntC { static constexpr int value = N; };
-
 // ---------------------------------------------------------------------------------
-// Prefill tile routine with two wavefronts per SIMD ("narrow" wavefronts: 32 columns each).
+// Prefill tile routine for int4 with two wavefronts per SIMD that split the k range.
 //
 // A single wavefront issues at most one instruction every ~5 cycles whatever its kind, and an
-// MFMA holds the SIMD's vector issue port for about 8 of its 16 cycles; with one wavefront
+// MFMA holds the SIMD's vector issue port for about 8 of its 16 cycles: with one wavefront
 // per SIMD the decode instructions and the MFMAs of a k step add up instead of overlapping.
-// Here each wavefront owns 32 columns for all rows of the tile (two MFMAs per x fragment), so
-// that a CU holds 8 of them and every weight element is still decoded exactly once per tile.
-// The NW = 8 wavefronts of the workgroup share a tile of 256 columns.
+// Here the workgroup has 8 wavefronts.  Wavefront wv owns the 64 columns of group wv & 3 for
+// all rows of the tile (4 MFMAs per x fragment), but only one of the two 32-k sub-steps of
+// every 64-k step: the pair (wv, wv + 4) shares a SIMD and accumulates two partial sums that
+// are added once per tile through LDS.  Every weight element is still decoded exactly once
+// per tile, a lane decodes 4 nibbles of a dword at a time (2.5 VALU instructions per
+// element), and each wavefront reads half of the x fragments.
+//
+// Each wavefront alternates a decode phase (its sub-step of the packed stage -> 4 bf16 B
+// fragments in registers) and an MFMA phase.  The phases of a pair are kept in opposition by
+// the position of the step's barrier: the wavefronts of sub-step 0 take it after their MFMA
+// phase, those of sub-step 1 half way through their decode phase, so that after every
+// barrier one wavefront of the SIMD starts decoding while the other starts multiplying.
 //
 // Everything the k loop consumes -- x tile, packed weight tile, scales -- is brought in by
-// LDS-direct loads into a ring of S stages per operand.  Schedule of k step kt (two 32-k
-// sub-steps, 4 MT MFMAs per wavefront):
-//   first MFMA slots   issue the loads of x stage kt+S-1 and of weight/scale stage kt+S
-//                      (weights run one stage ahead of x because their dwords are pulled
-//                      into registers a step before they are decoded);
-//   whole step         MFMAs on x stage kt, decode of the next sub-step, this lane's packed
-//                      dwords of stage kt+1 read from LDS as soon as the registers holding
-//                      stage kt's have been decoded;
-//   R fragments before the end   wait until this wavefront's own loads issued S-2 steps ago
-//                      (x stage kt+1, weight stage kt+2) have landed, then the step's only
-//                      barrier; the x fragment reads that follow already belong to step kt+1,
-//                      so no LDS latency is exposed at the step boundary.
-// A stage is overwritten by loads issued after the barrier that follows its last read.
-// vmcnt counts this wavefront's loads in order; every wavefront issues the same number NI
-// of them per step (waves without a row block of their own repeat one), so "at most
-// (S-2) NI outstanding" means exactly "the group issued S-2 steps ago has landed".
+// LDS-direct loads into a ring of 5 stages.  The loads of stage kt+4 (it replaces stage kt-1,
+// last read before barrier kt-1) and the LDS reads of the packed dwords of stage kt+1 are
+// spread between the MFMAs of step kt; before barrier kt each wavefront waits until its own
+// loads of stage kt+2 have landed.  vmcnt counts a wavefront's loads in order and every
+// wavefront issues the same number NI of them per step (waves without a row block of their
+// own repeat one), so "at most 2 NI outstanding" means exactly that.
 //
-// int4 layout.  Wavefront wv handles, of the tile's dword columns, the 16 starting at
-// 16 (wv >> 2), and of each dword the byte np = wv & 3: lane (i, q) owns columns
-// 8 (16 (wv >> 2) + i) + 2 np + {0, 1} (MFMA t = the nibble of that byte) for its 8 k rows.
-// Decode of a k-row pair (a, b): v_perm gathers the two bytes, the low nibbles (& 0x0f0f)
-// and high nibbles (>> 4 & 0x0f0f) are bytes 0x00..0x0f, which read as OCP e4m3 are
-// exactly q / 512 -- v_cvt_pk_f32_fp8 converts both rows at once -- and one fma per element
-// applies 512 * scale and the zero point: q s - 8 s = (q - 8) s exactly.
+// Decode of a k-row pair (a, b) of one dword column: v_perm gathers the two bytes of each row
+// this lane owns, the low nibbles (& 0x0f0f0f0f) and high nibbles (>> 4 & 0x0f0f0f0f) are bytes
+// 0x00..0x0f, which read as OCP e4m3 are exactly q / 512 -- v_cvt_pk_f32_fp8 converts two at
+// once -- and one fma per element applies 512 * scale and the zero point:
+// q s - 8 s = (q - 8) s exactly.
 // ---------------------------------------------------------------------------------
-template <int FMT, int NW>
-struct NarrowTraits;
+constexpr int PAIR_CAPB = 10;                         // x stages hold 160 rows
+constexpr int PAIR_MT_MAX = 10;
+constexpr int PAIR_A_UNITS = 16 * PAIR_CAPB * 8;      // 16-byte units of one x stage
+constexpr int PAIR_B_UNITS = 64 * 8;                  // packed int4 tile of one k step: 64 rows of 128 bytes
+constexpr int PAIR_SC_UNITS = 64;                     // 2 scale rows (one per sub-step) of 256 bf16
+constexpr int PAIR_STAGES = 5;
+constexpr int PAIR_LDS_UNITS = PAIR_STAGES * (PAIR_A_UNITS + PAIR_B_UNITS + PAIR_SC_UNITS);
 
-template <int NW>
-struct NarrowTraits<MOE_FMT_INT4, NW> {
-    static_assert(NW == 8, "the LDS layout of the packed tile is written for 8 wavefronts (128-byte rows)");
-    static constexpr int MT_MAX = 10;            // 160 rows: the largest tile that keeps every value in registers
-    static constexpr int ROW_UNITS = NW;         // 16-byte chunks of one packed row of the tile (32 NW columns)
-    static constexpr int B_LDS_UNITS = 64 * ROW_UNITS;   // packed tile of one k step: 64 rows
-    static constexpr int SC_UNITS = 8 * NW;      // scale block of one k step: 2 rows (one per sub-step) of 32 NW bf16
-    struct Ctx {
-        rsrc_t rw, rs;
-        int N, n0, i, q, wv, dg, np;
-        uint32_t gmul, sel, mask;   // scale-row multiplier (see BCtx), v_perm selector, 0x0f0f
-    };
-    struct Raw {
-        uint32_t r[2][8];
-        uint32_t sc[2];
-    };
-    __device__ static __forceinline__ int col(const Ctx& c, int t) { return 8 * (16 * c.dg + c.i) + 2 * c.np + t; }
-    __device__ static __forceinline__ void init(Ctx& c, const GemmParams& P, int g, int n0) {
-        const int tid = threadIdx.x, lane = tid & 63;
-        c.N = P.N; c.n0 = n0;
-        c.i = lane & 15; c.q = lane >> 4; c.wv = __builtin_amdgcn_readfirstlane(tid >> 6);
-        c.dg = c.wv >> 2; c.np = c.wv & 3;
-        const int64_t KN = (int64_t)P.K * P.N;
-        c.rw = make_rsrc(P.w + g * (KN >> 1), KN >> 1);
-        c.rs = make_rsrc(static_cast<const uint16_t*>(P.scale) + (int64_t)g * P.scale_rows * P.N,
-                         (int64_t)P.scale_rows * P.N * 2);
-        const uint32_t per = (uint32_t)((P.K / P.scale_rows) >> 5);  // sub-steps per scale group
-        c.gmul = per == 1 ? 0u : 0xffffffffu / per + 1u;
-        c.sel = 0x0c0c0000u | ((4u + (uint32_t)c.np) << 8) | (uint32_t)c.np;   // byte np of a, byte np of b, 0, 0
-        c.mask = 0x0f0fu;
-        asm volatile("" : "+s"(c.mask));   // kept opaque so that it stays one SGPR operand
-    }
-    // LDS-direct load of the packed tile, one instruction per wavefront and k step: 8 consecutive
-    // LDS rows starting at row 8 wv, lane l at byte 16 l of that block.  The four q groups of a
-    // wavefront read the same dword columns of four different rows at once; the two 64-byte
-    // halves of the rows with odd (row >> 3) are swapped to spread them over the banks.
-    __device__ static __forceinline__ int dma_voff(const Ctx& c, int lane) {
-        return (lane >> 3) * (c.N >> 1) + (((lane & 7) ^ (4 * (c.wv & 1))) * 16);
-    }
-    __device__ static __forceinline__ int dma_soff(const Ctx& c) { return (64 / NW) * c.wv * (c.N >> 1) + (c.n0 >> 1); }
-    __device__ static __forceinline__ int scale_row(const Ctx& c, uint32_t sub) {
-        return c.gmul ? (int)__umulhi(sub, c.gmul) : (int)sub;
-    }
-    __device__ static __forceinline__ void load_sub(Raw& raw, const Ctx& c, int s, const u32x4_t* tile) {
-        const uint32_t* t32 = reinterpret_cast<const uint32_t*>(tile);
-        const int d = 16 * c.dg + c.i;  // dword of the row
-        const int unit = (d >> 2) ^ (4 * (c.q & 1));
-#pragma unroll
-        for (int j = 0; j < 8; ++j) raw.r[s][j] = t32[((32 * s + 8 * c.q + j) * 8 + unit) * 4 + (d & 3)];
-    }
-    __device__ static __forceinline__ void load_scale(Raw& raw, const Ctx& c, int s, const u32x4_t* stile) {
-        raw.sc[s] = *reinterpret_cast<const uint32_t*>(reinterpret_cast<const uint16_t*>(stile) + 32 * NW * s + col(c, 0));
-    }
-    struct Dq {
-        float m[2], z[2];
-        uint32_t pr;   // gathered bytes of the current row pair
-        __device__ __forceinline__ void prep(const Raw& raw, int s) {
-            const uint32_t sc = raw.sc[s];
-            const float s0 = bf16_lo(sc), s1 = bf16_hi(sc);
-            m[0] = s0 * 512.f; m[1] = s1 * 512.f;
-            z[0] = -8.f * s0; z[1] = -8.f * s1;
-        }
-        // half unit: nibble t of row pair p -> dword p of the fragment of MFMA t
-        __device__ __forceinline__ void unit(const Raw& raw, const Ctx& c, int s, int p, int t, u32x4_t out[2]) {
-            if (t == 0) pr = __builtin_amdgcn_perm(raw.r[s][2 * p + 1], raw.r[s][2 * p], c.sel);
-            const uint32_t nib = (t == 0 ? pr : pr >> 4) & c.mask;
-            const f32x2_t f = __builtin_amdgcn_cvt_pk_f32_fp8(nib, false);
-            out[t][p] = pack_bf16_rne(fmaf(f[0], m[t], z[t]), fmaf(f[1], m[t], z[t]));
-        }
-    };
-};
-
-// NW wavefronts per workgroup, S stages, x buffers for CAPB row blocks.
-template <int FMT, int MT, int CAPB, int NW, int S>
-__device__ __forceinline__ void gemm_tile_narrow(const GemmParams& P, u32x4_t* smem, int g, int64_t row0, int rows, int n0) {
-    using T = NarrowTraits<FMT, NW>;
-    constexpr int BK = 64, NS = 2;
-    static_assert(S == 3 || S == 4, "ring of 3 or 4 stages");
-    constexpr int A_UNITS = 16 * CAPB * 8, B_UNITS = T::B_LDS_UNITS, SC_UNITS = T::SC_UNITS;
+template <int MT>
+__device__ __forceinline__ void gemm_tile_pair_int4(const GemmParams& P, u32x4_t* smem, int g, int64_t row0, int rows, int n0) {
+    constexpr int BK = 64, S = PAIR_STAGES;
     u32x4_t* lds_a = smem;
-    u32x4_t* lds_b = lds_a + S * A_UNITS;
-    u32x4_t* lds_s = lds_b + S * B_UNITS;
+    u32x4_t* lds_b = lds_a + S * PAIR_A_UNITS;
+    u32x4_t* lds_s = lds_b + S * PAIR_B_UNITS;
 
-    const int lane = threadIdx.x & 63;
-    typename T::Ctx c;
-    T::init(c, P, g, n0);
-    typename T::Dq dq;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int i = lane & 15, q = lane >> 4;
+    const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int cw = wv & 3;                                    // column group: 64 columns
+    // the sub-step of every step this wavefront owns.  The SIMD's issue arbitration favours the
+    // wavefront in the lower slot (wv < 4); measured, the pair runs 20 % faster when that one takes
+    // the role whose barrier sits inside the decode phase
+    const int h = 1 - (wv >> 2);
+    const int col0 = 128 * (cw >> 1) + 8 * i + 4 * (cw & 1);  // this lane's 4 columns (MFMA t = column col0 + t)
+    const int nk = P.K / BK;
 
+    const int64_t KN = (int64_t)P.K * P.N;
+    const rsrc_t rw = make_rsrc(P.w + g * (KN >> 1), KN >> 1);
+    const rsrc_t rs = make_rsrc(static_cast<const uint16_t*>(P.scale) + (int64_t)g * P.scale_rows * P.N,
+                                (int64_t)P.scale_rows * P.N * 2);
+    const uint32_t per = (uint32_t)((P.K / P.scale_rows) >> 5);      // 32-k sub-steps per scale group
+    const uint32_t gmul = per == 1 ? 0u : 0xffffffffu / per + 1u;   // sub-step -> scale row as a multiply
+    auto scale_row = [&](uint32_t sub) { return gmul ? (int)__umulhi(sub, gmul) : (int)sub; };
     // x rows through a buffer resource that ends after the last valid row (padded rows read as
     // zeros).  Load instruction j covers rows 8j + (lane >> 3); position lane & 7 of a row
     // holds chunk (lane & 7) ^ (row & 7), the swizzle a_lds_unit expects.
     const rsrc_t rx = make_rsrc(P.x + row0 * (int64_t)P.K, (int64_t)rows * P.K * 2);
     const int va = ((lane >> 3) * P.K + (((lane & 7) ^ (lane >> 3)) * 8)) * 2;
-    const int vb = T::dma_voff(c, lane);
-
-    constexpr int NA = (2 * MT + NW - 1) / NW;   // x load instructions per wavefront per step
-    constexpr int NI = NA + 2;                   // + one packed-tile instruction + this wavefront's share of the scales
-    constexpr int SLOTS = 2 * MT;                // MFMAs per sub-step
-    constexpr int LEAD = S - 1;                  // x stage loaded during step kt: kt + LEAD; weights: kt + LEAD + 1
-    static_assert((S - 2) * NI <= 63, "vmcnt range");
-
-    // Loads.  Everything that does not change from step to step is computed here; per load the
-    // loop only adds a running k offset to a per-tile constant.  Stage numbers are compile-time
-    // constants (the k loop is unrolled).
-    int ja[NA], ca[NA];                    // x block of the m-th x load: LDS unit offset and byte offset of its rows
+    // packed tile: instruction wv brings rows 8 wv + (lane >> 3) into the 1 KB block wv of the stage;
+    // the two 64-byte halves of the rows with odd (row >> 3) are swapped, so that the four q groups
+    // of a wavefront read from both halves of the banks
+    const int vb = (lane >> 3) * (P.N >> 1) + (((lane & 7) ^ (4 * (wv & 1))) * 16);
+    constexpr int NA = (2 * MT + 7) / 8;   // x load instructions per wavefront per step
+    constexpr int NI = NA + 2;             // + one packed-tile instruction + an eighth of the scales
+    int ja[NA], ca[NA];
 #pragma unroll
     for (int m = 0; m < NA; ++m) {
-        int j = c.wv + NW * m;
-        if (NW * NA > 2 * MT) j = j % (2 * MT);   // repeat a block rather than issue fewer loads
+        int j = wv + 8 * m;
+        if (8 * NA > 2 * MT) j = j % (2 * MT);   // repeat a block rather than issue fewer loads
         ja[m] = j * 64;
         ca[m] = 8 * j * P.K * 2;
     }
-    const int cb = T::dma_soff(c);
+    const int cb = 8 * wv * (P.N >> 1) + (n0 >> 1);
     const int kb_step = BK * (P.N >> 1);
-    // scales: the stage's block is 2 rows of 64 NW bytes; wavefront wv fetches 128 bytes of it with
-    // its first 8 lanes
-    constexpr int SEGS = NW / 2;                           // 128-byte segments per scale row of the tile
-    const int srow = c.wv / SEGS;
-    const int cs = n0 * 2 + (c.wv % SEGS) * 128;
+    const int cs = n0 * 2 + (wv & 3) * 128;    // scales: bytes [128 (wv & 3), +128) of row wv >> 2, 8 lanes
     const int lane16 = lane * 16;
     const bool s_lane = lane < 8;
-    // m-th load of the group issued during step kt: x stage kt+LEAD (LDS stage SA), weight and
-    // scale stage kt+LEAD+1 (LDS stage SB)
-    auto issue = [&](int m, int kt, int SA, int SB) {
+    // m-th load of group kt (stage kt+4 of x, packed tile and scales), into LDS stage ST
+    auto issue = [&](int m, int kt, int ST) {
         if (m < NA) {
-            lds_load16(rx, lds_a + SA * A_UNITS + ja[m], va, ca[m] + (kt + LEAD) * (BK * 2));
+            lds_load16(rx, lds_a + ST * PAIR_A_UNITS + ja[m], va, ca[m] + (kt + 4) * (BK * 2));
         } else if (m == NA) {
-            lds_load16(c.rw, lds_b + SB * B_UNITS + c.wv * 64, vb, cb + (kt + LEAD + 1) * kb_step);
+            lds_load16(rw, lds_b + ST * PAIR_B_UNITS + wv * 64, vb, cb + (kt + 4) * kb_step);
         } else {
-            const int grow = T::scale_row(c, (uint32_t)((kt + LEAD + 1) * NS + srow));
-            if (s_lane) lds_load16(c.rs, lds_s + SB * SC_UNITS + c.wv * 8, lane16, grow * (P.N * 2) + cs);
+            const int grow = scale_row((uint32_t)((kt + 4) * 2 + (wv >> 2)));
+            if (s_lane) lds_load16(rs, lds_s + ST * PAIR_SC_UNITS + wv * 8, lane16, grow * (P.N * 2) + cs);
         }
     };
+    auto issue_group = [&](int kt, int ST) {
+#pragma unroll
+        for (int m = 0; m < NI; ++m) issue(m, kt, ST);
+    };
 
-    f32x4_t acc[MT][2];
+    // perm selector: bytes 2hh, 2hh+1 of row a, then of row b (hh = half of the dword this lane owns)
+    const uint32_t h2 = 2u * (uint32_t)(cw & 1);
+    uint32_t sel = h2 | ((h2 + 1u) << 8) | ((4u + h2) << 16) | ((5u + h2) << 24);
+    uint32_t mask = 0x0f0f0f0fu;
+    asm volatile("" : "+s"(mask), "+s"(sel));   // kept opaque so that each stays one SGPR operand
+    const int d = 16 * (cw >> 1) + i;            // dword column of this lane
+    const int unit = (d >> 2) ^ (4 * (q & 1));
+
+    // The accumulators are zeroed by asm so that the compiler cannot re-materialize the zeros
+    // right in front of the first MFMA that accumulates into them: a VALU write of an MFMA's
+    // accumulator input needs wait states the compiler only inserts for MFMAs it can see.
+    f32x4_t acc[MT][4];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-        for (int t = 0; t < 2; ++t) acc[mt][t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-
-    typename T::Raw raw;
-    const int nk = P.K / BK;
-    constexpr int RING = 3, F = NS * MT;
+        for (int t = 0; t < 4; ++t)
+            asm volatile("v_mov_b32 %0, 0\n\tv_mov_b32 %1, 0\n\tv_mov_b32 %2, 0\n\tv_mov_b32 %3, 0"
+                         : "=v"(acc[mt][t][0]), "=v"(acc[mt][t][1]), "=v"(acc[mt][t][2]), "=v"(acc[mt][t][3]));
+    u32x4_t bf[4], afr[4];
+    constexpr int RING = 3;
     constexpr int R = RING < MT ? RING : MT;   // x fragments read ahead of their MFMAs
 
-    __syncthreads();  // every wavefront is done with the previous tile (its loads have been drained)
-    // weight stage 0 first, then the groups the steady state would have issued before step 0
-#pragma unroll
-    for (int m = NA; m < NI; ++m) issue(m, -LEAD - 1, 0, 0);
-#pragma unroll
-    for (int kt = -LEAD; kt < 0; ++kt)
-#pragma unroll
-        for (int m = 0; m < NI; ++m) issue(m, kt, (kt + LEAD) % S, (kt + LEAD + 1) % S);
-    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"((S - 2) * NI) : "memory");   // x 0, weights 0 and 1 are in LDS
+    // groups -4 .. -1: stages 0 .. 3; stages 0 and 1 must have landed before the first barrier
+    issue_group(-4, 0);
+    issue_group(-3, 1);
+    issue_group(-2, 2);
+    issue_group(-1, 3);
+    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(2 * NI) : "memory");
 
+    // this lane's packed dwords and scales of its sub-step of LDS stage st
+    uint32_t r[8];
+    u32x2_t sc;
+    auto read_raw = [&](int st) {
+        const uint32_t* t32 = reinterpret_cast<const uint32_t*>(lds_b + st * PAIR_B_UNITS);
+        const uint16_t* sc16 = reinterpret_cast<const uint16_t*>(lds_s + st * PAIR_SC_UNITS);
 #pragma unroll
-    for (int s = 0; s < NS; ++s) {
-        T::load_sub(raw, c, s, lds_b);
-        T::load_scale(raw, c, s, lds_s);
-    }
-    u32x4_t bf[2][2];
-    dq.prep(raw, 0);
-#pragma unroll
-    for (int p = 0; p < 4; ++p)
-#pragma unroll
-        for (int t = 0; t < 2; ++t) dq.unit(raw, c, 0, p, t, bf[0]);
-
-    // ring of 4 x fragments; fragment f of step kt lives in afr[(kt F + f) & 3], F is even
-    u32x4_t afr[4];
-    auto read_a = [&](const u32x4_t* la, int f, int ring) {
-        afr[ring & 3] = la[a_lds_unit<BK>(16 * (f % MT) + c.i, 4 * (f / MT) + c.q)];
+        for (int j = 0; j < 8; ++j) r[j] = t32[((32 * h + 8 * q + j) * 8 + unit) * 4 + (d & 3)];
+        sc = *reinterpret_cast<const u32x2_t*>(sc16 + 256 * h + col0);
     };
-#pragma unroll
-    for (int f = 0; f < R; ++f) read_a(lds_a, f, f);
+    read_raw(0);
 
-    // one k step; Q = kt mod (unroll factor) as a compile-time constant
-    auto step = [&](int kt, auto qc) {
-        constexpr int Q = decltype(qc)::value;
-        constexpr int base = (F & 3) ? 2 * (Q & 1) : 0;   // (kt F) & 3; the unroll factor is even
-        const u32x4_t* la = lds_a + (Q % S) * A_UNITS;
-        const u32x4_t* la_next = lds_a + ((Q + 1) % S) * A_UNITS;
-        const u32x4_t* btile = lds_b + ((Q + 1) % S) * B_UNITS;
-        const u32x4_t* stile = lds_s + ((Q + 1) % S) * SC_UNITS;
-        __builtin_amdgcn_sched_barrier(0);
+    // One data step; st = step mod 5 is its LDS stage, sn the next one, sl the stage this step's loads
+    // go to (wave-uniform).
+    auto step = [&](int kt, int st, int sn, int sl) {
+        const u32x4_t* la = lds_a + st * PAIR_A_UNITS;
+        // ---- decode phase: this wavefront's sub-step of the packed stage -> bf[0..3]
+        float m[4], z[4];
+        const float s0 = bf16_lo(sc[0]), s1 = bf16_hi(sc[0]), s2 = bf16_lo(sc[1]), s3 = bf16_hi(sc[1]);
+        m[0] = s0 * 512.f; m[1] = s1 * 512.f; m[2] = s2 * 512.f; m[3] = s3 * 512.f;
+        z[0] = -8.f * s0; z[1] = -8.f * s1; z[2] = -8.f * s2; z[3] = -8.f * s3;
+        // Written stage by stage over two row pairs at a time so that consecutive instructions are
+        // independent (a VALU result is not available to the very next instruction); the fences
+        // keep the scheduler from folding the stages back into per-element chains.
 #pragma unroll
-        for (int s = 0; s < NS; ++s) {
-            const int sn = (s + 1) % NS;                 // sub-step being decoded
-            u32x4_t* bcur = bf[s & 1];
-            u32x4_t* bnxt = bf[(s + 1) & 1];
-#pragma unroll
-            for (int slot = 0; slot < SLOTS; ++slot) {
-                const int mt = slot >> 1, t = slot & 1, f = s * MT + mt;
-                if (s == NS - 1 && slot == 2 * (MT - R))
-                    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"((S - 2) * NI) : "memory");
-                if (t == 0) {
-                    const int fr = f + R;
-                    if (fr < F) read_a(la, fr, base + fr); else read_a(la_next, fr - F, base + fr);
+        for (int p0 = 0; p0 < 4; p0 += 2) {
+            if (p0 == 2) {
+                if (h == 1) {
+                    // barrier kt-1 for the wavefronts that own sub-step 1, half way through their decode
+                    // (not in the tile's first step: the barrier of the prologue stands for it); x stage
+                    // kt is visible behind it
+                    if (kt > 0) asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(2 * NI) : "memory");
                 }
-                mfma_16x16x32(acc[mt][t], afr[(base + f) & 3], bcur[t]);
-                if (s == 0) {
-                    // this step's loads, spread over the slots of the first sub-step
+                // first x fragments of the MFMA phase, read under the rest of the decode
 #pragma unroll
-                    for (int m = (slot * NI + SLOTS - 1) / SLOTS; m < ((slot + 1) * NI + SLOTS - 1) / SLOTS; ++m)
-                        issue(m, kt, (Q + LEAD) % S, (Q + LEAD + 1) % S);
-                    if (slot == 0) {
-                        // sub-step 0 of step kt+1: its registers were decoded during the previous step
-                        T::load_sub(raw, c, 0, btile);
-                        T::load_scale(raw, c, 0, stile);
-                    }
-                }
-                if (slot == SLOTS - 1) {
-                    // decode of the next sub-step (the compiler places it; the other wavefront of
-                    // the SIMD runs MFMAs meanwhile), then refill of the registers just decoded
-                    dq.prep(raw, sn);
-#pragma unroll
-                    for (int u = 0; u < 8; ++u) dq.unit(raw, c, sn, u >> 1, u & 1, bnxt);
-                    if (sn != 0) {
-                        T::load_sub(raw, c, sn, btile);
-                        T::load_scale(raw, c, sn, stile);
-                    }
-                }
-                __builtin_amdgcn_sched_barrier(0);
+                for (int f = 0; f < R; ++f) afr[f & 3] = la[a_lds_unit<BK>(16 * f + i, 4 * h + q)];
             }
+            uint32_t pr[2], lo[2], hi[2];
+            f32x2_t a02[2], b02[2], a13[2], b13[2];
+            float wa[2][4], wb[2][4];
+#pragma unroll
+            for (int p = 0; p < 2; ++p) pr[p] = __builtin_amdgcn_perm(r[2 * (p0 + p) + 1], r[2 * (p0 + p)], sel);   // a.b0 a.b1 b.b0 b.b1
+#pragma unroll
+            for (int p = 0; p < 2; ++p) { lo[p] = pr[p] & mask; hi[p] = pr[p] >> 4; }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int p = 0; p < 2; ++p) {
+                hi[p] &= mask;
+                a02[p] = __builtin_amdgcn_cvt_pk_f32_fp8(lo[p], false);
+                b02[p] = __builtin_amdgcn_cvt_pk_f32_fp8(lo[p], true);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int p = 0; p < 2; ++p) {
+                a13[p] = __builtin_amdgcn_cvt_pk_f32_fp8(hi[p], false);
+                b13[p] = __builtin_amdgcn_cvt_pk_f32_fp8(hi[p], true);
+            }
+#pragma unroll
+            for (int p = 0; p < 2; ++p) {
+                wa[p][0] = fmaf(a02[p][0], m[0], z[0]); wb[p][0] = fmaf(b02[p][0], m[0], z[0]);
+                wa[p][2] = fmaf(a02[p][1], m[2], z[2]); wb[p][2] = fmaf(b02[p][1], m[2], z[2]);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int p = 0; p < 2; ++p) {
+                wa[p][1] = fmaf(a13[p][0], m[1], z[1]); wb[p][1] = fmaf(b13[p][0], m[1], z[1]);
+                wa[p][3] = fmaf(a13[p][1], m[3], z[3]); wb[p][3] = fmaf(b13[p][1], m[3], z[3]);
+            }
+#pragma unroll
+            for (int p = 0; p < 2; ++p) {
+                bf[0][p0 + p] = pack_bf16_rne(wa[p][0], wb[p][0]);
+                bf[2][p0 + p] = pack_bf16_rne(wa[p][2], wb[p][2]);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int p = 0; p < 2; ++p) {
+                bf[1][p0 + p] = pack_bf16_rne(wa[p][1], wb[p][1]);
+                bf[3][p0 + p] = pack_bf16_rne(wa[p][3], wb[p][3]);
+            }
+            __builtin_amdgcn_sched_barrier(0);
         }
+        // ---- MFMA phase, at raised issue priority: the other wavefront of the SIMD is decoding
+        // meanwhile and would otherwise win the arbitration whenever both are ready, starving
+        // the matrix pipe; its VALU instructions fit into the gaps the MFMAs leave
+        __builtin_amdgcn_s_setprio(3);
+        // Both kinds of wavefront are past barrier kt-1 here: this step's loads (stage kt+4 replaces
+        // stage kt-1) and the packed dwords of the next step (stage kt+1, visible since that
+        // barrier) are fetched between the MFMAs.
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            if (mt + R < MT) afr[(mt + R) & 3] = la[a_lds_unit<BK>(16 * (mt + R) + i, 4 * h + q)];
+#pragma unroll
+            for (int t = 0; t < 4; ++t) mfma_16x16x32_v(acc[mt][t], afr[mt & 3], bf[t]);
+#pragma unroll
+            for (int m = (mt * NI + MT - 1) / MT; m < ((mt + 1) * NI + MT - 1) / MT; ++m) issue(m, kt, sl);
+            if (mt == 0) read_raw(sn);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        __builtin_amdgcn_s_setprio(0);
+        if (h == 0) asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(2 * NI) : "memory");   // barrier kt
     };
-    constexpr int U = S == 4 ? 4 : 6;   // multiple of S (stage numbers) and of 2 (fragment ring)
-    for (int kt = 0; kt < nk; kt += U) {
-        step(kt, IntC<0>{});
-        if (kt + 1 < nk) step(kt + 1, IntC<1>{});
-        if (kt + 2 < nk) step(kt + 2, IntC<2>{});
-        if (kt + 3 < nk) step(kt + 3, IntC<3>{});
-        if constexpr (U == 6) {
-            if (kt + 4 < nk) step(kt + 4, IntC<4>{});
-            if (kt + 5 < nk) step(kt + 5, IntC<5>{});
-        }
+    for (int kt = 0, st = 0, sl = S - 1; kt < nk; ++kt) {
+        const int sn = st == S - 1 ? 0 : st + 1;
+        step(kt, st, sn, sl);
+        st = sn;
+        sl = sl == S - 1 ? 0 : sl + 1;
     }
-    // drain this wavefront's loads (they target stages past K and are never read) before the next
-    // tile reuses the ring; the accumulators were last written by MFMAs the compiler cannot see
-    asm volatile("s_waitcnt vmcnt(0)\n\ts_nop 15\n\ts_nop 15" ::: "memory");
+    if (h == 1) asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(2 * NI) : "memory");       // barrier nk-1
+    // drain this wavefront's loads (they target stages past K and are never read); the
+    // accumulators were last written by MFMAs the compiler cannot see: wait out their latency
+    asm volatile("s_waitcnt vmcnt(0)\n\ts_nop 15\n\ts_nop 15\n\ts_barrier" ::: "memory");
 
-    // epilogue through a buffer resource that ends after the tile's last valid row: stores to
-    // padded rows fall outside it and are dropped
-    const rsrc_t ry = make_rsrc(P.y + row0 * (int64_t)P.N, (int64_t)rows * P.N * 2);
-    const int vy = (4 * c.q * P.N + n0 + T::col(c, 0)) * 2;
+    // ---- add the partial sums of wavefront wv + 4 to those of wv, two row blocks per round,
+    // through two alternating LDS buffers (in the x stage area, free now)
+    constexpr int RB = 2, ROUNDS = (MT + RB - 1) / RB;
+    u32x4_t* red = smem;   // [2 buffers][4 column groups][RB * 4 fragments][64 lanes]
+    auto red_unit = [&](int buf, int k) { return ((buf * 4 + cw) * (RB * 4) + k) * 64 + lane; };
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt)
+    for (int rd = 0; rd <= ROUNDS; ++rd) {
+        if (h == 1 && rd < ROUNDS) {
 #pragma unroll
-        for (int r = 0; r < 4; ++r)
-            __builtin_amdgcn_raw_buffer_store_b32(pack_bf16_rne(acc[mt][0][r], acc[mt][1][r]), ry, vy, (16 * mt + r) * P.N * 2, 0);
+            for (int b = 0; b < RB; ++b)
+#pragma unroll
+                for (int t = 0; t < 4; ++t)
+                    if (rd * RB + b < MT) red[red_unit(rd & 1, b * 4 + t)] = __builtin_bit_cast(u32x4_t, acc[rd * RB + b][t]);
+        }
+        if (h == 0 && rd > 0) {
+#pragma unroll
+            for (int b = 0; b < RB; ++b)
+#pragma unroll
+                for (int t = 0; t < 4; ++t)
+                    if ((rd - 1) * RB + b < MT)
+                        acc[(rd - 1) * RB + b][t] += __builtin_bit_cast(f32x4_t, red[red_unit((rd - 1) & 1, b * 4 + t)]);
+        }
+        if (rd < ROUNDS) __syncthreads();
+    }
+
+    if (h == 0) {
+        // epilogue through a buffer resource that ends after the tile's last valid row: stores to
+        // padded rows fall outside it and are dropped
+        const rsrc_t ry = make_rsrc(P.y + row0 * (int64_t)P.N, (int64_t)rows * P.N * 2);
+        const int vy = (4 * q * P.N + n0 + col0) * 2;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                u32x2_t v;
+                v[0] = pack_bf16_rne(acc[mt][0][r], acc[mt][1][r]);
+                v[1] = pack_bf16_rne(acc[mt][2][r], acc[mt][3][r]);
+                __builtin_amdgcn_raw_buffer_store_b64(v, ry, vy, (16 * mt + r) * P.N * 2, 0);
+            }
+    }
+    __syncthreads();   // the reduction buffers are read: the next tile may load into the ring
 }
 
 // ---------------------------------------------------------------------------------
@@ -993,26 +998,22 @@ __device__ __forceinline__ void expert_chunks(int m, int& chunks, int& bpc) {
 //   GK_GENERAL  4 wavefronts of 64 columns, one workgroup per CU, tiles of up to 192 rows
 //   GK_SKINNY   the same tile routine with tiles of at most 32 rows and several workgroups per CU
 //               (decode-sized batches are HBM bound: more weight bytes in flight)
-//   GK_NARROW8  8 wavefronts of 32 columns, one workgroup per CU (containers with NarrowTraits)
-enum { GK_GENERAL = 0, GK_SKINNY = 1, GK_NARROW8 = 2 };
+//   GK_PAIR     int4 prefill: 8 wavefronts, k range split between the two wavefronts of a SIMD
+enum { GK_GENERAL = 0, GK_SKINNY = 1, GK_PAIR = 2 };
 
 template <int FMT, int KIND>
 struct KernelCfg {
-    static constexpr bool NARROW = KIND == GK_NARROW8;
-    static constexpr int WAVES = KIND == GK_NARROW8 ? 8 : 4;
-    static constexpr int BN = NARROW ? 32 * WAVES : GM_BN;                       // columns per tile
+    static_assert(KIND != GK_PAIR || FMT == MOE_FMT_INT4, "the k-split tile routine decodes int4 only");
+    static constexpr int WAVES = KIND == GK_PAIR ? 8 : 4;
+    static constexpr int BN = GM_BN;                                             // columns per tile
     static constexpr int WG_PER_CU = KIND == GK_SKINNY ? GM_SKINNY_WAVES : 1;
-    static constexpr int STAGES = 4;                                             // narrow kernel only
-    static constexpr int CAPB = KIND == GK_SKINNY ? GM_SKINNY_BLOCKS : GM_MT_MAX;
-    static constexpr int fmt_mt_max() {
-        if constexpr (NARROW) return NarrowTraits<FMT, WAVES>::MT_MAX;
-        else return BTraits<FMT>::MT_MAX;
-    }
+    static constexpr int CAPB = KIND == GK_SKINNY ? GM_SKINNY_BLOCKS : KIND == GK_PAIR ? PAIR_CAPB : GM_MT_MAX;
+    static constexpr int fmt_mt_max() { return KIND == GK_PAIR ? PAIR_MT_MAX : BTraits<FMT>::MT_MAX; }
     static constexpr int MTM = CAPB < fmt_mt_max() ? CAPB : fmt_mt_max();        // row blocks per tile
     // 16-byte LDS units of the tile routine (the tile prefix array follows them)
     static constexpr int lds_units() {
-        if constexpr (NARROW)
-            return STAGES * (16 * CAPB * 8 + NarrowTraits<FMT, WAVES>::B_LDS_UNITS + NarrowTraits<FMT, WAVES>::SC_UNITS);
+        if constexpr (KIND == GK_PAIR)
+            return PAIR_LDS_UNITS;
         else
             return 2 * 16 * CAPB * (BTraits<FMT>::BK / 8) + 2 * BTraits<FMT>::B_LDS_UNITS;
     }
@@ -1021,8 +1022,8 @@ struct KernelCfg {
 template <int FMT, int MT, int KIND>
 __device__ __forceinline__ void run_tile(const GemmParams& P, u32x4_t* smem, int g, int64_t row0, int rows, int n0) {
     using C = KernelCfg<FMT, KIND>;
-    if constexpr (C::NARROW)
-        gemm_tile_narrow<FMT, MT, C::CAPB, C::WAVES, C::STAGES>(P, smem, g, row0, rows, n0);
+    if constexpr (KIND == GK_PAIR)
+        gemm_tile_pair_int4<MT>(P, smem, g, row0, rows, n0);
     else
         gemm_tile<FMT, MT, C::CAPB>(P, smem, smem + 2 * 16 * C::CAPB * (BTraits<FMT>::BK / 8), g, row0, rows, n0);
 }
@@ -1184,7 +1185,7 @@ static int launch_gemm_fmt(const moe_grouped_args* a, hipStream_t stream) {
     // device) are HBM bound: use the small-tile kernel.  An expert with more than 32 rows then
     // costs one pass over its weights per 32 rows.
     if (a->M <= 24 * a->G) return launch_gemm_kind<FMT, GK_SKINNY>(P, a, stream);
-    if constexpr (FMT == MOE_FMT_INT4) return launch_gemm_kind<FMT, GK_NARROW8>(P, a, stream);
+    if constexpr (FMT == MOE_FMT_INT4) return launch_gemm_kind<FMT, GK_PAIR>(P, a, stream);
     else return launch_gemm_kind<FMT, GK_GENERAL>(P, a, stream);
 }
 
