@@ -374,6 +374,201 @@ __global__ __launch_bounds__(256) void gemv_nmajor_kernel(const uint16_t* __rest
     }
 }
 
+// ---------------------------------------------------------------------------------
+// MOE_FMT_FP4_B32 on the matrix cores.  The VALU path above spends (1 + rows) / 2
+// instructions per weight element, more than the ~2.4 per element the chip can issue while
+// HBM delivers 4-bit codes at full rate.  Here a wavefront owns 16 weight rows (the MFMA
+// columns) and up to 16 activation rows (the MFMA rows): per 32-k scale block one
+// v_mfma_f32_16x16x32_bf16 on exactly decoded e2m1 values (v_cvt_scalef32_pk_bf16_fp4 with
+// scale 1.0, two codes per instruction) and one fma per accumulator register that applies
+// the block's scale to the partial sum -- the same arithmetic as the VALU path (weights are
+// not rounded to bf16).
+//
+// Weight loads stay 16 bytes per lane: lane (i, q) = (lane & 15, lane >> 4) reads scale block
+// 4 c + q of weight row i, so a load instruction covers 64 contiguous bytes of 16 rows.
+// The MFMA wants the 4 q lanes of a column to hold the 4 dwords of ONE block (a block has
+// one scale, and the MFMA sums over q): a 4x4 transpose of the dwords across the q lanes,
+// two v_permlane32_swap and two v_permlane16_swap per 16 bytes.
+//
+// Scales: every lane of a column needs the same 4 scales per load, 8 bytes of a row -- read
+// that way, each 64-byte piece of a scale row is fetched from HBM several times.  Instead the
+// 4 q lanes of a row read 128 contiguous bytes of it once per 4 loop iterations (lane q: the
+// 16 scales of iteration 4 T + q) and the iteration's scales are picked up from the lane that
+// holds them with ds_bpermute.
+//
+// x (<= 16 rows of a chunk of K) is staged in LDS; the 16-byte units of row r are XOR-swizzled
+// with r so that the fragment reads of the 16 lanes of a q group fall into different banks.
+// ---------------------------------------------------------------------------------
+constexpr int GF_WAVES = 8;               // wavefronts per workgroup
+constexpr int GF_NR_WG = 16 * GF_WAVES;   // weight rows per workgroup
+constexpr int GF_ROWS = 16;               // activation rows per pass
+constexpr int GF_LDS_UNITS = 4096;        // 64 KiB of x per staged chunk
+constexpr int GF_U = 4;                   // 128-k groups (one 16-byte load per lane each) per loop iteration
+constexpr int GF_KSTEP = 128 * GF_U;      // k per loop iteration; K must be a multiple
+
+__device__ __forceinline__ uint32_t e2m1_pair_bf16(uint32_t word, int sel) {
+    switch (sel) {
+        case 0: return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(word, 1.0f, 0));
+        case 1: return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(word, 1.0f, 1));
+        case 2: return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(word, 1.0f, 2));
+        default: return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(word, 1.0f, 3));
+    }
+}
+
+// MB = activation rows staged and multiplied (4, 8 or 16); lanes of MFMA rows >= MB supply zeros.
+template <int MB>
+__device__ __forceinline__ void gemv_fp4_mfma_rows(const uint8_t* __restrict__ wg, const uint16_t* __restrict__ sg,
+                                                   const uint16_t* __restrict__ x, uint16_t* __restrict__ y,
+                                                   u32x4_t* xs, int64_t row0, int mg, int n0, int N, int K) {
+    constexpr int KC = GF_LDS_UNITS / MB * 8;   // k per staged chunk: 8192, 4096 or 2048
+    constexpr int RS = KC / 8;                  // row stride in 16-byte units
+    constexpr int U = GF_U;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int i = lane & 15, q = lane >> 4;
+    const int n = n0 + wave * 16 + i;
+    const int nn = min(n, N - 1);
+    // 32-bit byte offsets from the expert's (wavefront-uniform) base pointers: an expert's weight
+    // slab is smaller than 4 GiB
+    const uint32_t woff = (uint32_t)nn * (uint32_t)(K / 2) + q * 16;
+    const uint32_t soff = (uint32_t)nn * (uint32_t)(K / 32) * 2;
+    f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+
+    for (int kc0 = 0; kc0 < K; kc0 += KC) {
+        const int klen = min(KC, K - kc0);
+        __syncthreads();
+        for (int t = threadIdx.x; t < MB * (klen / 8); t += 64 * GF_WAVES) {
+            const int r = t / (klen / 8), k8 = t % (klen / 8);
+            u32x4_t v = {0u, 0u, 0u, 0u};
+            if (r < mg) v = *reinterpret_cast<const u32x4_t*>(x + (row0 + r) * (int64_t)K + kc0 + k8 * 8);
+            xs[r * RS + (k8 ^ r)] = v;
+        }
+        __syncthreads();
+
+        const int niter = klen / GF_KSTEP;             // iterations of U groups
+        const int nblk = klen / 32;                    // scale blocks of the chunk (>= 16)
+        const uint8_t* wp = wg + (kc0 >> 1);                                   // group c of the chunk: + 64 c bytes
+        const uint8_t* sp = reinterpret_cast<const uint8_t*>(sg) + (kc0 >> 5) * 2;   // block b of the chunk: + 2 b bytes
+        // x fragment of block 4 c + j: unit (16 c + 4 j + q) ^ r of row r = xj[j][16 c].  MFMA rows
+        // >= MB read row i % MB again: their products land in accumulator rows that are not stored.
+        const int r = i % MB;
+        const u32x4_t* xj[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) xj[j] = xs + r * RS + ((4 * j + q) ^ r);
+
+        // one 128-k group: w = this lane's 16 bytes (block 4 c + q of its row), s0/s1 = the 4 scales of
+        // blocks 4 c .. 4 c + 3 as two bf16 pairs
+        auto group = [&](const u32x4_t& w, uint32_t s0, uint32_t s1, int c) {
+            // 4x4 transpose of the dwords over the q lanes: b[j] = this lane's 8 codes of block 4 c + j
+            const u32x2_t t02 = __builtin_amdgcn_permlane32_swap(w[0], w[2], false, false);
+            const u32x2_t t13 = __builtin_amdgcn_permlane32_swap(w[1], w[3], false, false);
+            const u32x2_t b01 = __builtin_amdgcn_permlane16_swap(t02[0], t13[0], false, false);
+            const u32x2_t b23 = __builtin_amdgcn_permlane16_swap(t02[1], t13[1], false, false);
+            const uint32_t b[4] = {b01[0], b01[1], b23[0], b23[1]};
+            const float s[4] = {bf16_lo(s0), bf16_hi(s0), bf16_lo(s1), bf16_hi(s1)};
+            // two blocks at a time: enough independent MFMAs to cover their latency, few enough
+            // live registers for 4 wavefronts per SIMD
+#pragma unroll
+            for (int j0 = 0; j0 < 4; j0 += 2) {
+                u32x4_t aw[2], bw[2];
+                f32x4_t part[2];
+#pragma unroll
+                for (int j = 0; j < 2; ++j) aw[j] = xj[j0 + j][16 * c];
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+#pragma unroll
+                    for (int d = 0; d < 4; ++d) bw[j][d] = e2m1_pair_bf16(b[j0 + j], d);
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+                    part[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, aw[j]),
+                                                                      __builtin_bit_cast(bf16x8_t, bw[j]),
+                                                                      f32x4_t{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+#pragma unroll
+                    for (int rr = 0; rr < 4; ++rr) acc[rr] = fmaf(part[j][rr], s[j0 + j], acc[rr]);
+            }
+        };
+        auto fetch_w = [&](u32x4_t (&w)[U], int it) {
+#pragma unroll
+            for (int u = 0; u < U; ++u)
+                w[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(wp + (woff + (uint32_t)((it * U + u) * 64))));
+        };
+        // the 16 scales of iteration 4 T + q of this lane's row (clamped into the chunk: iterations
+        // past its end do not exist)
+        auto fetch_s = [&](u32x4_t (&sv)[2], int T) {
+            const int b0 = min(64 * T + 16 * q, nblk - 16);
+            sv[0] = *reinterpret_cast<const u32x4_t*>(sp + (soff + (uint32_t)(b0 * 2)));
+            sv[1] = *reinterpret_cast<const u32x4_t*>(sp + (soff + (uint32_t)(b0 * 2 + 16)));
+        };
+        u32x4_t sc[2], sn[2];
+        // iteration `it` on the weights in w; rotates the scale registers every 4 iterations
+        auto iteration = [&](const u32x4_t (&w)[U], int it) {
+            const int t = it & 3;
+            if (t == 0) {
+                sc[0] = sn[0];
+                sc[1] = sn[1];
+                if (it + 4 < niter) fetch_s(sn, (it >> 2) + 1);
+            }
+            // this iteration's scales live in lane (i, t)
+            const int src = (16 * t + i) * 4;
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const uint32_t s0 = (uint32_t)__builtin_amdgcn_ds_bpermute(src, (int)sc[u >> 1][2 * (u & 1)]);
+                const uint32_t s1 = (uint32_t)__builtin_amdgcn_ds_bpermute(src, (int)sc[u >> 1][2 * (u & 1) + 1]);
+                group(w[u], s0, s1, it * U + u);
+            }
+        };
+        // two register sets of weights: the loads of iteration it + 1 are in flight behind iteration it
+        u32x4_t wa[U], wb[U];
+        fetch_s(sn, 0);
+        fetch_w(wa, 0);
+        for (int it = 0; it < niter; it += 2) {
+            if (it + 1 < niter) fetch_w(wb, it + 1);
+            iteration(wa, it);
+            if (it + 1 < niter) {
+                if (it + 2 < niter) fetch_w(wa, it + 2);
+                iteration(wb, it + 1);
+            }
+        }
+    }
+    // lane (i, q) holds column n, rows 4 q .. 4 q + 3
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        const int m = 4 * q + r;
+        if (m < mg && n < N) y[(row0 + m) * (int64_t)N + n] = (uint16_t)(pack_bf16_rne(acc[r], 0.f) & 0xffffu);
+    }
+}
+
+__global__ __launch_bounds__(64 * GF_WAVES, 4) void gemv_fp4_mfma_kernel(const uint16_t* __restrict__ x,
+                                                                         const uint8_t* __restrict__ w,
+                                                                         const uint16_t* __restrict__ scale,
+                                                                         const int64_t* __restrict__ gl,
+                                                                         uint16_t* __restrict__ y, int64_t M, int K,
+                                                                         int N) {
+    extern __shared__ u32x4_t xs[];
+    const int g = blockIdx.y, n0 = blockIdx.x * GF_NR_WG;
+    int64_t start, end;
+    group_rows(gl, g, M, start, end);
+    if (end <= start) return;
+    const uint8_t* wg = w + (int64_t)g * N * ((int64_t)K / 2);
+    const uint16_t* sg = scale + (int64_t)g * N * (K / 32);
+    for (int64_t row0 = start; row0 < end; row0 += GF_ROWS) {
+        const int mg = (int)min((int64_t)GF_ROWS, end - row0);
+        if (mg <= 4) gemv_fp4_mfma_rows<4>(wg, sg, x, y, xs, row0, mg, n0, N, K);
+        else if (mg <= 8) gemv_fp4_mfma_rows<8>(wg, sg, x, y, xs, row0, mg, n0, N, K);
+        else gemv_fp4_mfma_rows<16>(wg, sg, x, y, xs, row0, mg, n0, N, K);
+    }
+}
+
+static int launch_fp4_mfma(const moe_grouped_args* a, hipStream_t stream) {
+    dim3 grid((unsigned)((a->N + GF_NR_WG - 1) / GF_NR_WG), (unsigned)a->G);
+    hipLaunchKernelGGL(gemv_fp4_mfma_kernel, grid, dim3(64 * GF_WAVES), (size_t)GF_LDS_UNITS * 16, stream,
+                       static_cast<const uint16_t*>(a->x), static_cast<const uint8_t*>(a->weight),
+                       static_cast<const uint16_t*>(a->scale), a->group_list, static_cast<uint16_t*>(a->y), a->M,
+                       (int)a->K, (int)a->N);
+    return hipGetLastError() == hipSuccess ? MOE_OK : MOE_ERR_LAUNCH;
+}
+
 template <int FMT>
 static int launch_kmajor(const moe_grouped_args* a, hipStream_t stream) {
     const int kc = (int)(a->K < GV_KC ? a->K : GV_KC);
@@ -409,7 +604,9 @@ static int launch_nmajor(const moe_grouped_args* a, hipStream_t stream) {
 int launch_grouped_gemv(const moe_grouped_args* a, hipStream_t stream) {
     switch (a->format) {
         case MOE_FMT_BF16: return launch_kmajor<MOE_FMT_BF16>(a, stream);
-        case MOE_FMT_FP4_B32: return launch_kmajor<MOE_FMT_FP4_B32>(a, stream);
+        case MOE_FMT_FP4_B32:
+            // the matrix-core kernel takes K in whole loop iterations
+            return a->K % GF_KSTEP == 0 ? launch_fp4_mfma(a, stream) : launch_kmajor<MOE_FMT_FP4_B32>(a, stream);
         case MOE_FMT_FP4_REF: return launch_nmajor<MOE_FMT_FP4_REF>(a, stream);
         case MOE_FMT_FP8_REF: return launch_nmajor<MOE_FMT_FP8_REF>(a, stream);
         case MOE_FMT_INT4: return launch_nmajor<MOE_FMT_INT4>(a, stream);
