@@ -92,7 +92,10 @@ int moe_dequant_fp4_bf16_validate(const moe_dequant_args* a) {
 }
 
 // GEMM: the workgroup tile spans 64 k and 256 n.
-int moe_grouped_gemm_validate(const moe_grouped_args* a) { return validate_grouped(a, 64, 256); }
+int moe_grouped_gemm_validate(const moe_grouped_args* a) {
+    // the fp4_b32 tile routine steps through K 128 at a time
+    return validate_grouped(a, a && a->format == MOE_FMT_FP4_B32 ? 128 : 64, 256);
+}
 
 // GEMV: N-contiguous containers are read 256 columns per wavefront step,
 // K-contiguous ones 8 k per lane.

@@ -1190,12 +1190,9 @@ static int launch_gemm_fmt(const moe_grouped_args* a, hipStream_t stream) {
 }
 
 int launch_grouped_gemm(const moe_grouped_args* a, hipStream_t stream) {
-    // Decode-sized batches on the K-contiguous containers (on average at most 4 rows per
-    // expert) are pure weight streaming: the GEMV kernel reads every weight row as one
-    // contiguous run and is the faster of the two there.  It keeps the dequantized weights in
-    // fp32 instead of rounding them to bf16 first, which stays inside the op's tolerance.
-    if ((a->format == MOE_FMT_FP4_B32 || a->format == MOE_FMT_BF16) && a->M <= 4 * a->G)
-        return launch_grouped_gemv(a, stream);
+    // Decode-sized batches on the K-contiguous containers go to the weight-streaming GEMV kernels,
+    // run with this op's arithmetic.
+    if (gemv_preferred(a)) return launch_grouped_gemv(a, stream, true);
     switch (a->format) {
         case MOE_FMT_FP4_REF: return launch_gemm_fmt<MOE_FMT_FP4_REF>(a, stream);
         case MOE_FMT_FP8_REF: return launch_gemm_fmt<MOE_FMT_FP8_REF>(a, stream);

@@ -405,6 +405,7 @@ constexpr int GF_ROWS = 16;               // activation rows per pass
 constexpr int GF_LDS_UNITS = 4096;        // 64 KiB of x per staged chunk
 constexpr int GF_U = 4;                   // 128-k groups (one 16-byte load per lane each) per loop iteration
 constexpr int GF_KSTEP = 128 * GF_U;      // k per loop iteration; K must be a multiple
+constexpr int GF_GEMM_ROWS_PER_EXPERT = 20;// grouped GEMM calls with at most this many rows per expert on average come here
 
 __device__ __forceinline__ uint32_t e2m1_pair_bf16(uint32_t word, int sel) {
     switch (sel) {
@@ -415,8 +416,11 @@ __device__ __forceinline__ uint32_t e2m1_pair_bf16(uint32_t word, int sel) {
     }
 }
 
-// MB = activation rows staged and multiplied (4, 8 or 16); lanes of MFMA rows >= MB supply zeros.
-template <int MB>
+// MB = activation rows staged and multiplied (4, 8 or 16).  ROUNDW selects the arithmetic of the
+// grouped GEMM op (grouped_matmul_antiquant.h:537-662: weights are RNE_bf16(e2m1 * scale), so the
+// scale has to be applied per element before the MFMA: ~2 VALU instructions per element) instead of
+// that of the GEMV op (fp32 weights: the scale is applied to the block's partial sum).
+template <int MB, bool ROUNDW>
 __device__ __forceinline__ void gemv_fp4_mfma_rows(const uint8_t* __restrict__ wg, const uint16_t* __restrict__ sg,
                                                    const uint16_t* __restrict__ x, uint16_t* __restrict__ y,
                                                    u32x4_t* xs, int64_t row0, int mg, int n0, int N, int K) {
@@ -431,19 +435,10 @@ __device__ __forceinline__ void gemv_fp4_mfma_rows(const uint8_t* __restrict__ w
     // slab is smaller than 4 GiB
     const uint32_t woff = (uint32_t)nn * (uint32_t)(K / 2) + q * 16;
     const uint32_t soff = (uint32_t)nn * (uint32_t)(K / 32) * 2;
-    f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+    f32x4_t acc = {0.f, 0.f, 0.f, 0.f}, acc2 = {0.f, 0.f, 0.f, 0.f};
 
     for (int kc0 = 0; kc0 < K; kc0 += KC) {
         const int klen = min(KC, K - kc0);
-        __syncthreads();
-        for (int t = threadIdx.x; t < MB * (klen / 8); t += 64 * GF_WAVES) {
-            const int r = t / (klen / 8), k8 = t % (klen / 8);
-            u32x4_t v = {0u, 0u, 0u, 0u};
-            if (r < mg) v = *reinterpret_cast<const u32x4_t*>(x + (row0 + r) * (int64_t)K + kc0 + k8 * 8);
-            xs[r * RS + (k8 ^ r)] = v;
-        }
-        __syncthreads();
-
         const int niter = klen / GF_KSTEP;             // iterations of U groups
         const int nblk = klen / 32;                    // scale blocks of the chunk (>= 16)
         const uint8_t* wp = wg + (kc0 >> 1);                                   // group c of the chunk: + 64 c bytes
@@ -470,22 +465,37 @@ __device__ __forceinline__ void gemv_fp4_mfma_rows(const uint8_t* __restrict__ w
 #pragma unroll
             for (int j0 = 0; j0 < 4; j0 += 2) {
                 u32x4_t aw[2], bw[2];
-                f32x4_t part[2];
 #pragma unroll
                 for (int j = 0; j < 2; ++j) aw[j] = xj[j0 + j][16 * c];
+                if constexpr (ROUNDW) {
 #pragma unroll
-                for (int j = 0; j < 2; ++j)
+                    for (int j = 0; j < 2; ++j) {
+                        bw[j][0] = e2m1_pair_scaled_bf16<0>(b[j0 + j], s[j0 + j]);
+                        bw[j][1] = e2m1_pair_scaled_bf16<1>(b[j0 + j], s[j0 + j]);
+                        bw[j][2] = e2m1_pair_scaled_bf16<2>(b[j0 + j], s[j0 + j]);
+                        bw[j][3] = e2m1_pair_scaled_bf16<3>(b[j0 + j], s[j0 + j]);
+                    }
+                    // two accumulators, so that consecutive MFMAs do not depend on each other
+                    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, aw[0]),
+                                                                  __builtin_bit_cast(bf16x8_t, bw[0]), acc, 0, 0, 0);
+                    acc2 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, aw[1]),
+                                                                   __builtin_bit_cast(bf16x8_t, bw[1]), acc2, 0, 0, 0);
+                } else {
+                    f32x4_t part[2];
 #pragma unroll
-                    for (int d = 0; d < 4; ++d) bw[j][d] = e2m1_pair_bf16(b[j0 + j], d);
+                    for (int j = 0; j < 2; ++j)
 #pragma unroll
-                for (int j = 0; j < 2; ++j)
-                    part[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, aw[j]),
-                                                                      __builtin_bit_cast(bf16x8_t, bw[j]),
-                                                                      f32x4_t{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+                        for (int d = 0; d < 4; ++d) bw[j][d] = e2m1_pair_bf16(b[j0 + j], d);
 #pragma unroll
-                for (int j = 0; j < 2; ++j)
+                    for (int j = 0; j < 2; ++j)
+                        part[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, aw[j]),
+                                                                          __builtin_bit_cast(bf16x8_t, bw[j]),
+                                                                          f32x4_t{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
 #pragma unroll
-                    for (int rr = 0; rr < 4; ++rr) acc[rr] = fmaf(part[j][rr], s[j0 + j], acc[rr]);
+                    for (int j = 0; j < 2; ++j)
+#pragma unroll
+                        for (int rr = 0; rr < 4; ++rr) acc[rr] = fmaf(part[j][rr], s[j0 + j], acc[rr]);
+                }
             }
         };
         auto fetch_w = [&](u32x4_t (&w)[U], int it) {
@@ -522,6 +532,15 @@ __device__ __forceinline__ void gemv_fp4_mfma_rows(const uint8_t* __restrict__ w
         u32x4_t wa[U], wb[U];
         fetch_s(sn, 0);
         fetch_w(wa, 0);
+        // stage this chunk of x while the first weights are on their way
+        __syncthreads();
+        for (int t = threadIdx.x; t < MB * (klen / 8); t += 64 * GF_WAVES) {
+            const int r = t / (klen / 8), k8 = t % (klen / 8);
+            u32x4_t v = {0u, 0u, 0u, 0u};
+            if (r < mg) v = *reinterpret_cast<const u32x4_t*>(x + (row0 + r) * (int64_t)K + kc0 + k8 * 8);
+            xs[r * RS + (k8 ^ r)] = v;
+        }
+        __syncthreads();
         for (int it = 0; it < niter; it += 2) {
             if (it + 1 < niter) fetch_w(wb, it + 1);
             iteration(wa, it);
@@ -535,10 +554,11 @@ __device__ __forceinline__ void gemv_fp4_mfma_rows(const uint8_t* __restrict__ w
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
         const int m = 4 * q + r;
-        if (m < mg && n < N) y[(row0 + m) * (int64_t)N + n] = (uint16_t)(pack_bf16_rne(acc[r], 0.f) & 0xffffu);
+        if (m < mg && n < N) y[(row0 + m) * (int64_t)N + n] = (uint16_t)(pack_bf16_rne(acc[r] + acc2[r], 0.f) & 0xffffu);
     }
 }
 
+template <bool ROUNDW>
 __global__ __launch_bounds__(64 * GF_WAVES, 4) void gemv_fp4_mfma_kernel(const uint16_t* __restrict__ x,
                                                                          const uint8_t* __restrict__ w,
                                                                          const uint16_t* __restrict__ scale,
@@ -554,15 +574,16 @@ __global__ __launch_bounds__(64 * GF_WAVES, 4) void gemv_fp4_mfma_kernel(const u
     const uint16_t* sg = scale + (int64_t)g * N * (K / 32);
     for (int64_t row0 = start; row0 < end; row0 += GF_ROWS) {
         const int mg = (int)min((int64_t)GF_ROWS, end - row0);
-        if (mg <= 4) gemv_fp4_mfma_rows<4>(wg, sg, x, y, xs, row0, mg, n0, N, K);
-        else if (mg <= 8) gemv_fp4_mfma_rows<8>(wg, sg, x, y, xs, row0, mg, n0, N, K);
-        else gemv_fp4_mfma_rows<16>(wg, sg, x, y, xs, row0, mg, n0, N, K);
+        if (mg <= 4) gemv_fp4_mfma_rows<4, ROUNDW>(wg, sg, x, y, xs, row0, mg, n0, N, K);
+        else if (mg <= 8) gemv_fp4_mfma_rows<8, ROUNDW>(wg, sg, x, y, xs, row0, mg, n0, N, K);
+        else gemv_fp4_mfma_rows<16, ROUNDW>(wg, sg, x, y, xs, row0, mg, n0, N, K);
     }
 }
 
+template <bool ROUNDW>
 static int launch_fp4_mfma(const moe_grouped_args* a, hipStream_t stream) {
     dim3 grid((unsigned)((a->N + GF_NR_WG - 1) / GF_NR_WG), (unsigned)a->G);
-    hipLaunchKernelGGL(gemv_fp4_mfma_kernel, grid, dim3(64 * GF_WAVES), (size_t)GF_LDS_UNITS * 16, stream,
+    hipLaunchKernelGGL(gemv_fp4_mfma_kernel<ROUNDW>, grid, dim3(64 * GF_WAVES), (size_t)GF_LDS_UNITS * 16, stream,
                        static_cast<const uint16_t*>(a->x), static_cast<const uint8_t*>(a->weight),
                        static_cast<const uint16_t*>(a->scale), a->group_list, static_cast<uint16_t*>(a->y), a->M,
                        (int)a->K, (int)a->N);
@@ -601,12 +622,24 @@ static int launch_nmajor(const moe_grouped_args* a, hipStream_t stream) {
     return hipGetLastError() == hipSuccess ? MOE_OK : MOE_ERR_LAUNCH;
 }
 
-int launch_grouped_gemv(const moe_grouped_args* a, hipStream_t stream) {
+bool gemv_preferred(const moe_grouped_args* a) {
+    // Decode-sized batches on the K-contiguous containers are pure weight streaming: these kernels
+    // read every weight row as contiguous runs.  The bf16 vector kernel takes 4 rows of an expert per
+    // pass over its weights (same arithmetic as the GEMM: the weights are bf16 already).  The
+    // matrix-core fp4_b32 kernel takes 16 and has a variant with the GEMM's weight rounding; the
+    // bound is where the small-tile GEMM kernel overtakes it (measured at DeepSeek-V3 shapes).
+    if (a->format == MOE_FMT_FP4_B32) return a->K % GF_KSTEP == 0 && a->M <= GF_GEMM_ROWS_PER_EXPERT * a->G;
+    if (a->format == MOE_FMT_BF16) return a->M <= 4 * a->G;
+    return false;
+}
+
+int launch_grouped_gemv(const moe_grouped_args* a, hipStream_t stream, bool gemm_rounding) {
     switch (a->format) {
         case MOE_FMT_BF16: return launch_kmajor<MOE_FMT_BF16>(a, stream);
         case MOE_FMT_FP4_B32:
             // the matrix-core kernel takes K in whole loop iterations
-            return a->K % GF_KSTEP == 0 ? launch_fp4_mfma(a, stream) : launch_kmajor<MOE_FMT_FP4_B32>(a, stream);
+            if (a->K % GF_KSTEP != 0) return gemm_rounding ? MOE_ERR_BAD_SHAPE : launch_kmajor<MOE_FMT_FP4_B32>(a, stream);
+            return gemm_rounding ? launch_fp4_mfma<true>(a, stream) : launch_fp4_mfma<false>(a, stream);
         case MOE_FMT_FP4_REF: return launch_nmajor<MOE_FMT_FP4_REF>(a, stream);
         case MOE_FMT_FP8_REF: return launch_nmajor<MOE_FMT_FP8_REF>(a, stream);
         case MOE_FMT_INT4: return launch_nmajor<MOE_FMT_INT4>(a, stream);

@@ -6,6 +6,9 @@
 
 namespace moe {
 int launch_dequant_fp4_bf16(const moe_dequant_args* a, hipStream_t stream);
-int launch_grouped_gemv(const moe_grouped_args* a, hipStream_t stream);
+// gemm_rounding: use the grouped GEMM's arithmetic (weights rounded to bf16) where the two ops differ.
+int launch_grouped_gemv(const moe_grouped_args* a, hipStream_t stream, bool gemm_rounding = false);
+// True when the GEMV launcher is the faster path for a grouped GEMM call of this shape.
+bool gemv_preferred(const moe_grouped_args* a);
 int launch_grouped_gemm(const moe_grouped_args* a, hipStream_t stream);
 }  // namespace moe

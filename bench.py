@@ -205,13 +205,16 @@ def run_extra(torch, mg, gen, iters, warmup):
         mg.dequant_fp4_bf16(w.data_ptr(), s.data_ptr(), wd.data_ptr(), G * N, K, 32, stream())
 
     sep = Op(mg, torch, "gemm", "bf16", x, wd, None, None, gl, y2)
-    t_f, t_d, t_s = time_launches(torch, [fused, dq_all, sep], max(iters // 2, 5), warmup)
+    y3 = torch.empty(M, N, dtype=torch.bfloat16, device="cuda")
+    gemv = Op(mg, torch, "gemv", "fp4_b32", x, w, s, None, gl, y3)   # same kernel with the GEMV op's fp32 weights
+    t_f, t_d, t_s, t_v = time_launches(torch, [fused, dq_all, sep, gemv], max(iters // 2, 5), warmup)
     nbytes = A * (N * K // 2 + N * (K // 32) * 2) + M * K * 2 + M * N * 2
     diff = float((y.float() - y2.float()).abs().max())
     out["fused_fp4_gemm_decode_256e"] = dict(active_experts=A, rows=M, bytes=nbytes, us=t_f * 1e6,
                                              GBps=nbytes / t_f / 1e9, frac_hbm=nbytes / t_f / 1e9 / PEAK_HBM_GBS,
                                              separate_us=(t_d + t_s) * 1e6, separate_dequant_us=t_d * 1e6,
                                              separate_gemm_us=t_s * 1e6, speedup_vs_separate=(t_d + t_s) / t_f,
+                                             gemv_op_us=t_v * 1e6, gemv_op_frac_hbm=nbytes / t_v / 1e9 / PEAK_HBM_GBS,
                                              max_abs_diff_fused_vs_separate=diff)
     return out
 

@@ -76,6 +76,7 @@ typedef enum moe_status {
  * MOE_FMT_FP4_B32  uint8 [G, N, K/2] e2m1, K-contiguous, low nibble = even k;
  *                  scale bf16 [G, N, K/32]; W = bf16(e2m1(code) * float(scale)).
  *                  One expert is exactly a moe_dequant_fp4_bf16 input of N rows, K cols.
+ *                  K % 32 == 0 (grouped GEMM: K % 128 == 0).
  * MOE_FMT_BF16     bf16 [G, N, K], K-contiguous; no scale.
  *
  * GEMM rounds W to bf16 before the product (reference phase 1); GEMV keeps the

@@ -86,6 +86,14 @@ def test_gemm_needs_offset_only_for_int8_and_gemv_rejects_int8():
     assert mg.lib.moe_grouped_gemv_validate(ctypes.byref(gargs(2))) == mg.ERR_BAD_FORMAT
 
 
+def test_fp4_b32_k_alignment_differs_between_gemm_and_gemv():
+    # the GEMM tile routine of fp4_b32 steps through K 128 at a time; the GEMV reads whole 32-k blocks
+    assert mg.lib.moe_grouped_gemm_validate(ctypes.byref(gargs(4, K=192, scale_rows=6))) == mg.ERR_BAD_ALIGNMENT
+    assert mg.lib.moe_grouped_gemm_validate(ctypes.byref(gargs(4, K=256, scale_rows=8))) == mg.MOE_OK
+    assert mg.lib.moe_grouped_gemv_validate(ctypes.byref(gargs(4, K=192, scale_rows=6))) == mg.MOE_OK
+    assert mg.lib.moe_grouped_gemv_validate(ctypes.byref(gargs(4, K=48, scale_rows=1))) == mg.ERR_BAD_ALIGNMENT
+
+
 def test_dequant_validate():
     val = mg.lib.moe_dequant_fp4_bf16_validate
     ok = mg.DequantArgs(P, P, P, 16, 256, 32, 0)
