@@ -11,7 +11,10 @@ namespace moe {
 // 16-byte vectors.  Consecutive lanes take consecutive dwords, so every load
 // instruction of a wavefront covers 256 contiguous bytes and every store 1 KiB.
 // The tensors are addressed flat: rows are contiguous and cols % BLOCK == 0, so
-// element e uses scale e / BLOCK.
+// element e uses scale e / BLOCK.  Measured on MI355X (7168 x 2048 and 64 times that):
+// one dword per thread, ordinary loads and nontemporal stores is the fastest combination
+// at both sizes (nontemporal loads cost 25 % at the small size, 4 dwords per thread 12 % at
+// the large one); at 7168 x 2048 it takes 6.6 us where writing the output alone takes 6.4.
 template <int BLOCK, int UNROLL>
 __global__ __launch_bounds__(256) void dequant_fp4_bf16_kernel(const uint32_t* __restrict__ codes,
                                                                const uint16_t* __restrict__ scale,
@@ -24,7 +27,7 @@ __global__ __launch_bounds__(256) void dequant_fp4_bf16_kernel(const uint32_t* _
     for (int u = 0; u < UNROLL; ++u) {
         const int64_t i = base + u * 256;
         if (i < nwords) {
-            w[u] = __builtin_nontemporal_load(codes + i);
+            w[u] = codes[i];
             s[u] = bf16_bits_to_f32(scale[(i * 8) / BLOCK]);
         }
     }
@@ -45,7 +48,7 @@ __global__ __launch_bounds__(256) void dequant_fp4_bf16_kernel(const uint32_t* _
 int launch_dequant_fp4_bf16(const moe_dequant_args* a, hipStream_t stream) {
     const int64_t nwords = a->rows * a->cols / 8;
     if (nwords == 0) return MOE_OK;
-    constexpr int UNROLL = 4;
+    constexpr int UNROLL = 1;
     const int64_t blocks = (nwords + 256 * UNROLL - 1) / (256 * UNROLL);
     if (blocks > 0x7fffffffLL) return MOE_ERR_TOO_LARGE;
     const uint32_t* codes = static_cast<const uint32_t*>(a->codes);

@@ -100,6 +100,32 @@ def time_batch(torch, fn, iters, warmup):
     return e0.elapsed_time(e1) / iters * 1e-3
 
 
+def time_graph(torch, fn, iters, warmup):
+    """Like time_batch, but the `iters` launches are captured into one HIP graph and replayed, so
+    that the host's launch rate (a few microseconds per call from Python) does not enter.
+    Returns None if the capture fails."""
+    try:
+        for _ in range(warmup):
+            fn()
+        torch.cuda.synchronize()
+        side = torch.cuda.Stream()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=side):
+            for _ in range(iters):
+                fn()
+        g.replay()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        g.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / iters * 1e-3
+    except Exception as ex:  # noqa: BLE001
+        print(f"graph timing unavailable: {ex}", file=sys.stderr)
+        return None
+
+
 def bf16_normal(torch, shape, std=1.0):
     return (torch.randn(shape, device="cuda", dtype=torch.float32) * std).to(torch.bfloat16)
 
@@ -148,11 +174,15 @@ def run_extra(torch, mg, gen, iters, warmup):
     nbytes = R * C // 2 + R * (C // 32) * 2 + R * C * 2
     t_rot = time_batch(torch, dq_rot, 320, warmup + nbuf)
     t_same = time_batch(torch, dq_same, 320, warmup)
+    t_graph = time_graph(torch, dq_rot, 320, warmup)
     out["fp4_dequant_7168x2048"] = dict(bytes=nbytes, us=t_rot * 1e6, GBps=nbytes / t_rot / 1e9,
                                         frac_hbm=nbytes / t_rot / 1e9 / PEAK_HBM_GBS, us_same_buffer=t_same * 1e6,
                                         GBps_same_buffer=nbytes / t_same / 1e9,
+                                        us_graph_replay=None if t_graph is None else t_graph * 1e6,
+                                        frac_hbm_graph_replay=None if t_graph is None else nbytes / t_graph / 1e9 / PEAK_HBM_GBS,
                                         note="320 back-to-back launches between two events, rotating over 16 buffer "
-                                             "sets (cold) / on the same buffers (Infinity Cache warm)")
+                                             "sets (cold) / on the same buffers (Infinity Cache warm); graph_replay: the same 320 "
+                                             "rotating launches captured in one HIP graph (no host launch cost)")
     del codes, scales, outs
 
     # c2: grouped GEMV decode, 64 experts, 32 rows (4 tokens x top-8), K=7168, N=2048, bf16 weights [G,N,K]
