@@ -171,6 +171,49 @@ void DequantFp4(at::Tensor weight, at::Tensor scale, at::Tensor output) {
     check_status(moe_dequant_fp4_bf16(&a, current_stream(weight)), "dequant_fp4");
 }
 
+// Extra entry points: the weight preparation the reference's tests do on the host with torch
+// reshapes (repack_weight + repack_weight_step2, anti_quant_fp8_scale + transpose;
+// grouped_gemm/test/python/test_group_gemm_fp4.py:86-142, :180-186), as GPU ops that return new tensors.
+
+// checkpoint codes uint8 [G, N, K/2] -> "fp4" op weight int8 [G, K, N/2]
+at::Tensor RepackWeightFp4(at::Tensor weight) {
+    if (!weight.defined() || !weight.is_cuda()) fail("weight must be a GPU tensor");
+    check_tensor(weight, "weight", at::kByte, 3, weight);
+    const int64_t G = weight.size(0), N = weight.size(1), K = weight.size(2) * 2;
+    at::Tensor out = at::empty({G, K, N / 2}, weight.options().dtype(at::kChar));
+    moe_prepack_fp4_args a = {};
+    a.codes = weight.data_ptr();
+    a.weight_out = out.data_ptr();
+    a.G = G; a.N = N; a.K = K;
+    c10::DeviceGuard guard(weight.device());
+    check_status(moe_prepack_fp4_ref(&a, current_stream(weight)), "repack_weight_fp4");
+    return out;
+}
+
+// checkpoint scales bf16 [G, N, K/16] (x optional fp32 scale_2 [G, 1 or 2, 1]) -> bf16 [G, K/16, N]
+at::Tensor MergeScaleFp4(at::Tensor scale, c10::optional<at::Tensor> scale_2) {
+    if (!scale.defined() || !scale.is_cuda()) fail("scale must be a GPU tensor");
+    check_tensor(scale, "scale", at::kBFloat16, 3, scale);
+    const int64_t G = scale.size(0), N = scale.size(1), KB = scale.size(2);
+    at::Tensor out = at::empty({G, KB, N}, scale.options());
+    moe_prepack_fp4_args a = {};
+    a.scale = scale.data_ptr();
+    a.scale_out = out.data_ptr();
+    a.G = G; a.N = N; a.K = KB * 16;
+    at::Tensor s2;
+    if (scale_2 && scale_2->defined()) {
+        s2 = *scale_2;
+        if (!s2.is_cuda() || s2.device() != scale.device()) fail("scale_2 must be on the same device as scale");
+        if (s2.scalar_type() != at::kFloat || !s2.is_contiguous()) fail("scale_2 must be a contiguous float32 tensor");
+        if (s2.numel() != G && s2.numel() != 2 * G) fail("scale_2 must hold one or two factors per expert");
+        a.scale2 = s2.data_ptr();
+        a.scale2_cols = static_cast<int32_t>(s2.numel() / G);
+    }
+    c10::DeviceGuard guard(scale.device());
+    check_status(moe_prepack_fp4_ref(&a, current_stream(scale)), "merge_scale_fp4");
+    return out;
+}
+
 }  // namespace
 
 PYBIND11_MODULE(cinfer_ascendc, m) {
@@ -180,4 +223,8 @@ PYBIND11_MODULE(cinfer_ascendc, m) {
     m.def("grouped_gemm", &GroupedGemm, "x"_a, "weight"_a, "antiquantScaleOptional"_a, "antiquantOffsetOptional"_a,
           "groupListOptional"_a, "computeType"_a, "output"_a, "GROUP GEMM.");
     m.def("dequant_fp4", &DequantFp4, "weight"_a, "scale"_a, "output"_a, "FP4 (e2m1) -> BF16 block dequant.");
+    m.def("repack_weight_fp4", &RepackWeightFp4, "weight"_a,
+          "Checkpoint fp4 codes [G, N, K/2] -> the \"fp4\" op weight [G, K, N/2].");
+    m.def("merge_scale_fp4", &MergeScaleFp4, "scale"_a, "scale_2"_a = pybind11::none(),
+          "Checkpoint block scales [G, N, K/16] (x scale_2) -> the \"fp4\" op scale [G, K/16, N].");
 }

@@ -105,7 +105,25 @@ int moe_grouped_gemv_validate(const moe_grouped_args* a) {
     return validate_grouped(a, k_major ? 32 : 64, k_major ? 1 : 256);
 }
 
+int moe_prepack_fp4_ref_validate(const moe_prepack_fp4_args* a) {
+    if (!a) return MOE_ERR_NULL_POINTER;
+    if (a->reserved != 0 || a->scale2_cols < 0 || a->scale2_cols > 2) return MOE_ERR_BAD_FORMAT;
+    if (a->G <= 0 || a->N <= 0 || a->K <= 0) return MOE_ERR_BAD_SHAPE;
+    if (!fits_i32(a->G) || !fits_i32(a->N) || !fits_i32(a->K)) return MOE_ERR_TOO_LARGE;
+    if (a->K % 64 || a->N % 256) return MOE_ERR_BAD_ALIGNMENT;
+    // grid dimensions: experts in z, 64-row tiles of N in y
+    if (a->G > 65535 || a->N / 64 > 65535) return MOE_ERR_TOO_LARGE;
+    if (!a->codes != !a->weight_out || !a->scale != !a->scale_out) return MOE_ERR_NULL_POINTER;
+    if (!a->codes && !a->scale) return MOE_ERR_NULL_POINTER;
+    if (a->scale2_cols > 0 && a->scale && !a->scale2) return MOE_ERR_NULL_POINTER;
+    if (!aligned16(a->codes) || !aligned16(a->weight_out) || !aligned16(a->scale) || !aligned16(a->scale_out) ||
+        (reinterpret_cast<uintptr_t>(a->scale2) & 3u))
+        return MOE_ERR_BAD_ALIGNMENT;
+    return MOE_OK;
+}
+
 size_t moe_dequant_fp4_bf16_workspace_bytes(const moe_dequant_args*) { return 0; }
+size_t moe_prepack_fp4_ref_workspace_bytes(const moe_prepack_fp4_args*) { return 0; }
 size_t moe_grouped_gemm_workspace_bytes(const moe_grouped_args*) { return 0; }
 size_t moe_grouped_gemv_workspace_bytes(const moe_grouped_args*) { return 0; }
 
@@ -113,6 +131,12 @@ int moe_dequant_fp4_bf16(const moe_dequant_args* a, moe_stream_t stream) {
     int rc = moe_dequant_fp4_bf16_validate(a);
     if (rc != MOE_OK) return rc;
     return moe::launch_dequant_fp4_bf16(a, static_cast<hipStream_t>(stream));
+}
+
+int moe_prepack_fp4_ref(const moe_prepack_fp4_args* a, moe_stream_t stream) {
+    int rc = moe_prepack_fp4_ref_validate(a);
+    if (rc != MOE_OK) return rc;
+    return moe::launch_prepack_fp4_ref(a, static_cast<hipStream_t>(stream));
 }
 
 int moe_grouped_gemm(const moe_grouped_args* a, moe_stream_t stream) {

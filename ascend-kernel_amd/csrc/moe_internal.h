@@ -11,4 +11,5 @@ int launch_grouped_gemv(const moe_grouped_args* a, hipStream_t stream, bool gemm
 // True when the GEMV launcher is the faster path for a grouped GEMM call of this shape.
 bool gemv_preferred(const moe_grouped_args* a);
 int launch_grouped_gemm(const moe_grouped_args* a, hipStream_t stream);
+int launch_prepack_fp4_ref(const moe_prepack_fp4_args* a, hipStream_t stream);
 }  // namespace moe

@@ -24,6 +24,7 @@ SYMBOLS = (
     "moe_dequant_fp4_bf16_validate", "moe_grouped_gemm_validate", "moe_grouped_gemv_validate",
     "moe_dequant_fp4_bf16_workspace_bytes", "moe_grouped_gemm_workspace_bytes", "moe_grouped_gemv_workspace_bytes",
     "moe_dequant_fp4_bf16", "moe_grouped_gemm", "moe_grouped_gemv",
+    "moe_prepack_fp4_ref_validate", "moe_prepack_fp4_ref_workspace_bytes", "moe_prepack_fp4_ref",
 )
 
 
@@ -40,6 +41,13 @@ class DequantArgs(ctypes.Structure):
                 ("reserved", ctypes.c_int32)]
 
 
+class PrepackFp4Args(ctypes.Structure):
+    _fields_ = [("codes", ctypes.c_void_p), ("scale", ctypes.c_void_p), ("scale2", ctypes.c_void_p),
+                ("weight_out", ctypes.c_void_p), ("scale_out", ctypes.c_void_p),
+                ("G", ctypes.c_int64), ("N", ctypes.c_int64), ("K", ctypes.c_int64),
+                ("scale2_cols", ctypes.c_int32), ("reserved", ctypes.c_int32)]
+
+
 if not os.path.exists(LIB_PATH):
     raise ImportError(f"{LIB_PATH} is missing: build it with `python ascend-kernel_amd/build.py` "
                       "(there is no CPU fallback)")
@@ -50,7 +58,8 @@ lib.moe_strerror.restype = ctypes.c_char_p
 lib.moe_strerror.argtypes = [ctypes.c_int]
 lib.moe_format_from_compute_type.restype = ctypes.c_int
 lib.moe_format_from_compute_type.argtypes = [ctypes.c_char_p]
-for _n, _t in (("dequant_fp4_bf16", DequantArgs), ("grouped_gemm", GroupedArgs), ("grouped_gemv", GroupedArgs)):
+for _n, _t in (("dequant_fp4_bf16", DequantArgs), ("grouped_gemm", GroupedArgs), ("grouped_gemv", GroupedArgs),
+               ("prepack_fp4_ref", PrepackFp4Args)):
     getattr(lib, f"moe_{_n}_validate").restype = ctypes.c_int
     getattr(lib, f"moe_{_n}_validate").argtypes = [ctypes.POINTER(_t)]
     getattr(lib, f"moe_{_n}_workspace_bytes").restype = ctypes.c_size_t
@@ -96,3 +105,11 @@ def grouped_gemm(args: GroupedArgs, stream: int = 0) -> None:
 
 def grouped_gemv(args: GroupedArgs, stream: int = 0) -> None:
     _check(lib.moe_grouped_gemv(ctypes.byref(args), ctypes.c_void_p(stream)), "moe_grouped_gemv")
+
+
+def prepack_fp4_ref(codes_ptr, scale_ptr, scale2_ptr, weight_out_ptr, scale_out_ptr, G: int, N: int, K: int,
+                    scale2_cols: int = 0, stream: int = 0) -> None:
+    """Checkpoint codes [G,N,K/2] / scales [G,N,K/16] -> the "fp4" container [G,K,N/2] / [G,K/16,N]."""
+    a = PrepackFp4Args(codes_ptr or None, scale_ptr or None, scale2_ptr or None, weight_out_ptr or None,
+                       scale_out_ptr or None, G, N, K, scale2_cols, 0)
+    _check(lib.moe_prepack_fp4_ref(ctypes.byref(a), ctypes.c_void_p(stream)), "moe_prepack_fp4_ref")

@@ -185,6 +185,23 @@ def run_extra(torch, mg, gen, iters, warmup):
                                              "rotating launches captured in one HIP graph (no host launch cost)")
     del codes, scales, outs
 
+    # weight preparation for the reference's "fp4" container: checkpoint codes [G, N, K/2] + scales [G, N, K/16]
+    # -> [G, K, N/2] + [G, K/16, N] (nibble transpose + tile permutation, scale merge + transpose)
+    G, K, N = 32, 7168, 2048
+    ck = torch.randint(0, 256, (G, N, K // 2), dtype=torch.uint8, device="cuda")
+    sck = bf16_uniform(torch, (G, N, K // 16), 1.0, 448.0)
+    s2 = torch.rand(G, 1, device="cuda") * 1e-2
+    wo = torch.empty(G, K, N // 2, dtype=torch.int8, device="cuda")
+    so = torch.empty(G, K // 16, N, dtype=torch.bfloat16, device="cuda")
+
+    def pp():
+        mg.prepack_fp4_ref(ck.data_ptr(), sck.data_ptr(), s2.data_ptr(), wo.data_ptr(), so.data_ptr(), G, N, K, 1, stream())
+
+    t = time_batch(torch, pp, 20, warmup)
+    nbytes = 2 * (ck.numel() + sck.numel() * 2)
+    out["prepack_fp4_ref_32e"] = dict(bytes=nbytes, us=t * 1e6, GBps=nbytes / t / 1e9, frac_hbm=nbytes / t / 1e9 / PEAK_HBM_GBS)
+    del ck, sck, wo, so
+
     # c2: grouped GEMV decode, 64 experts, 32 rows (4 tokens x top-8), K=7168, N=2048, bf16 weights [G,N,K]
     G, K, N = 64, 7168, 2048
     counts = routed_counts(torch, 4, G, 8, gen, max_rows=4)

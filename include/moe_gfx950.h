@@ -121,6 +121,26 @@ typedef struct moe_dequant_args {
     int32_t reserved; /* must be 0 */
 } moe_dequant_args;
 
+/* Checkpoint tensors of the reference's NVFP4-style weights -> the MOE_FMT_FP4_REF container
+ * (what the reference test builds on the host with repack_weight + repack_weight_step2 and the
+ * scale merge / transpose, grouped_gemm/test/python/test_group_gemm_fp4.py:86-94, :105-142,
+ * :180-186).  Bit-exact.  Either half may be skipped by passing NULL for both of its pointers.
+ *   codes       uint8 [G, N, K/2], even k in the low nibble   -> weight_out int8 [G, K, N/2]
+ *   scale       bf16  [G, N, K/16]                            -> scale_out  bf16 [G, K/16, N]
+ *   scale2      optional fp32 [G, scale2_cols] second-level scale, multiplied in (fp32 product,
+ *               RNE to bf16): scale2_cols = 1, or 2 for one factor per half of the N rows
+ * K % 64 == 0, N % 256 == 0. */
+typedef struct moe_prepack_fp4_args {
+    const void *codes;
+    const void *scale;
+    const void *scale2;
+    void *weight_out;
+    void *scale_out;
+    int64_t G, N, K;
+    int32_t scale2_cols; /* 0 (scale2 ignored), 1 or 2 */
+    int32_t reserved;    /* must be 0 */
+} moe_prepack_fp4_args;
+
 int moe_abi_version(void);
 const char *moe_strerror(int status);
 
@@ -132,17 +152,20 @@ int moe_format_from_compute_type(const char *compute_type);
 int moe_dequant_fp4_bf16_validate(const moe_dequant_args *args);
 int moe_grouped_gemm_validate(const moe_grouped_args *args);
 int moe_grouped_gemv_validate(const moe_grouped_args *args);
+int moe_prepack_fp4_ref_validate(const moe_prepack_fp4_args *args);
 
 /* Device scratch the launch needs: 0 for every op (kept for callers that follow
  * the reference's two-phase GetWorkspaceSize protocol). */
 size_t moe_dequant_fp4_bf16_workspace_bytes(const moe_dequant_args *args);
 size_t moe_grouped_gemm_workspace_bytes(const moe_grouped_args *args);
 size_t moe_grouped_gemv_workspace_bytes(const moe_grouped_args *args);
+size_t moe_prepack_fp4_ref_workspace_bytes(const moe_prepack_fp4_args *args);
 
 /* Launches (validate first, then enqueue on `stream`). */
 int moe_dequant_fp4_bf16(const moe_dequant_args *args, moe_stream_t stream);
 int moe_grouped_gemm(const moe_grouped_args *args, moe_stream_t stream);
 int moe_grouped_gemv(const moe_grouped_args *args, moe_stream_t stream);
+int moe_prepack_fp4_ref(const moe_prepack_fp4_args *args, moe_stream_t stream);
 
 #ifdef __cplusplus
 }

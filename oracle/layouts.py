@@ -90,3 +90,28 @@ def fp8ref_dequant_numpy(w: np.ndarray, scale: np.ndarray, round_bf16: bool) -> 
         val = bf16_bits_to_f32(f32_to_bf16_bits(val))
     val = val.reshape(G, K // 128, N // 128, 128, 128).transpose(0, 1, 3, 2, 4)
     return np.ascontiguousarray(val).reshape(G, K, N)
+
+
+def fp4ref_scale_from_checkpoint(scale_bits: np.ndarray, scale2: np.ndarray | None = None) -> np.ndarray:
+    """Checkpoint block scales bf16 bits [G, N, K/16] (+ optional fp32 second-level scale
+    [G, 1] or [G, 2]) -> the op's scale tensor, bf16 bits [G, K/16, N].
+
+    anti_quant_fp8_scale (test_group_gemm_fp4.py:86-94): the bf16 tensor is multiplied in place by
+    the fp32 factor -- an fp32 product rounded to nearest even -- one factor per expert, or one
+    for each half of the N rows; then transposed (:185-186)."""
+    from . import bf16_bits_to_f32, f32_to_bf16_bits
+
+    s = np.asarray(scale_bits, dtype=np.uint16)
+    G, N, KB = s.shape
+    if scale2 is not None:
+        s2 = np.asarray(scale2, dtype=np.float32).reshape(G, -1)
+        f = bf16_bits_to_f32(s)
+        if s2.shape[1] == 1:
+            f = f * s2[:, :, None]
+        else:
+            assert s2.shape[1] == 2 and N % 2 == 0
+            f = f.copy()
+            f[:, : N // 2, :] *= s2[:, 0, None, None]
+            f[:, N // 2 :, :] *= s2[:, 1, None, None]
+        s = f32_to_bf16_bits(f.astype(np.float32))
+    return np.ascontiguousarray(s.transpose(0, 2, 1))

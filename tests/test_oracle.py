@@ -212,6 +212,32 @@ def test_expand_int8_int4_fp4b32_bf16_closed_forms():
     assert np.array_equal(got, wf[1].float().numpy().T)
 
 
+def test_scale_merge_and_transpose_against_torch_in_place_multiply():
+    """anti_quant_fp8_scale (test_group_gemm_fp4.py:86-94) multiplies the bf16 scale tensor in
+    place by the fp32 second-level scale; torch computes that product in fp32 and rounds to
+    nearest even.  Then the test transposes to [G, K/16, N] (:185-186)."""
+    rng = np.random.default_rng(11)
+    G, N, KB = 3, 8, 12
+    sc = torch.from_numpy(rng.uniform(1.0, 448.0, (G, N, KB)).astype(np.float32)).to(torch.bfloat16)
+    # one factor per expert (scale_2.shape[-2] == 1)
+    s2 = torch.from_numpy(rng.uniform(1e-4, 1e-2, (G, 1, 1)).astype(np.float32))
+    ref = sc.clone()
+    ref *= s2
+    ref = ref.to(torch.bfloat16).transpose(1, 2).contiguous()
+    got = L.fp4ref_scale_from_checkpoint(bf16_bits(sc), s2.numpy().reshape(G, 1))
+    assert np.array_equal(got, bf16_bits(ref))
+    # two factors: first / second half of the N rows
+    s2 = torch.from_numpy(rng.uniform(1e-4, 1e-2, (G, 2, 1)).astype(np.float32))
+    ref = sc.clone()
+    ref[..., : N // 2, :] *= s2[..., 0, :].unsqueeze(-1)
+    ref[..., N // 2 :, :] *= s2[..., 1, :].unsqueeze(-1)
+    ref = ref.to(torch.bfloat16).transpose(1, 2).contiguous()
+    got = L.fp4ref_scale_from_checkpoint(bf16_bits(sc), s2.numpy().reshape(G, 2))
+    assert np.array_equal(got, bf16_bits(ref))
+    # no second-level scale: a plain transpose
+    assert np.array_equal(L.fp4ref_scale_from_checkpoint(bf16_bits(sc)), bf16_bits(sc.transpose(1, 2).contiguous()))
+
+
 # ---------------------------------------------------------------- grouped_gemm
 @pytest.mark.parametrize("group_list", [[2, 3, 4, 256], [12, 25, 44, 48], [1, 2, 3, 4], [0, 0, 5, 5], [3, 3, 3, 3]])
 def test_grouped_gemm_against_torch_fp64(group_list):
