@@ -18,7 +18,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(HERE)
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libmoe_gfx950.so")
-KERNEL_SOURCES = ["moe_abi.cpp", "moe_dequant.hip", "moe_prepack.hip", "moe_gemv.hip", "moe_gemm.hip"]
+KERNEL_SOURCES = ["moe_abi.cpp", "moe_dequant.hip", "moe_prepack.hip", "moe_route.hip", "moe_gemv.hip", "moe_gemm.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 # -packed-fp32-ops off: the compiler must not form v_pk_*_f32 from scalar float code
 HIP_FLAGS = ["-O3", "--offload-arch=gfx950", "-std=c++17", "-fPIC", "-Xclang", "-target-feature", "-Xclang",

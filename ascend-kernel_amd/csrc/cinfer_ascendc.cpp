@@ -11,6 +11,8 @@
 // reference does.
 #include <c10/core/DeviceGuard.h>
 #include <c10/hip/HIPStream.h>
+
+#include <tuple>
 #include <torch/extension.h>
 
 #include <stdexcept>
@@ -214,6 +216,42 @@ at::Tensor MergeScaleFp4(at::Tensor scale, c10::optional<at::Tensor> scale_2) {
     return out;
 }
 
+// Extra entry point: routing.  logits fp32 [T, E], x bf16 [T, K] -> (x_sorted bf16 [T*topk, K],
+// group_list int64 [E], topk_weight fp32 [T, topk], topk_ids int32 [T, topk], row_of_choice int32
+// [T*topk]): what a caller needs before grouped_gemm (rows sorted by expert + the cumulative
+// group_list of grouped_matmul_utils.h:304-320) and after it (where each token's k results are).
+std::tuple<at::Tensor, at::Tensor, at::Tensor, at::Tensor, at::Tensor> MoeRoute(at::Tensor logits, at::Tensor x, int64_t topk) {
+    if (!logits.defined() || !logits.is_cuda()) fail("logits must be a GPU tensor");
+    check_tensor(logits, "logits", at::kFloat, 2, logits);
+    check_tensor(x, "x", at::kBFloat16, 2, logits);
+    const int64_t T = logits.size(0), E = logits.size(1), K = x.size(1);
+    if (x.size(0) != T) fail("x must have one row per row of logits");
+    if (topk <= 0 || topk > E) fail("topk must be in [1, number of experts]");
+    const auto opt = logits.options();
+    at::Tensor x_sorted = at::empty({T * topk, K}, x.options());
+    at::Tensor group_list = at::empty({E}, opt.dtype(at::kLong));
+    at::Tensor weight = at::empty({T, topk}, opt);
+    at::Tensor ids = at::empty({T, topk}, opt.dtype(at::kInt));
+    at::Tensor row_token = at::empty({T * topk}, opt.dtype(at::kInt));
+    at::Tensor row_of_choice = at::empty({T * topk}, opt.dtype(at::kInt));
+    moe_route_args a = {};
+    a.logits = logits.data_ptr();
+    a.x = x.data_ptr();
+    a.topk_ids = ids.data_ptr();
+    a.topk_weight = weight.data_ptr();
+    a.group_list = group_list.data_ptr<int64_t>();
+    a.row_token = row_token.data_ptr();
+    a.row_of_choice = row_of_choice.data_ptr();
+    a.x_sorted = x_sorted.data_ptr();
+    a.T = T; a.E = E; a.K = K;
+    a.topk = static_cast<int32_t>(topk);
+    at::Tensor ws = at::empty({static_cast<int64_t>(moe_route_workspace_bytes(&a)) + 4}, opt.dtype(at::kByte));
+    a.workspace = ws.data_ptr();
+    c10::DeviceGuard guard(logits.device());
+    check_status(moe_route(&a, current_stream(logits)), "moe_route");
+    return {x_sorted, group_list, weight, ids, row_of_choice};
+}
+
 }  // namespace
 
 PYBIND11_MODULE(cinfer_ascendc, m) {
@@ -223,6 +261,8 @@ PYBIND11_MODULE(cinfer_ascendc, m) {
     m.def("grouped_gemm", &GroupedGemm, "x"_a, "weight"_a, "antiquantScaleOptional"_a, "antiquantOffsetOptional"_a,
           "groupListOptional"_a, "computeType"_a, "output"_a, "GROUP GEMM.");
     m.def("dequant_fp4", &DequantFp4, "weight"_a, "scale"_a, "output"_a, "FP4 (e2m1) -> BF16 block dequant.");
+    m.def("moe_route", &MoeRoute, "logits"_a, "x"_a, "topk"_a,
+          "Router logits -> (x_sorted, group_list, topk_weight, topk_ids, row_of_choice).");
     m.def("repack_weight_fp4", &RepackWeightFp4, "weight"_a,
           "Checkpoint fp4 codes [G, N, K/2] -> the \"fp4\" op weight [G, K, N/2].");
     m.def("merge_scale_fp4", &MergeScaleFp4, "scale"_a, "scale_2"_a = pybind11::none(),

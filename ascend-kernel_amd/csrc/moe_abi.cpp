@@ -2,6 +2,7 @@
 // error strings, and the extern "C" entry points that hand over to the launchers.
 #include <cstdint>
 #include <cstring>
+#include <initializer_list>
 
 #include "moe_internal.h"
 
@@ -122,6 +123,30 @@ int moe_prepack_fp4_ref_validate(const moe_prepack_fp4_args* a) {
     return MOE_OK;
 }
 
+int moe_route_validate(const moe_route_args* a) {
+    if (!a) return MOE_ERR_NULL_POINTER;
+    if (a->reserved != 0) return MOE_ERR_BAD_FORMAT;
+    if (a->T < 0 || a->E <= 0 || a->topk <= 0 || a->K < 0) return MOE_ERR_BAD_SHAPE;
+    if (a->E > 1024 || a->topk > a->E) return MOE_ERR_BAD_SHAPE;
+    if (!fits_i32(a->T) || !fits_i32(a->K) || !fits_i32(a->T * a->topk)) return MOE_ERR_TOO_LARGE;
+    if (!a->group_list) return MOE_ERR_NULL_POINTER;
+    if (a->T > 0 && (!a->topk_ids || !a->row_token || !a->row_of_choice || !a->workspace)) return MOE_ERR_NULL_POINTER;
+    if (a->T > 0 && a->logits && !a->topk_weight) return MOE_ERR_NULL_POINTER;
+    if (!a->x != !a->x_sorted) return MOE_ERR_NULL_POINTER;
+    if (a->x && (a->K <= 0 || a->K % 8)) return MOE_ERR_BAD_ALIGNMENT;
+    if (!aligned16(a->x) || !aligned16(a->x_sorted) || (reinterpret_cast<uintptr_t>(a->group_list) & 7u)) return MOE_ERR_BAD_ALIGNMENT;
+    for (const void* p : {a->logits, static_cast<const void*>(a->topk_ids), static_cast<const void*>(a->topk_weight),
+                          static_cast<const void*>(a->row_token), static_cast<const void*>(a->row_of_choice),
+                          static_cast<const void*>(a->workspace)})
+        if (reinterpret_cast<uintptr_t>(p) & 3u) return MOE_ERR_BAD_ALIGNMENT;
+    return MOE_OK;
+}
+
+size_t moe_route_workspace_bytes(const moe_route_args* a) {
+    if (!a || a->T <= 0 || a->E <= 0 || a->topk <= 0) return 0;
+    return moe::route_workspace_bytes(a);
+}
+
 size_t moe_dequant_fp4_bf16_workspace_bytes(const moe_dequant_args*) { return 0; }
 size_t moe_prepack_fp4_ref_workspace_bytes(const moe_prepack_fp4_args*) { return 0; }
 size_t moe_grouped_gemm_workspace_bytes(const moe_grouped_args*) { return 0; }
@@ -137,6 +162,12 @@ int moe_prepack_fp4_ref(const moe_prepack_fp4_args* a, moe_stream_t stream) {
     int rc = moe_prepack_fp4_ref_validate(a);
     if (rc != MOE_OK) return rc;
     return moe::launch_prepack_fp4_ref(a, static_cast<hipStream_t>(stream));
+}
+
+int moe_route(const moe_route_args* a, moe_stream_t stream) {
+    int rc = moe_route_validate(a);
+    if (rc != MOE_OK) return rc;
+    return moe::launch_route(a, static_cast<hipStream_t>(stream));
 }
 
 int moe_grouped_gemm(const moe_grouped_args* a, moe_stream_t stream) {

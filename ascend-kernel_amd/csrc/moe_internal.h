@@ -12,4 +12,6 @@ int launch_grouped_gemv(const moe_grouped_args* a, hipStream_t stream, bool gemm
 bool gemv_preferred(const moe_grouped_args* a);
 int launch_grouped_gemm(const moe_grouped_args* a, hipStream_t stream);
 int launch_prepack_fp4_ref(const moe_prepack_fp4_args* a, hipStream_t stream);
+int launch_route(const moe_route_args* a, hipStream_t stream);
+size_t route_workspace_bytes(const moe_route_args* a);
 }  // namespace moe

@@ -25,6 +25,7 @@ SYMBOLS = (
     "moe_dequant_fp4_bf16_workspace_bytes", "moe_grouped_gemm_workspace_bytes", "moe_grouped_gemv_workspace_bytes",
     "moe_dequant_fp4_bf16", "moe_grouped_gemm", "moe_grouped_gemv",
     "moe_prepack_fp4_ref_validate", "moe_prepack_fp4_ref_workspace_bytes", "moe_prepack_fp4_ref",
+    "moe_route_validate", "moe_route_workspace_bytes", "moe_route",
 )
 
 
@@ -48,6 +49,14 @@ class PrepackFp4Args(ctypes.Structure):
                 ("scale2_cols", ctypes.c_int32), ("reserved", ctypes.c_int32)]
 
 
+class RouteArgs(ctypes.Structure):
+    _fields_ = [("logits", ctypes.c_void_p), ("x", ctypes.c_void_p), ("topk_ids", ctypes.c_void_p),
+                ("topk_weight", ctypes.c_void_p), ("group_list", ctypes.c_void_p), ("row_token", ctypes.c_void_p),
+                ("row_of_choice", ctypes.c_void_p), ("x_sorted", ctypes.c_void_p), ("workspace", ctypes.c_void_p),
+                ("T", ctypes.c_int64), ("E", ctypes.c_int64), ("K", ctypes.c_int64),
+                ("topk", ctypes.c_int32), ("reserved", ctypes.c_int32)]
+
+
 if not os.path.exists(LIB_PATH):
     raise ImportError(f"{LIB_PATH} is missing: build it with `python ascend-kernel_amd/build.py` "
                       "(there is no CPU fallback)")
@@ -59,7 +68,7 @@ lib.moe_strerror.argtypes = [ctypes.c_int]
 lib.moe_format_from_compute_type.restype = ctypes.c_int
 lib.moe_format_from_compute_type.argtypes = [ctypes.c_char_p]
 for _n, _t in (("dequant_fp4_bf16", DequantArgs), ("grouped_gemm", GroupedArgs), ("grouped_gemv", GroupedArgs),
-               ("prepack_fp4_ref", PrepackFp4Args)):
+               ("prepack_fp4_ref", PrepackFp4Args), ("route", RouteArgs)):
     getattr(lib, f"moe_{_n}_validate").restype = ctypes.c_int
     getattr(lib, f"moe_{_n}_validate").argtypes = [ctypes.POINTER(_t)]
     getattr(lib, f"moe_{_n}_workspace_bytes").restype = ctypes.c_size_t
@@ -113,3 +122,18 @@ def prepack_fp4_ref(codes_ptr, scale_ptr, scale2_ptr, weight_out_ptr, scale_out_
     a = PrepackFp4Args(codes_ptr or None, scale_ptr or None, scale2_ptr or None, weight_out_ptr or None,
                        scale_out_ptr or None, G, N, K, scale2_cols, 0)
     _check(lib.moe_prepack_fp4_ref(ctypes.byref(a), ctypes.c_void_p(stream)), "moe_prepack_fp4_ref")
+
+
+def route_args(logits_ptr, x_ptr, topk_ids_ptr, topk_weight_ptr, group_list_ptr, row_token_ptr, row_of_choice_ptr,
+               x_sorted_ptr, workspace_ptr, T: int, E: int, K: int, topk: int) -> RouteArgs:
+    n = lambda p: p or None
+    return RouteArgs(n(logits_ptr), n(x_ptr), n(topk_ids_ptr), n(topk_weight_ptr), n(group_list_ptr), n(row_token_ptr),
+                     n(row_of_choice_ptr), n(x_sorted_ptr), n(workspace_ptr), T, E, K, topk, 0)
+
+
+def route_workspace_bytes(args: RouteArgs) -> int:
+    return int(lib.moe_route_workspace_bytes(ctypes.byref(args)))
+
+
+def route(args: RouteArgs, stream: int = 0) -> None:
+    _check(lib.moe_route(ctypes.byref(args), ctypes.c_void_p(stream)), "moe_route")

@@ -202,6 +202,26 @@ def run_extra(torch, mg, gen, iters, warmup):
     out["prepack_fp4_ref_32e"] = dict(bytes=nbytes, us=t * 1e6, GBps=nbytes / t / 1e9, frac_hbm=nbytes / t / 1e9 / PEAK_HBM_GBS)
     del ck, sck, wo, so
 
+    # routing for configuration 4: 4096 tokens, 256 experts, top-8, K = 7168: logits -> top-k -> group_list
+    # and the token rows gathered into expert order
+    T, E, K, topk = 4096, 256, 7168, 8
+    lg = torch.randn(T, E, device="cuda")
+    xr = bf16_normal(torch, (T, K))
+    n = T * topk
+    ids = torch.empty(n, dtype=torch.int32, device="cuda"); wt = torch.empty(n, device="cuda")
+    glr = torch.empty(E, dtype=torch.int64, device="cuda")
+    rt = torch.empty(n, dtype=torch.int32, device="cuda"); roc = torch.empty(n, dtype=torch.int32, device="cuda")
+    xs = torch.empty(n, K, dtype=torch.bfloat16, device="cuda")
+    ra = mg.route_args(lg.data_ptr(), xr.data_ptr(), ids.data_ptr(), wt.data_ptr(), glr.data_ptr(), rt.data_ptr(),
+                       roc.data_ptr(), xs.data_ptr(), 0, T, E, K, topk)
+    ws = torch.empty(mg.route_workspace_bytes(ra) + 4, dtype=torch.uint8, device="cuda")
+    ra.workspace = ws.data_ptr()
+    t = time_batch(torch, lambda: mg.route(ra, stream()), 20, warmup)
+    nbytes = T * E * 4 + T * K * 2 + n * K * 2      # logits + x read (x rows are re-read from cache) + sorted rows written
+    out["routing_4096x256_top8"] = dict(bytes=nbytes, us=t * 1e6, GBps=nbytes / t / 1e9, frac_hbm=nbytes / t / 1e9 / PEAK_HBM_GBS,
+                                        note="5 kernels: top-k, histogram, scan, rank, row gather")
+    del lg, xr, xs
+
     # c2: grouped GEMV decode, 64 experts, 32 rows (4 tokens x top-8), K=7168, N=2048, bf16 weights [G,N,K]
     G, K, N = 64, 7168, 2048
     counts = routed_counts(torch, 4, G, 8, gen, max_rows=4)

@@ -141,6 +141,36 @@ typedef struct moe_prepack_fp4_args {
     int32_t reserved;    /* must be 0 */
 } moe_prepack_fp4_args;
 
+/* Routing: router logits -> top-k experts per token -> rows sorted by expert and the cumulative
+ * group_list the grouped ops read (the reference leaves this step to its caller, which uses
+ * torch_npu.npu_moe_init_routing for it; group_list as in
+ * grouped_gemm/op_kernel/grouped_matmul_utils.h:304-320).  All device pointers.
+ *   logits       fp32 [T, E], or NULL when topk_ids is already filled by the caller
+ *   topk_ids     int32 [T, topk]   out (in, if logits is NULL); ids outside [0, E) are dropped
+ *   topk_weight  fp32 [T, topk]    out: softmax probability of each chosen expert (not
+ *                                  renormalised over the k); ignored if logits is NULL
+ *   group_list   int64 [E]         out: rows of experts 0..e, cumulative
+ *   row_token    int32 [T * topk]  out: token whose activations sorted row r holds
+ *   row_of_choice int32 [T * topk] out: sorted row of choice (t, j) at [t * topk + j], -1 if dropped
+ *   x            bf16 [T, K] or NULL;  x_sorted  bf16 [T * topk, K] out: x[row_token[r]]
+ *   workspace    moe_route_workspace_bytes(args) bytes of device scratch, 4-byte aligned
+ * Sorted order: by expert id, then by t * topk + j (stable).  Ties between logits go to the
+ * lower expert id.  E <= 1024, topk <= E, K % 8 == 0. */
+typedef struct moe_route_args {
+    const void *logits;
+    const void *x;
+    void *topk_ids;
+    void *topk_weight;
+    int64_t *group_list;
+    void *row_token;
+    void *row_of_choice;
+    void *x_sorted;
+    void *workspace;
+    int64_t T, E, K;
+    int32_t topk;
+    int32_t reserved; /* must be 0 */
+} moe_route_args;
+
 int moe_abi_version(void);
 const char *moe_strerror(int status);
 
@@ -153,19 +183,22 @@ int moe_dequant_fp4_bf16_validate(const moe_dequant_args *args);
 int moe_grouped_gemm_validate(const moe_grouped_args *args);
 int moe_grouped_gemv_validate(const moe_grouped_args *args);
 int moe_prepack_fp4_ref_validate(const moe_prepack_fp4_args *args);
+int moe_route_validate(const moe_route_args *args);
 
-/* Device scratch the launch needs: 0 for every op (kept for callers that follow
- * the reference's two-phase GetWorkspaceSize protocol). */
+/* Device scratch the launch needs (the reference's two-phase GetWorkspaceSize protocol): 0 for
+ * every op except moe_route, whose caller passes that many bytes in args->workspace. */
 size_t moe_dequant_fp4_bf16_workspace_bytes(const moe_dequant_args *args);
 size_t moe_grouped_gemm_workspace_bytes(const moe_grouped_args *args);
 size_t moe_grouped_gemv_workspace_bytes(const moe_grouped_args *args);
 size_t moe_prepack_fp4_ref_workspace_bytes(const moe_prepack_fp4_args *args);
+size_t moe_route_workspace_bytes(const moe_route_args *args);
 
 /* Launches (validate first, then enqueue on `stream`). */
 int moe_dequant_fp4_bf16(const moe_dequant_args *args, moe_stream_t stream);
 int moe_grouped_gemm(const moe_grouped_args *args, moe_stream_t stream);
 int moe_grouped_gemv(const moe_grouped_args *args, moe_stream_t stream);
 int moe_prepack_fp4_ref(const moe_prepack_fp4_args *args, moe_stream_t stream);
+int moe_route(const moe_route_args *args, moe_stream_t stream);
 
 #ifdef __cplusplus
 }

@@ -238,6 +238,52 @@ def test_scale_merge_and_transpose_against_torch_in_place_multiply():
     assert np.array_equal(L.fp4ref_scale_from_checkpoint(bf16_bits(sc)), bf16_bits(sc.transpose(1, 2).contiguous()))
 
 
+def test_routing_sort_brute_force_and_invariants():
+    """route_sort is a stable sort of the (token, choice) pairs by expert id: checked against a
+    pure-Python insertion into per-expert lists, and against what any such sort must satisfy."""
+    from oracle import routing as R
+
+    rng = np.random.default_rng(21)
+    T, k, E = 37, 3, 7
+    ids = rng.integers(0, E, (T, k)).astype(np.int32)
+    ids[5, 1] = -1      # dropped
+    ids[9, 0] = E       # dropped
+    gl, row_token, roc = R.route_sort(ids, E)
+    buckets = [[] for _ in range(E)]
+    for t in range(T):
+        for j in range(k):
+            if 0 <= ids[t, j] < E:
+                buckets[ids[t, j]].append((t, j))
+    flat = [tj for b in buckets for tj in b]
+    assert list(gl) == list(np.cumsum([len(b) for b in buckets]))
+    assert [t for t, _ in flat] == list(row_token)
+    for r, (t, j) in enumerate(flat):
+        assert roc[t * k + j] == r
+    assert roc[5 * k + 1] == -1 and roc[9 * k + 0] == -1
+    # invariants: expert ids of the sorted rows are non-decreasing, row_of_choice is a bijection onto the rows
+    valid = roc >= 0
+    sorted_ids = np.empty(valid.sum(), dtype=np.int64)
+    sorted_ids[roc[valid]] = ids.reshape(-1)[valid]
+    assert (np.diff(sorted_ids) >= 0).all() and gl[-1] == valid.sum()
+    assert sorted(roc[valid]) == list(range(valid.sum()))
+
+
+def test_routing_topk_against_torch_topk_and_softmax():
+    from oracle import routing as R
+
+    g = torch.Generator().manual_seed(4)
+    logits = torch.randn(50, 64, generator=g)
+    ids, w = R.route_topk(logits.numpy(), 8)
+    tv, ti = torch.topk(logits, 8, dim=1)          # distinct values: no tie-breaking involved
+    assert np.array_equal(ids, ti.numpy().astype(np.int32))
+    assert np.allclose(w, torch.softmax(logits, dim=1).gather(1, ti).numpy(), rtol=1e-6, atol=1e-8)
+    # ties go to the lower expert id
+    tie = np.zeros((1, 6), dtype=np.float32)
+    tie[0, 4] = 1.0
+    ids, _ = R.route_topk(tie, 3)
+    assert list(ids[0]) == [4, 0, 1]
+
+
 # ---------------------------------------------------------------- grouped_gemm
 @pytest.mark.parametrize("group_list", [[2, 3, 4, 256], [12, 25, 44, 48], [1, 2, 3, 4], [0, 0, 5, 5], [3, 3, 3, 3]])
 def test_grouped_gemm_against_torch_fp64(group_list):
