@@ -103,11 +103,12 @@ void fill_grouped(moe_grouped_args& a, const at::Tensor& x, const at::Tensor& we
             want(scale, "scale", {G, scale_rows, N});
             break;
         case MOE_FMT_FP4_B32:
+        case MOE_FMT_FP4_B16:
             check_tensor(weight, "weight", at::kByte, 3, x);
             N = weight.size(1);
             want(weight, "weight", {G, N, K / 2});
             check_tensor(scale, "scale", at::kBFloat16, 3, x);
-            want(scale, "scale", {G, N, K / 32});
+            want(scale, "scale", {G, N, K / (fmt == MOE_FMT_FP4_B32 ? 32 : 16)});
             break;
         default:  // MOE_FMT_BF16
             check_tensor(weight, "weight", at::kBFloat16, 3, x);

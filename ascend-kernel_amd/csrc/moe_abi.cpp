@@ -38,6 +38,7 @@ int validate_grouped(const moe_grouped_args* a, int64_t k_mult, int64_t n_mult) 
             if ((a->K / a->scale_rows) % 32) return MOE_ERR_BAD_ALIGNMENT;
             break;
         case MOE_FMT_FP4_B32:
+        case MOE_FMT_FP4_B16:
             if (a->K % 32) return MOE_ERR_BAD_ALIGNMENT;
             break;
         default:
@@ -76,6 +77,7 @@ int moe_format_from_compute_type(const char* s) {
     if (!std::strcmp(s, "int8")) return MOE_FMT_INT8;
     if (!std::strcmp(s, "int4")) return MOE_FMT_INT4;
     if (!std::strcmp(s, "fp4_b32")) return MOE_FMT_FP4_B32;
+    if (!std::strcmp(s, "fp4_b16")) return MOE_FMT_FP4_B16;
     if (!std::strcmp(s, "bf16")) return MOE_FMT_BF16;
     return MOE_ERR_BAD_FORMAT;
 }
@@ -95,14 +97,15 @@ int moe_dequant_fp4_bf16_validate(const moe_dequant_args* a) {
 // GEMM: the workgroup tile spans 64 k and 256 n.
 int moe_grouped_gemm_validate(const moe_grouped_args* a) {
     // the fp4_b32 tile routine steps through K 128 at a time
-    return validate_grouped(a, a && a->format == MOE_FMT_FP4_B32 ? 128 : 64, 256);
+    const bool fp4_k = a && (a->format == MOE_FMT_FP4_B32 || a->format == MOE_FMT_FP4_B16);
+    return validate_grouped(a, fp4_k ? 128 : 64, 256);
 }
 
 // GEMV: N-contiguous containers are read 256 columns per wavefront step,
 // K-contiguous ones 8 k per lane.
 int moe_grouped_gemv_validate(const moe_grouped_args* a) {
     if (a && a->format == MOE_FMT_INT8) return MOE_ERR_BAD_FORMAT;  // the GEMV op has no offset operand
-    const bool k_major = a && (a->format == MOE_FMT_BF16 || a->format == MOE_FMT_FP4_B32);
+    const bool k_major = a && (a->format == MOE_FMT_BF16 || a->format == MOE_FMT_FP4_B32 || a->format == MOE_FMT_FP4_B16);
     return validate_grouped(a, k_major ? 32 : 64, k_major ? 1 : 256);
 }
 

@@ -325,12 +325,12 @@ struct BTraits<MOE_FMT_FP8_REF> : BTraitsByte<MOE_FMT_FP8_REF> {
     };
 };
 
-// -------------------------------------------------------- fp4 block-32, [N, K/2]
+// ------------------------------------------- fp4 block-32 / block-16, [N, K/2]
 // K-contiguous: MFMA t, lane (i, q) owns column 64w + 16t + i and loads the 16 bytes
-// holding k = k0 + 32q + [0,32) (exactly one scale block); sub-step s uses
+// holding k = k0 + 32q + [0,32) (one scale block of 32, or two of 16); sub-step s uses
 // k = k0 + 32q + 8s + [0,8), so the matching x chunk is 4q + s.
-template <>
-struct BTraits<MOE_FMT_FP4_B32> {
+template <int BLK>
+struct BTraitsFp4K {
     static constexpr int BK = 128, NS = 4;
     static constexpr int B_LDS_UNITS = 0, B_LOADS = 1;
     // One 16-byte load per t serves all 4 sub-steps, so the registers cannot be reloaded
@@ -338,9 +338,10 @@ struct BTraits<MOE_FMT_FP4_B32> {
     // ignores its sub-step argument and is called once per step).
     static constexpr bool DOUBLE_RAW = true;
     static constexpr int MT_MAX = 10;  // larger tiles spill: BK = 128 doubles the x staging registers
+    static constexpr int SPB = 32 / BLK;   // scales per 16-byte load
     struct Raw {
         u32x4_t r[4];
-        float sc[4];
+        uint32_t sc[4];   // block 32: the scale as fp32 bits; block 16: the two bf16 scales, unpacked where used
     };
     __device__ static __forceinline__ void stage_load(u32x4_t*, const BCtx&, int) {}
     __device__ static __forceinline__ void stage_store(u32x4_t*, const u32x4_t*, const BCtx&) {}
@@ -349,14 +350,17 @@ struct BTraits<MOE_FMT_FP4_B32> {
     __device__ static __forceinline__ int col(const BCtx& c, int t) { return 64 * c.w + 16 * t + c.i; }
     __device__ static __forceinline__ void init(BCtx& c) {
         c.vw = (64 * c.w + c.i) * (c.K >> 1) + 16 * c.q;
-        c.vs = ((64 * c.w + c.i) * (c.K >> 5) + c.q) * 2;
+        c.vs = ((64 * c.w + c.i) * (c.K / BLK) + SPB * c.q) * 2;
     }
     __device__ static __forceinline__ void load_sub(Raw& raw, const BCtx& c, int k0, int, const u32x4_t*) {
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
             raw.r[t] = ldg_b128(c.rw, c.vw, (c.n0 + 16 * t) * (c.K >> 1) + (k0 >> 1));
-            raw.sc[t] = bf16_bits_to_f32(
-                __builtin_amdgcn_raw_buffer_load_b16(c.rs, c.vs, ((c.n0 + 16 * t) * (c.K >> 5) + (k0 >> 5)) * 2, 0));
+            const int so = ((c.n0 + 16 * t) * (c.K / BLK) + k0 / BLK) * 2;
+            if constexpr (BLK == 32)
+                raw.sc[t] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b16(c.rs, c.vs, so, 0) << 16;
+            else
+                raw.sc[t] = ldg_b32(c.rs, c.vs, so);
         }
     }
     struct Dq {
@@ -364,13 +368,19 @@ struct BTraits<MOE_FMT_FP4_B32> {
         __device__ __forceinline__ void prep(const Raw&, const BCtx&, int) {}
         __device__ __forceinline__ void unit(const Raw& raw, const BCtx&, int s, int p, int t, u32x4_t out[4]) {
             const uint32_t wd = pinned(raw.r[t][s]);
-            out[t][p] = pinned(p == 0   ? e2m1_pair_scaled_bf16<0>(wd, raw.sc[t])
-                               : p == 1 ? e2m1_pair_scaled_bf16<1>(wd, raw.sc[t])
-                               : p == 2 ? e2m1_pair_scaled_bf16<2>(wd, raw.sc[t])
-                                        : e2m1_pair_scaled_bf16<3>(wd, raw.sc[t]));
+            // sub-steps 0, 1 / 2, 3 are the two blocks of 16
+            const float sc = BLK == 32 ? __uint_as_float(raw.sc[t]) : (s >> 1) ? bf16_hi(raw.sc[t]) : bf16_lo(raw.sc[t]);
+            out[t][p] = pinned(p == 0   ? e2m1_pair_scaled_bf16<0>(wd, sc)
+                               : p == 1 ? e2m1_pair_scaled_bf16<1>(wd, sc)
+                               : p == 2 ? e2m1_pair_scaled_bf16<2>(wd, sc)
+                                        : e2m1_pair_scaled_bf16<3>(wd, sc));
         }
     };
 };
+template <>
+struct BTraits<MOE_FMT_FP4_B32> : BTraitsFp4K<32> {};
+template <>
+struct BTraits<MOE_FMT_FP4_B16> : BTraitsFp4K<16> {};
 
 // ------------------------------------------------------------------ bf16, [N, K]
 // K-contiguous: lane (i, q) loads 32 contiguous bytes, k = k0 + 16q + [0,16); sub-step
@@ -455,6 +465,10 @@ __device__ __forceinline__ void make_ctx(BCtx& c, const GemmParams& P, int g, in
         case MOE_FMT_FP4_B32:
             c.rw = make_rsrc(P.w + g * (KN >> 1), KN >> 1);
             c.rs = make_rsrc(static_cast<const uint16_t*>(P.scale) + g * (KN >> 5), KN >> 4);
+            break;
+        case MOE_FMT_FP4_B16:
+            c.rw = make_rsrc(P.w + g * (KN >> 1), KN >> 1);
+            c.rs = make_rsrc(static_cast<const uint16_t*>(P.scale) + g * (KN >> 4), KN >> 3);
             break;
         default:
             c.rw = make_rsrc(P.w + g * KN * 2, KN * 2);
@@ -1199,6 +1213,7 @@ int launch_grouped_gemm(const moe_grouped_args* a, hipStream_t stream) {
         case MOE_FMT_INT8: return launch_gemm_fmt<MOE_FMT_INT8>(a, stream);
         case MOE_FMT_INT4: return launch_gemm_fmt<MOE_FMT_INT4>(a, stream);
         case MOE_FMT_FP4_B32: return launch_gemm_fmt<MOE_FMT_FP4_B32>(a, stream);
+        case MOE_FMT_FP4_B16: return launch_gemm_fmt<MOE_FMT_FP4_B16>(a, stream);
         case MOE_FMT_BF16: return launch_gemm_fmt<MOE_FMT_BF16>(a, stream);
         default: return MOE_ERR_BAD_FORMAT;
     }

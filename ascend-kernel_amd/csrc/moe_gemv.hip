@@ -44,11 +44,19 @@ struct KMajor<MOE_FMT_BF16> {
     static constexpr int CH = 8;      // k per lane per step (16 B of weights)
     static constexpr int NR_WG = 32;  // weight rows per workgroup: small enough that the last
                                       // round of workgroups does not leave CUs idle for long
+    static constexpr int BLK = 1;     // no scales (kept non-zero: it appears as a divisor in code shared with fp4)
 };
 template <>
 struct KMajor<MOE_FMT_FP4_B32> {
     static constexpr int CH = 32;     // one scale block (16 B of codes)
     static constexpr int NR_WG = 64;  // decode-bound: fewer x refills per weight byte pay more
+    static constexpr int BLK = 32;
+};
+template <>
+struct KMajor<MOE_FMT_FP4_B16> {
+    static constexpr int CH = 32;     // two scale blocks per 16 B of codes
+    static constexpr int NR_WG = 64;
+    static constexpr int BLK = 16;
 };
 
 // LDS position (in 16-byte units) of the 8 k starting at k8*8, laid out so that the
@@ -117,12 +125,19 @@ __device__ __forceinline__ void gemv_kmajor_rows(const uint8_t* __restrict__ wg,
 #pragma unroll
                     for (int j = 0; j < GVK_NRW; ++j) {
                         const int nn = min(n + j, N - 1);
-                        const float s = bf16_bits_to_f32(sg[(int64_t)nn * (K / 32) + (kc0 + k) / 32]);
+                        constexpr int BLK = KMajor<FMT>::BLK;
+                        const uint16_t* sp = sg + (int64_t)nn * (K / BLK) + (kc0 + k) / BLK;
+                        const float s = bf16_bits_to_f32(sp[0]);
                         float part[MG];
 #pragma unroll
                         for (int r = 0; r < MG; ++r) part[r] = 0.f;
 #pragma unroll
                         for (int d = 0; d < 4; ++d) {
+                            if (BLK == 16 && d == 2) {
+                                // second block of 16: close the first one
+#pragma unroll
+                                for (int r = 0; r < MG; ++r) { acc[j][r] = fmaf(part[r], s, acc[j][r]); part[r] = 0.f; }
+                            }
                             // exact e2m1 -> bf16 pairs (scale 1.0); the block scale is applied to the
                             // 32-element partial sum
                             uint32_t p0 = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w[j][d], 1.0f, 0));
@@ -137,8 +152,9 @@ __device__ __forceinline__ void gemv_kmajor_rows(const uint8_t* __restrict__ wg,
                                 part[r] = dot2_bf16(p3, xv[r][d][3], part[r]);
                             }
                         }
+                        const float s_last = BLK == 16 ? bf16_bits_to_f32(sp[1]) : s;
 #pragma unroll
-                        for (int r = 0; r < MG; ++r) acc[j][r] = fmaf(part[r], s, acc[j][r]);
+                        for (int r = 0; r < MG; ++r) acc[j][r] = fmaf(part[r], s_last, acc[j][r]);
                     }
                 }
             }
@@ -165,7 +181,7 @@ __global__ __launch_bounds__(256) void gemv_kmajor_kernel(const uint16_t* __rest
     group_rows(gl, g, M, start, end);
     if (end <= start) return;
     const uint8_t* wg = w + (int64_t)g * N * (FMT == MOE_FMT_BF16 ? (int64_t)K * 2 : (int64_t)K / 2);
-    const uint16_t* sg = FMT == MOE_FMT_BF16 ? nullptr : scale + (int64_t)g * N * (K / 32);
+    const uint16_t* sg = FMT == MOE_FMT_BF16 ? nullptr : scale + (int64_t)g * N * (K / KMajor<FMT>::BLK);
     for (int64_t row0 = start; row0 < end; row0 += GV_ROWS) {
         const int mg = (int)min((int64_t)GV_ROWS, end - row0);
         switch (mg) {
@@ -640,6 +656,7 @@ int launch_grouped_gemv(const moe_grouped_args* a, hipStream_t stream, bool gemm
             // the matrix-core kernel takes K in whole loop iterations
             if (a->K % GF_KSTEP != 0) return gemm_rounding ? MOE_ERR_BAD_SHAPE : launch_kmajor<MOE_FMT_FP4_B32>(a, stream);
             return gemm_rounding ? launch_fp4_mfma<true>(a, stream) : launch_fp4_mfma<false>(a, stream);
+        case MOE_FMT_FP4_B16: return gemm_rounding ? MOE_ERR_BAD_SHAPE : launch_kmajor<MOE_FMT_FP4_B16>(a, stream);
         case MOE_FMT_FP4_REF: return launch_nmajor<MOE_FMT_FP4_REF>(a, stream);
         case MOE_FMT_FP8_REF: return launch_nmajor<MOE_FMT_FP8_REF>(a, stream);
         case MOE_FMT_INT4: return launch_nmajor<MOE_FMT_INT4>(a, stream);

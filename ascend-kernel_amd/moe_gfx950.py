@@ -14,7 +14,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libmoe_gfx950.so")
 
 MOE_OK = 0
-FMT_FP4_REF, FMT_FP8_REF, FMT_INT8, FMT_INT4, FMT_FP4_B32, FMT_BF16 = range(6)
+FMT_FP4_REF, FMT_FP8_REF, FMT_INT8, FMT_INT4, FMT_FP4_B32, FMT_BF16, FMT_FP4_B16 = range(7)
 ERR_NULL_POINTER, ERR_BAD_FORMAT, ERR_BAD_SHAPE, ERR_BAD_ALIGNMENT, ERR_TOO_LARGE, ERR_LAUNCH, ERR_NO_DEVICE = (
     -1, -2, -3, -4, -5, -6, -7)
 

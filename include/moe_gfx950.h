@@ -78,6 +78,11 @@ typedef enum moe_status {
  *                  One expert is exactly a moe_dequant_fp4_bf16 input of N rows, K cols.
  *                  K % 32 == 0 (grouped GEMM: K % 128 == 0).
  * MOE_FMT_BF16     bf16 [G, N, K], K-contiguous; no scale.
+ * MOE_FMT_FP4_B16  as MOE_FMT_FP4_B32 with one scale per 16 k: scale bf16 [G, N, K/16].  This is the
+ *                  reference checkpoint's own orientation (codes [G, N, K/2], block scales
+ *                  [G, N, K/16], grouped_gemm/test/python/test_group_gemm_fp4.py:46-64) with the
+ *                  second-level scale multiplied in: no repacking between checkpoint and op.
+ *                  K % 32 == 0 (grouped GEMM: K % 128 == 0).
  *
  * GEMM rounds W to bf16 before the product (reference phase 1); GEMV keeps the
  * fp32 product un-rounded (grouped_soft_gemv/op_kernel/gemv_impl.h:147-199).
@@ -89,7 +94,8 @@ typedef enum moe_weight_format {
     MOE_FMT_INT4 = 3,
     MOE_FMT_FP4_B32 = 4,
     MOE_FMT_BF16 = 5,
-    MOE_FMT_COUNT = 6
+    MOE_FMT_FP4_B16 = 6,
+    MOE_FMT_COUNT = 7
 } moe_weight_format;
 
 /* Arguments of both grouped ops.  x, y are row-major bf16; group_list is the
@@ -174,7 +180,7 @@ typedef struct moe_route_args {
 int moe_abi_version(void);
 const char *moe_strerror(int status);
 
-/* "fp4" | "fp8" (reference values) | "int8" | "int4" | "fp4_b32" | "bf16";
+/* "fp4" | "fp8" (reference values) | "int8" | "int4" | "fp4_b32" | "bf16" | "fp4_b16";
  * returns the moe_weight_format or MOE_ERR_BAD_FORMAT. */
 int moe_format_from_compute_type(const char *compute_type);
 

@@ -18,7 +18,7 @@ import numpy as np
 _HERE = os.path.dirname(os.path.abspath(__file__))
 _LIB_PATH = os.path.join(_HERE, "libmoe_oracle.so")
 
-FMT_FP4_REF, FMT_FP8_REF, FMT_INT8, FMT_INT4, FMT_FP4_B32, FMT_BF16 = range(6)
+FMT_FP4_REF, FMT_FP8_REF, FMT_INT8, FMT_INT4, FMT_FP4_B32, FMT_BF16, FMT_FP4_B16 = range(7)
 FMT_BY_NAME = {
     "fp4": FMT_FP4_REF,
     "fp8": FMT_FP8_REF,
@@ -26,6 +26,7 @@ FMT_BY_NAME = {
     "int4": FMT_INT4,
     "fp4_b32": FMT_FP4_B32,
     "bf16": FMT_BF16,
+    "fp4_b16": FMT_FP4_B16,
 }
 
 
@@ -129,7 +130,7 @@ def _logical_knG(fmt: int, w: np.ndarray):
         return G, w.shape[1], w.shape[2] * 2
     if fmt in (FMT_FP8_REF, FMT_INT8):
         return G, w.shape[1], w.shape[2]
-    if fmt == FMT_FP4_B32:
+    if fmt in (FMT_FP4_B32, FMT_FP4_B16):
         return G, w.shape[2] * 2, w.shape[1]
     if fmt == FMT_BF16:
         return G, w.shape[2], w.shape[1]

@@ -41,7 +41,9 @@ enum {
     ORC_FMT_INT8 = 2,    /* int8 [G,K,N]; scale bf16 [G,N]; offset bf16 [G,N]                 */
     ORC_FMT_INT4 = 3,    /* uint8 [G,K,N/2] low nibble = even n; zero point 8; scale bf16 [G,K/gs,N] */
     ORC_FMT_FP4_B32 = 4, /* uint8 [G,N,K/2] low nibble = even k; scale bf16 [G,N,K/32]        */
-    ORC_FMT_BF16 = 5     /* bf16 [G,N,K]                                                       */
+    ORC_FMT_BF16 = 5,    /* bf16 [G,N,K]                                                       */
+    ORC_FMT_FP4_B16 = 6  /* as ORC_FMT_FP4_B32 with scale bf16 [G,N,K/16]: the checkpoint orientation of
+                            grouped_gemm/test/python/test_group_gemm_fp4.py:46-64                     */
 };
 
 static inline float bf16_to_f32(uint16_t h) {
@@ -185,15 +187,16 @@ int orc_expand_weight(int fmt, const void *w, const void *scale, const void *off
                 float v = (float)(q - 8) * bf16_to_f32(sc[(k / gs) * N + n]);
                 out[k * N + n] = round_bf16 ? bf16_to_f32(f32_to_bf16_rne(v)) : v;
             }
-    } else if (fmt == ORC_FMT_FP4_B32) {
+    } else if (fmt == ORC_FMT_FP4_B32 || fmt == ORC_FMT_FP4_B16) {
+        const int64_t blk = fmt == ORC_FMT_FP4_B32 ? 32 : 16;
         const uint8_t *wb = (const uint8_t *)w + g * N * (K / 2);
-        const uint16_t *sc = (const uint16_t *)scale + g * N * (K / 32);
+        const uint16_t *sc = (const uint16_t *)scale + g * N * (K / blk);
 #pragma omp parallel for schedule(static)
         for (int64_t k = 0; k < K; ++k)
             for (int64_t n = 0; n < N; ++n) {
                 uint8_t byte = wb[n * (K / 2) + (k >> 1)];
                 uint8_t code = (k & 1) ? (byte >> 4) : (byte & 15);
-                float v = orc_e2m1_decode(code) * bf16_to_f32(sc[n * (K / 32) + k / 32]);
+                float v = orc_e2m1_decode(code) * bf16_to_f32(sc[n * (K / blk) + k / blk]);
                 out[k * N + n] = round_bf16 ? bf16_to_f32(f32_to_bf16_rne(v)) : v;
             }
     } else if (fmt == ORC_FMT_BF16) {

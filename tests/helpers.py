@@ -8,8 +8,8 @@ import torch
 import oracle
 from oracle import layouts as L
 
-FORMATS = ["fp4", "fp8", "int8", "int4", "fp4_b32", "bf16"]
-GEMV_FORMATS = ["fp4", "fp8", "int4", "fp4_b32", "bf16"]
+FORMATS = ["fp4", "fp8", "int8", "int4", "fp4_b32", "bf16", "fp4_b16"]
+GEMV_FORMATS = ["fp4", "fp8", "int4", "fp4_b32", "bf16", "fp4_b16"]
 
 
 def bits(t: torch.Tensor) -> np.ndarray:
@@ -66,6 +66,11 @@ def make_weights(fmt: str, rng, G: int, K: int, N: int, group: int = 128):
         codes = rng.integers(0, 16, (G, N, K), dtype=np.uint8)
         w = L.pack_nibbles_last(codes)
         scale = bits(bf16_uniform(rng, 2.0 ** -8, 2.0 ** -2, (G, N, K // 32)))
+        return dict(weight=w, scale=scale, offset=None, scale_rows=1)
+    if fmt == "fp4_b16":
+        codes = rng.integers(0, 16, (G, N, K), dtype=np.uint8)
+        w = L.pack_nibbles_last(codes)
+        scale = bits(bf16_uniform(rng, 2.0 ** -8, 2.0 ** -2, (G, N, K // 16)))
         return dict(weight=w, scale=scale, offset=None, scale_rows=1)
     if fmt == "bf16":
         w = bits((torch.from_numpy(rng.standard_normal((G, N, K)).astype(np.float32)) * 0.02).to(torch.bfloat16))

@@ -12,7 +12,7 @@ import helpers as H
 
 pytestmark = pytest.mark.gpu
 
-K_STEP = {"fp4": 64, "fp8": 128, "int8": 64, "int4": 128, "fp4_b32": 128, "bf16": 64}
+K_STEP = {"fp4": 64, "fp8": 128, "int8": 64, "int4": 128, "fp4_b32": 128, "bf16": 64, "fp4_b16": 128}
 
 
 def _say(msg):
@@ -58,7 +58,7 @@ def test_random_gemm(fmt, regime):
 def test_random_gemv(fmt, regime):
     seed = zlib.crc32(f"rand-gemv/{fmt}/{regime}".encode())
     rng = np.random.default_rng(seed)
-    k_major = fmt in ("fp4_b32", "bf16")
+    k_major = fmt in ("fp4_b32", "bf16", "fp4_b16")
     for rep in range(2):
         G = int(rng.integers(1, 8))
         K = int(rng.integers(1, 9)) * (32 if k_major and rep == 0 else K_STEP[fmt] * (4 if rep else 1))

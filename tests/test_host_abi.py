@@ -31,7 +31,7 @@ def test_compute_type_strings():
     # "fp4" / "fp8" are the reference's values (grouped_gemm/src/grouped_gemm.cpp:129-135)
     assert mg.format_from_compute_type("fp4") == mg.FMT_FP4_REF
     assert mg.format_from_compute_type("fp8") == mg.FMT_FP8_REF
-    assert [mg.format_from_compute_type(s) for s in ("int8", "int4", "fp4_b32", "bf16")] == [2, 3, 4, 5]
+    assert [mg.format_from_compute_type(s) for s in ("int8", "int4", "fp4_b32", "bf16", "fp4_b16")] == [2, 3, 4, 5, 6]
     for bad in ("", "FP4", "fp16", "int2"):
         assert mg.format_from_compute_type(bad) == mg.ERR_BAD_FORMAT
     assert mg.lib.moe_format_from_compute_type(None) == mg.ERR_BAD_FORMAT
@@ -55,11 +55,11 @@ def gargs(fmt, M=8, K=256, N=512, G=2, scale_rows=None, **kw):
 @pytest.mark.parametrize("op", ["gemm", "gemv"])
 def test_grouped_validate_accepts_good_and_rejects_bad(op):
     val = getattr(mg.lib, f"moe_grouped_{op}_validate")
-    fmts = [0, 1, 2, 3, 4, 5] if op == "gemm" else [0, 1, 3, 4, 5]
+    fmts = [0, 1, 2, 3, 4, 5, 6] if op == "gemm" else [0, 1, 3, 4, 5, 6]
     for fmt in fmts:
         assert val(ctypes.byref(gargs(fmt))) == mg.MOE_OK, fmt
     assert val(None) == mg.ERR_NULL_POINTER
-    assert val(ctypes.byref(gargs(0, format=6))) == mg.ERR_BAD_FORMAT
+    assert val(ctypes.byref(gargs(0, format=7))) == mg.ERR_BAD_FORMAT
     assert val(ctypes.byref(gargs(0, format=-1))) == mg.ERR_BAD_FORMAT
     assert val(ctypes.byref(gargs(0, reserved=1))) == mg.ERR_BAD_FORMAT
     assert val(ctypes.byref(gargs(0, M=-1))) == mg.ERR_BAD_SHAPE

@@ -206,6 +206,22 @@ def test_expand_int8_int4_fp4b32_bf16_closed_forms():
     for g in range(G):
         got = oracle.expand_weight(oracle.FMT_FP4_B32, wb, bf16_bits(sb), None, g, True)
         assert np.array_equal(got, dq[g].T)
+    # fp4_b16: the same container with one scale per 16 k (the checkpoint orientation of
+    # test_group_gemm_fp4.py:46-64); equals the reference test's own dequant expression
+    # (do_dequant_b, :67-75: decode * b_s per block of 16) and the stand-alone block-16 dequant
+    s16 = torch.from_numpy(rng.uniform(2**-8, 2**-2, (G, N, K // 16)).astype(np.float32)).to(torch.bfloat16)
+    dq = oracle.dequant_fp4_bf16(wb.reshape(G * N, K // 2), bf16_bits(s16).reshape(G * N, K // 16), 16)
+    dq = oracle.bf16_bits_to_f32(dq).reshape(G, N, K)
+    lut = torch.tensor([0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0])
+    cbt = torch.from_numpy(cb.astype(np.int64))
+    vals = torch.where((cbt >> 3).bool(), -1.0, 1.0) * lut[cbt & 7]
+    ref16 = (vals.view(G, N, K // 16, 16) * s16.float().view(G, N, K // 16, 1)).view(G, N, K)
+    for g in range(G):
+        got = oracle.expand_weight(oracle.FMT_FP4_B16, wb, bf16_bits(s16), None, g, True)
+        assert np.array_equal(got, dq[g].T)
+        assert np.array_equal(got, ref16[g].to(torch.bfloat16).float().numpy().T)
+        got = oracle.expand_weight(oracle.FMT_FP4_B16, wb, bf16_bits(s16), None, g, False)
+        assert np.array_equal(got, ref16[g].numpy().T)
     # bf16 [G, N, K]
     wf = torch.randn(G, N, K, generator=torch.Generator().manual_seed(1)).to(torch.bfloat16)
     got = oracle.expand_weight(oracle.FMT_BF16, bf16_bits(wf), None, None, 1, True)
