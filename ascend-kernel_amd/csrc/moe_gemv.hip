@@ -436,7 +436,11 @@ __device__ __forceinline__ uint32_t e2m1_pair_bf16(uint32_t word, int sel) {
 // grouped GEMM op (grouped_matmul_antiquant.h:537-662: weights are RNE_bf16(e2m1 * scale), so the
 // scale has to be applied per element before the MFMA: ~2 VALU instructions per element) instead of
 // that of the GEMV op (fp32 weights: the scale is applied to the block's partial sum).
-template <int MB, bool ROUNDW>
+// BLK = k per scale (32 or 16).  With 16, a 32-k block of a lane's row has two scales: the lanes
+// q < 2 of a column hold its first half, q >= 2 the second, so with the GEMM's rounding each lane
+// simply uses its half's scale, and with the GEMV's arithmetic the block takes two MFMAs, each on
+// one half of the lanes' codes (the other half zeroed), each partial sum scaled by its own scale.
+template <int MB, bool ROUNDW, int BLK>
 __device__ __forceinline__ void gemv_fp4_mfma_rows(const uint8_t* __restrict__ wg, const uint16_t* __restrict__ sg,
                                                    const uint16_t* __restrict__ x, uint16_t* __restrict__ y,
                                                    u32x4_t* xs, int64_t row0, int mg, int n0, int N, int K) {
@@ -450,15 +454,17 @@ __device__ __forceinline__ void gemv_fp4_mfma_rows(const uint8_t* __restrict__ w
     // 32-bit byte offsets from the expert's (wavefront-uniform) base pointers: an expert's weight
     // slab is smaller than 4 GiB
     const uint32_t woff = (uint32_t)nn * (uint32_t)(K / 2) + q * 16;
-    const uint32_t soff = (uint32_t)nn * (uint32_t)(K / 32) * 2;
+    const uint32_t soff = (uint32_t)nn * (uint32_t)(K / BLK) * 2;
+    constexpr int PER = BLK / 8;                // loop iterations per 128 bytes (64 scales) of a scale row
+    const bool hi_half = (q & 2) != 0;          // block 16: this lane's codes belong to the second scale of a block
     f32x4_t acc = {0.f, 0.f, 0.f, 0.f}, acc2 = {0.f, 0.f, 0.f, 0.f};
 
     for (int kc0 = 0; kc0 < K; kc0 += KC) {
         const int klen = min(KC, K - kc0);
         const int niter = klen / GF_KSTEP;             // iterations of U groups
-        const int nblk = klen / 32;                    // scale blocks of the chunk (>= 16)
+        const int nblk = klen / BLK;                   // scales of the chunk (>= 16)
         const uint8_t* wp = wg + (kc0 >> 1);                                   // group c of the chunk: + 64 c bytes
-        const uint8_t* sp = reinterpret_cast<const uint8_t*>(sg) + (kc0 >> 5) * 2;   // block b of the chunk: + 2 b bytes
+        const uint8_t* sp = reinterpret_cast<const uint8_t*>(sg) + (kc0 / BLK) * 2;  // scale b of the chunk: + 2 b bytes
         // x fragment of block 4 c + j: unit (16 c + 4 j + q) ^ r of row r = xj[j][16 c].  MFMA rows
         // >= MB read row i % MB again: their products land in accumulator rows that are not stored.
         const int r = i % MB;
@@ -468,14 +474,29 @@ __device__ __forceinline__ void gemv_fp4_mfma_rows(const uint8_t* __restrict__ w
 
         // one 128-k group: w = this lane's 16 bytes (block 4 c + q of its row), s0/s1 = the 4 scales of
         // blocks 4 c .. 4 c + 3 as two bf16 pairs
-        auto group = [&](const u32x4_t& w, uint32_t s0, uint32_t s1, int c) {
+        auto group = [&](const u32x4_t& w, const uint32_t (&sd)[BLK == 32 ? 2 : 4], int c) {
             // 4x4 transpose of the dwords over the q lanes: b[j] = this lane's 8 codes of block 4 c + j
             const u32x2_t t02 = __builtin_amdgcn_permlane32_swap(w[0], w[2], false, false);
             const u32x2_t t13 = __builtin_amdgcn_permlane32_swap(w[1], w[3], false, false);
             const u32x2_t b01 = __builtin_amdgcn_permlane16_swap(t02[0], t13[0], false, false);
             const u32x2_t b23 = __builtin_amdgcn_permlane16_swap(t02[1], t13[1], false, false);
             const uint32_t b[4] = {b01[0], b01[1], b23[0], b23[1]};
-            const float s[4] = {bf16_lo(s0), bf16_hi(s0), bf16_lo(s1), bf16_hi(s1)};
+            // s[j]: block 32: the scale of block j; block 16: the scale of this lane's half of block j
+            // (ROUNDW) / of the first half (else), s2[j] that of the second half
+            float s[4], s2[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                if constexpr (BLK == 32) {
+                    s[j] = (j & 1) ? bf16_hi(sd[j >> 1]) : bf16_lo(sd[j >> 1]);
+                    s2[j] = 0.f;
+                } else if constexpr (ROUNDW) {
+                    s[j] = hi_half ? bf16_hi(sd[j]) : bf16_lo(sd[j]);
+                    s2[j] = 0.f;
+                } else {
+                    s[j] = bf16_lo(sd[j]);
+                    s2[j] = bf16_hi(sd[j]);
+                }
+            }
             // two blocks at a time: enough independent MFMAs to cover their latency, few enough
             // live registers for 4 wavefronts per SIMD
 #pragma unroll
@@ -496,6 +517,27 @@ __device__ __forceinline__ void gemv_fp4_mfma_rows(const uint8_t* __restrict__ w
                                                                   __builtin_bit_cast(bf16x8_t, bw[0]), acc, 0, 0, 0);
                     acc2 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, aw[1]),
                                                                    __builtin_bit_cast(bf16x8_t, bw[1]), acc2, 0, 0, 0);
+                } else if constexpr (BLK == 16) {
+                    // per block: first-half lanes' codes, then second-half lanes' codes
+                    const uint32_t keep_lo = hi_half ? 0u : 0xffffffffu;
+#pragma unroll
+                    for (int j = 0; j < 2; ++j) {
+                        u32x4_t b_lo, b_hi;
+#pragma unroll
+                        for (int d = 0; d < 4; ++d) {
+                            b_lo[d] = e2m1_pair_bf16(b[j0 + j] & keep_lo, d);
+                            b_hi[d] = e2m1_pair_bf16(b[j0 + j] & ~keep_lo, d);
+                        }
+                        const f32x4_t p_lo = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                            __builtin_bit_cast(bf16x8_t, aw[j]), __builtin_bit_cast(bf16x8_t, b_lo), f32x4_t{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+                        const f32x4_t p_hi = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                            __builtin_bit_cast(bf16x8_t, aw[j]), __builtin_bit_cast(bf16x8_t, b_hi), f32x4_t{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+#pragma unroll
+                        for (int rr = 0; rr < 4; ++rr) {
+                            acc[rr] = fmaf(p_lo[rr], s[j0 + j], acc[rr]);
+                            acc2[rr] = fmaf(p_hi[rr], s2[j0 + j], acc2[rr]);
+                        }
+                    }
                 } else {
                     f32x4_t part[2];
 #pragma unroll
@@ -519,29 +561,39 @@ __device__ __forceinline__ void gemv_fp4_mfma_rows(const uint8_t* __restrict__ w
             for (int u = 0; u < U; ++u)
                 w[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(wp + (woff + (uint32_t)((it * U + u) * 64))));
         };
-        // the 16 scales of iteration 4 T + q of this lane's row (clamped into the chunk: iterations
-        // past its end do not exist)
+        // scales 64 T + 16 q .. + 15 of this lane's row in the chunk: those of iteration 4 T + q (block 32)
+        // or of half of iteration 2 T + (q >> 1) (block 16); clamped into the chunk (iterations past its
+        // end do not exist)
         auto fetch_s = [&](u32x4_t (&sv)[2], int T) {
             const int b0 = min(64 * T + 16 * q, nblk - 16);
             sv[0] = *reinterpret_cast<const u32x4_t*>(sp + (soff + (uint32_t)(b0 * 2)));
             sv[1] = *reinterpret_cast<const u32x4_t*>(sp + (soff + (uint32_t)(b0 * 2 + 16)));
         };
         u32x4_t sc[2], sn[2];
-        // iteration `it` on the weights in w; rotates the scale registers every 4 iterations
+        // iteration `it` on the weights in w; rotates the scale registers every PER iterations
         auto iteration = [&](const u32x4_t (&w)[U], int it) {
-            const int t = it & 3;
+            const int t = it & (PER - 1);
             if (t == 0) {
                 sc[0] = sn[0];
                 sc[1] = sn[1];
-                if (it + 4 < niter) fetch_s(sn, (it >> 2) + 1);
+                if (it + PER < niter) fetch_s(sn, it / PER + 1);
             }
-            // this iteration's scales live in lane (i, t)
-            const int src = (16 * t + i) * 4;
 #pragma unroll
             for (int u = 0; u < U; ++u) {
-                const uint32_t s0 = (uint32_t)__builtin_amdgcn_ds_bpermute(src, (int)sc[u >> 1][2 * (u & 1)]);
-                const uint32_t s1 = (uint32_t)__builtin_amdgcn_ds_bpermute(src, (int)sc[u >> 1][2 * (u & 1) + 1]);
-                group(w[u], s0, s1, it * U + u);
+                if constexpr (BLK == 32) {
+                    // this iteration's scales live in lane (i, t): 2 dwords per group
+                    const int src = (16 * t + i) * 4;
+                    const uint32_t sd[2] = {(uint32_t)__builtin_amdgcn_ds_bpermute(src, (int)sc[u >> 1][2 * (u & 1)]),
+                                            (uint32_t)__builtin_amdgcn_ds_bpermute(src, (int)sc[u >> 1][2 * (u & 1) + 1])};
+                    group(w[u], sd, it * U + u);
+                } else {
+                    // groups 0, 1 of the iteration live in lane (i, 2 t), groups 2, 3 in lane (i, 2 t + 1): 4 dwords each
+                    const int src = (16 * (2 * t + (u >> 1)) + i) * 4;
+                    uint32_t sd[4];
+#pragma unroll
+                    for (int d = 0; d < 4; ++d) sd[d] = (uint32_t)__builtin_amdgcn_ds_bpermute(src, (int)sc[u & 1][d]);
+                    group(w[u], sd, it * U + u);
+                }
             }
         };
         // two register sets of weights: the loads of iteration it + 1 are in flight behind iteration it
@@ -574,7 +626,7 @@ __device__ __forceinline__ void gemv_fp4_mfma_rows(const uint8_t* __restrict__ w
     }
 }
 
-template <bool ROUNDW>
+template <bool ROUNDW, int BLK>
 __global__ __launch_bounds__(64 * GF_WAVES, 4) void gemv_fp4_mfma_kernel(const uint16_t* __restrict__ x,
                                                                          const uint8_t* __restrict__ w,
                                                                          const uint16_t* __restrict__ scale,
@@ -587,19 +639,19 @@ __global__ __launch_bounds__(64 * GF_WAVES, 4) void gemv_fp4_mfma_kernel(const u
     group_rows(gl, g, M, start, end);
     if (end <= start) return;
     const uint8_t* wg = w + (int64_t)g * N * ((int64_t)K / 2);
-    const uint16_t* sg = scale + (int64_t)g * N * (K / 32);
+    const uint16_t* sg = scale + (int64_t)g * N * (K / BLK);
     for (int64_t row0 = start; row0 < end; row0 += GF_ROWS) {
         const int mg = (int)min((int64_t)GF_ROWS, end - row0);
-        if (mg <= 4) gemv_fp4_mfma_rows<4, ROUNDW>(wg, sg, x, y, xs, row0, mg, n0, N, K);
-        else if (mg <= 8) gemv_fp4_mfma_rows<8, ROUNDW>(wg, sg, x, y, xs, row0, mg, n0, N, K);
-        else gemv_fp4_mfma_rows<16, ROUNDW>(wg, sg, x, y, xs, row0, mg, n0, N, K);
+        if (mg <= 4) gemv_fp4_mfma_rows<4, ROUNDW, BLK>(wg, sg, x, y, xs, row0, mg, n0, N, K);
+        else if (mg <= 8) gemv_fp4_mfma_rows<8, ROUNDW, BLK>(wg, sg, x, y, xs, row0, mg, n0, N, K);
+        else gemv_fp4_mfma_rows<16, ROUNDW, BLK>(wg, sg, x, y, xs, row0, mg, n0, N, K);
     }
 }
 
-template <bool ROUNDW>
+template <bool ROUNDW, int BLK>
 static int launch_fp4_mfma(const moe_grouped_args* a, hipStream_t stream) {
     dim3 grid((unsigned)((a->N + GF_NR_WG - 1) / GF_NR_WG), (unsigned)a->G);
-    hipLaunchKernelGGL(gemv_fp4_mfma_kernel<ROUNDW>, grid, dim3(64 * GF_WAVES), (size_t)GF_LDS_UNITS * 16, stream,
+    hipLaunchKernelGGL((gemv_fp4_mfma_kernel<ROUNDW, BLK>), grid, dim3(64 * GF_WAVES), (size_t)GF_LDS_UNITS * 16, stream,
                        static_cast<const uint16_t*>(a->x), static_cast<const uint8_t*>(a->weight),
                        static_cast<const uint16_t*>(a->scale), a->group_list, static_cast<uint16_t*>(a->y), a->M,
                        (int)a->K, (int)a->N);
@@ -644,7 +696,8 @@ bool gemv_preferred(const moe_grouped_args* a) {
     // pass over its weights (same arithmetic as the GEMM: the weights are bf16 already).  The
     // matrix-core fp4_b32 kernel takes 16 and has a variant with the GEMM's weight rounding; the
     // bound is where the small-tile GEMM kernel overtakes it (measured at DeepSeek-V3 shapes).
-    if (a->format == MOE_FMT_FP4_B32) return a->K % GF_KSTEP == 0 && a->M <= GF_GEMM_ROWS_PER_EXPERT * a->G;
+    if (a->format == MOE_FMT_FP4_B32 || a->format == MOE_FMT_FP4_B16)
+        return a->K % GF_KSTEP == 0 && a->M <= GF_GEMM_ROWS_PER_EXPERT * a->G;
     if (a->format == MOE_FMT_BF16) return a->M <= 4 * a->G;
     return false;
 }
@@ -655,8 +708,10 @@ int launch_grouped_gemv(const moe_grouped_args* a, hipStream_t stream, bool gemm
         case MOE_FMT_FP4_B32:
             // the matrix-core kernel takes K in whole loop iterations
             if (a->K % GF_KSTEP != 0) return gemm_rounding ? MOE_ERR_BAD_SHAPE : launch_kmajor<MOE_FMT_FP4_B32>(a, stream);
-            return gemm_rounding ? launch_fp4_mfma<true>(a, stream) : launch_fp4_mfma<false>(a, stream);
-        case MOE_FMT_FP4_B16: return gemm_rounding ? MOE_ERR_BAD_SHAPE : launch_kmajor<MOE_FMT_FP4_B16>(a, stream);
+            return gemm_rounding ? launch_fp4_mfma<true, 32>(a, stream) : launch_fp4_mfma<false, 32>(a, stream);
+        case MOE_FMT_FP4_B16:
+            if (a->K % GF_KSTEP != 0) return gemm_rounding ? MOE_ERR_BAD_SHAPE : launch_kmajor<MOE_FMT_FP4_B16>(a, stream);
+            return gemm_rounding ? launch_fp4_mfma<true, 16>(a, stream) : launch_fp4_mfma<false, 16>(a, stream);
         case MOE_FMT_FP4_REF: return launch_nmajor<MOE_FMT_FP4_REF>(a, stream);
         case MOE_FMT_FP8_REF: return launch_nmajor<MOE_FMT_FP8_REF>(a, stream);
         case MOE_FMT_INT4: return launch_nmajor<MOE_FMT_INT4>(a, stream);

@@ -241,24 +241,25 @@ def test_gemv_parity_decode_shapes(fmt, K, N):
     H.assert_close(got, H.oracle_out(case, gemv=True), what=f"gemv {fmt} K={K} N={N}")
 
 
+@pytest.mark.parametrize("fmt", ["fp4_b32", "fp4_b16"])
 @pytest.mark.parametrize("K,N", [(1024, 256), (7168, 256), (8192 + 512, 256), (192, 256)])
-def test_gemv_fp4_b32_row_counts_up_to_and_beyond_16(K, N):
-    """The fp4_b32 GEMV multiplies up to 16 rows of an expert per pass on the matrix cores (staging
+def test_gemv_fp4_b32_row_counts_up_to_and_beyond_16(K, N, fmt):
+    """The K-contiguous fp4 GEMV (scales per 32 or per 16 k) multiplies up to 16 rows of an expert per pass on the matrix cores (staging
     4, 8 or 16 rows) and takes more rows 16 at a time; K = 192 is not a multiple of 512 and goes
     through the vector path."""
-    _say(f"gemv fp4_b32 rows K={K} N={N}")
+    _say(f"gemv {fmt} rows K={K} N={N}")
     counts = [1, 0, 4, 5, 8, 9, 16, 17, 40, 0, 3]
     gl = list(np.cumsum(counts))
-    case = H.make_case("fp4_b32", len(gl), K, N, gl, seed=K + N, extra_rows=2)
+    case = H.make_case(fmt, len(gl), K, N, gl, seed=K + N, extra_rows=2)
     dev = H.upload(case)
     got = H.run_cabi(case, dev, "gemv")
-    H.assert_close(got, H.oracle_out(case, gemv=True), rows=slice(0, gl[-1]), what=f"gemv fp4_b32 rows K={K} N={N}")
+    H.assert_close(got, H.oracle_out(case, gemv=True), rows=slice(0, gl[-1]), what=f"gemv {fmt} rows K={K} N={N}")
     assert (got[gl[-1]:] == 0x7FC0).all()
     if K % 128:
-        return  # the GEMM op takes fp4_b32 with K % 128 == 0 only
+        return  # the GEMM op takes these containers with K % 128 == 0 only
     # the grouped GEMM op at these sizes runs the same kernel with the GEMM's weight rounding
     got = H.run_cabi(case, dev, "gemm")
-    H.assert_close(got, H.oracle_out(case), rows=slice(0, gl[-1]), what=f"gemm fp4_b32 rows K={K} N={N}")
+    H.assert_close(got, H.oracle_out(case), rows=slice(0, gl[-1]), what=f"gemm {fmt} rows K={K} N={N}")
     assert (got[gl[-1]:] == 0x7FC0).all()
 
 
