@@ -41,11 +41,17 @@ __device__ __forceinline__ uint32_t e2m1_pair_scaled_bf16(uint32_t word, float s
     return pack_bf16_rne(v[0] * scale, v[1] * scale);
 }
 
-// e4m3 decode the way the reference does it (no NaN: 0x7F / 0xFF give +-480):
-// sign -> bit 31, low 7 bits -> bits 26:20 of an fp32 pattern, times 2^120.
-__device__ __forceinline__ float e4m3_ref_to_f32(uint32_t code) {
-    uint32_t bits = ((code & 0x80u) << 24) | ((code & 0x7fu) << 20);
-    return __uint_as_float(bits) * 0x1p120f;
+// Two e4m3 codes decoded the way the reference does it (no NaN: 0x7F / 0xFF give +-480), returned
+// as value / 256.  `pair` holds the codes in bytes 0 and 2, bytes 1 and 3 zero.  code << 7 with
+// the sign moved from bit 14 to bit 15 is an fp16 worth 2^-8 of the e4m3 value, subnormals
+// included (preCastFP8Weight, grouped_gemm/op_kernel/antiquant_impl.h:87-129, does the same);
+// fp16 -> fp32 is exact, so callers fold the 2^8 into their scale and round once.
+__device__ __forceinline__ f32x2_t e4m3_ref_pair_over_256(uint32_t pair) {
+    typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+    uint32_t h = pair << 7;
+    h += h & 0x40004000u;
+    const half2_t v = __builtin_bit_cast(half2_t, h);
+    return f32x2_t{(float)v[0], (float)v[1]};
 }
 
 __device__ __forceinline__ float wave_reduce_sum(float v) {

@@ -317,19 +317,13 @@ struct BTraits<MOE_FMT_FP8_REF> : BTraitsByte<MOE_FMT_FP8_REF> {
     struct Dq {
         __device__ __forceinline__ void init_tile(const BCtx&) {}
         __device__ __forceinline__ void prep(const Raw&, const BCtx&, int) {}
-        // Both k rows of a pair at once, through fp16 as the reference kernel does
-        // (preCastFP8Weight, grouped_gemm/op_kernel/antiquant_impl.h:87-129): code << 7 with the sign moved
-        // up one bit is an fp16 worth 2^-8 of the e4m3 value (0x7F / 0xFF give +-480 / 256, no NaN);
-        // fp16 -> fp32 is exact and the 2^8 goes into the block scale, so the product rounds once.
+        // both k rows of a pair at once (see e4m3_ref_pair_over_256): the 2^8 goes into the block scale
         __device__ __forceinline__ void unit(const Raw& raw, const BCtx&, int s, int p, int t, u32x4_t out[4]) {
-            typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
             const uint32_t a = pinned(raw.r[s][2 * p]), b = raw.r[s][2 * p + 1];
             const uint32_t sel = (uint32_t)t | 0x0c00u | ((uint32_t)(4 + t) << 16) | 0x0c000000u;   // [a.byte t, 0, b.byte t, 0]
-            uint32_t h = __builtin_amdgcn_perm(b, a, sel) << 7;
-            h += h & 0x40004000u;                        // sign: bit 14 -> bit 15 of each half
-            const half2_t v = __builtin_bit_cast(half2_t, h);
+            const f32x2_t v = e4m3_ref_pair_over_256(__builtin_amdgcn_perm(b, a, sel));
             const float sc = raw.s8[s] * 256.f;
-            out[t][p] = pinned(pack_bf16_rne((float)v[0] * sc, (float)v[1] * sc));
+            out[t][p] = pinned(pack_bf16_rne(v[0] * sc, v[1] * sc));
         }
     };
 };

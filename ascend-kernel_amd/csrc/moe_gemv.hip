@@ -257,17 +257,13 @@ __device__ __forceinline__ void gemv_nmajor_rows(const uint8_t* __restrict__ wg,
             float xr[MG];
 #pragma unroll
             for (int r = 0; r < MG; ++r) xr[r] = bf16_bits_to_f32(xs[r * K + k]);
-            // two codes at a time through fp16 (code << 7 with the sign moved up one bit is an fp16 worth
-            // 2^-8 of the e4m3 value, 0x7F / 0xFF included; gemv_impl.h:88-130 does the same)
-            typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+            // two codes at a time (see e4m3_ref_pair_over_256)
             const float s256 = s * 256.f;
 #pragma unroll
             for (int c = 0; c < 16; c += 2) {
                 const uint32_t sel = (uint32_t)(c & 3) | 0x0c00u | ((uint32_t)((c & 3) + 1) << 16) | 0x0c000000u;
-                uint32_t h = __builtin_amdgcn_perm(0u, wv[c >> 2], sel) << 7;
-                h += h & 0x40004000u;
-                const half2_t v = __builtin_bit_cast(half2_t, h);
-                const float w0 = (float)v[0] * s256, w1 = (float)v[1] * s256;
+                const f32x2_t v = e4m3_ref_pair_over_256(__builtin_amdgcn_perm(0u, wv[c >> 2], sel));
+                const float w0 = v[0] * s256, w1 = v[1] * s256;
 #pragma unroll
                 for (int r = 0; r < MG; ++r) {
                     acc[r][c] = fmaf(xr[r], w0, acc[r][c]);
