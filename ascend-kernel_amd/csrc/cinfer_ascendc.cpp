@@ -48,7 +48,8 @@ int parse_format(const char* computeType) {
 
 // Fills args from the tensors; returns the logical (K, N) through args.
 void fill_grouped(moe_grouped_args& a, const at::Tensor& x, const at::Tensor& weight, const at::Tensor& scale,
-                  const at::Tensor* offset, const at::Tensor& groupList, int fmt, const at::Tensor& output) {
+                  const at::Tensor* offset, const at::Tensor& groupList, int fmt, const at::Tensor& output,
+                  int epilogue = MOE_EPILOGUE_NONE) {
     if (!x.defined() || !x.is_cuda()) fail("x must be a GPU tensor");
     check_tensor(x, "x", at::kBFloat16, 2, x);
     check_tensor(output, "output", at::kBFloat16, 2, x);
@@ -116,7 +117,7 @@ void fill_grouped(moe_grouped_args& a, const at::Tensor& x, const at::Tensor& we
             want(weight, "weight", {G, N, K});
             break;
     }
-    want(output, "output", {M, N});
+    want(output, "output", {M, epilogue == MOE_EPILOGUE_SWIGLU ? N / 2 : N});
     a.x = x.data_ptr();
     a.weight = weight.data_ptr();
     a.scale = fmt == MOE_FMT_BF16 ? nullptr : scale.data_ptr();
@@ -126,7 +127,7 @@ void fill_grouped(moe_grouped_args& a, const at::Tensor& x, const at::Tensor& we
     a.M = M; a.K = K; a.N = N; a.G = G;
     a.scale_rows = scale_rows;
     a.format = fmt;
-    a.reserved = 0;
+    a.epilogue = epilogue;
 }
 
 moe_stream_t current_stream(const at::Tensor& x) {
@@ -142,6 +143,19 @@ void GroupedGemm(at::Tensor x, at::Tensor weight, at::Tensor antiquantScaleOptio
     fill_grouped(a, x, weight, antiquantScaleOptional, &antiquantOffsetOptional, groupListOptional, fmt, output);
     c10::DeviceGuard guard(x.device());
     check_status(moe_grouped_gemm(&a, current_stream(x)), "grouped_gemm");
+}
+
+// Extra entry point: grouped_gemm with the SwiGLU activation fused into its epilogue (see moe_epilogue in
+// moe_gfx950.h): weight columns in groups of (gate 2j, gate 2j+1, up 2j, up 2j+1), output [M, N/2].
+void GroupedGemmSwiglu(at::Tensor x, at::Tensor weight, at::Tensor antiquantScaleOptional,
+                       at::Tensor antiquantOffsetOptional, at::Tensor groupListOptional, const char* computeType,
+                       at::Tensor output) {
+    const int fmt = parse_format(computeType);
+    moe_grouped_args a;
+    fill_grouped(a, x, weight, antiquantScaleOptional, &antiquantOffsetOptional, groupListOptional, fmt, output,
+                 MOE_EPILOGUE_SWIGLU);
+    c10::DeviceGuard guard(x.device());
+    check_status(moe_grouped_gemm(&a, current_stream(x)), "grouped_gemm_swiglu");
 }
 
 // pybind.cpp:14-16
@@ -261,6 +275,9 @@ PYBIND11_MODULE(cinfer_ascendc, m) {
           "output"_a, "GROUP GEMV.");
     m.def("grouped_gemm", &GroupedGemm, "x"_a, "weight"_a, "antiquantScaleOptional"_a, "antiquantOffsetOptional"_a,
           "groupListOptional"_a, "computeType"_a, "output"_a, "GROUP GEMM.");
+    m.def("grouped_gemm_swiglu", &GroupedGemmSwiglu, "x"_a, "weight"_a, "antiquantScaleOptional"_a,
+          "antiquantOffsetOptional"_a, "groupListOptional"_a, "computeType"_a, "output"_a,
+          "GROUP GEMM with silu(gate) * up fused into the epilogue; output [M, N/2].");
     m.def("dequant_fp4", &DequantFp4, "weight"_a, "scale"_a, "output"_a, "FP4 (e2m1) -> BF16 block dequant.");
     m.def("moe_route", &MoeRoute, "logits"_a, "x"_a, "topk"_a,
           "Router logits -> (x_sorted, group_list, topk_weight, topk_ids, row_of_choice).");

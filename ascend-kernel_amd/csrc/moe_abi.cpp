@@ -13,9 +13,15 @@ inline bool fits_i32(int64_t v) { return v >= 0 && v <= 0x7fffffffLL; }
 
 // Checks shared by GEMM and GEMV.  k_mult / n_mult are what the op's kernels
 // need on top of what the container itself implies.
-int validate_grouped(const moe_grouped_args* a, int64_t k_mult, int64_t n_mult) {
+int validate_grouped(const moe_grouped_args* a, int64_t k_mult, int64_t n_mult, bool allow_epilogue) {
     if (!a) return MOE_ERR_NULL_POINTER;
-    if (a->format < 0 || a->format >= MOE_FMT_COUNT || a->reserved != 0) return MOE_ERR_BAD_FORMAT;
+    if (a->format < 0 || a->format >= MOE_FMT_COUNT) return MOE_ERR_BAD_FORMAT;
+    if (a->epilogue != MOE_EPILOGUE_NONE) {
+        // the fused activation lives in the GEMM kernels' epilogue for containers whose lanes own 4 adjacent columns
+        const bool n_contiguous = a->format == MOE_FMT_FP4_REF || a->format == MOE_FMT_FP8_REF ||
+                                  a->format == MOE_FMT_INT8 || a->format == MOE_FMT_INT4;
+        if (a->epilogue != MOE_EPILOGUE_SWIGLU || !allow_epilogue || !n_contiguous) return MOE_ERR_BAD_FORMAT;
+    }
     if (a->M < 0 || a->K <= 0 || a->N <= 0 || a->G <= 0) return MOE_ERR_BAD_SHAPE;
     // same limit as the reference: grouped_matmul_antiquant_tiling.cpp:260-264
     if (!fits_i32(a->M) || !fits_i32(a->K) || !fits_i32(a->N) || !fits_i32(a->G)) return MOE_ERR_TOO_LARGE;
@@ -98,7 +104,7 @@ int moe_dequant_fp4_bf16_validate(const moe_dequant_args* a) {
 int moe_grouped_gemm_validate(const moe_grouped_args* a) {
     // the fp4_b32 tile routine steps through K 128 at a time
     const bool fp4_k = a && (a->format == MOE_FMT_FP4_B32 || a->format == MOE_FMT_FP4_B16);
-    return validate_grouped(a, fp4_k ? 128 : 64, 256);
+    return validate_grouped(a, fp4_k ? 128 : 64, 256, true);
 }
 
 // GEMV: N-contiguous containers are read 256 columns per wavefront step,
@@ -106,7 +112,7 @@ int moe_grouped_gemm_validate(const moe_grouped_args* a) {
 int moe_grouped_gemv_validate(const moe_grouped_args* a) {
     if (a && a->format == MOE_FMT_INT8) return MOE_ERR_BAD_FORMAT;  // the GEMV op has no offset operand
     const bool k_major = a && (a->format == MOE_FMT_BF16 || a->format == MOE_FMT_FP4_B32 || a->format == MOE_FMT_FP4_B16);
-    return validate_grouped(a, k_major ? 32 : 64, k_major ? 1 : 256);
+    return validate_grouped(a, k_major ? 32 : 64, k_major ? 1 : 256, false);
 }
 
 int moe_prepack_fp4_ref_validate(const moe_prepack_fp4_args* a) {

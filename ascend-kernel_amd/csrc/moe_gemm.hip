@@ -42,6 +42,7 @@ struct GemmParams {
     uint16_t* y;
     int64_t M;
     int K, N, G, scale_rows;
+    int epilogue;   // moe_epilogue
 };
 
 // Buffer resources keep the addressing compact: one 128-bit descriptor in SGPRs per
@@ -75,6 +76,11 @@ __device__ __forceinline__ void mfma_16x16x32(f32x4_t& acc, const u32x4_t& a, co
 // the whole unified register file as VGPRs (otherwise the compiler splits it in two halves).
 __device__ __forceinline__ void mfma_16x16x32_v(f32x4_t& acc, const u32x4_t& a, const u32x4_t& b) {
     asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+v"(acc) : "v"(a), "v"(b));
+}
+
+// silu(g) * u on fp32 accumulators: g / (1 + exp(-g)) with the hardware exp and reciprocal.
+__device__ __forceinline__ float swiglu(float g, float u) {
+    return g * __builtin_amdgcn_rcpf(1.f + __expf(-g)) * u;
 }
 
 // Ties a value to the chain of volatile asm statements (the MFMAs): whatever is computed
@@ -489,6 +495,20 @@ __device__ __forceinline__ void store_tile(const GemmParams& P, const BCtx& c, f
                                FMT == MOE_FMT_FP8_REF);
     // through a buffer resource that ends after the tile's last valid row: stores to padded
     // rows fall outside it and are dropped
+    if (N_CONTIG && P.epilogue == MOE_EPILOGUE_SWIGLU) {
+        // this lane's 4 columns are (gate, gate, up, up) of 2 output columns; y has N / 2 columns
+        const int NO = P.N >> 1;
+        const rsrc_t ro = make_rsrc(P.y + row0 * (int64_t)NO, (int64_t)rows * NO * 2);
+        const int vo = (4 * c.q * NO + ((n0 + T::col(c, 0)) >> 1)) * 2;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                __builtin_amdgcn_raw_buffer_store_b32(
+                    pack_bf16_rne(swiglu(acc[mt][0][r], acc[mt][2][r]), swiglu(acc[mt][1][r], acc[mt][3][r])), ro, vo,
+                    (16 * mt + r) * NO * 2, 0);
+        return;
+    }
     const rsrc_t ry = make_rsrc(P.y + row0 * (int64_t)P.N, (int64_t)rows * P.N * 2);
     const int vy = (4 * c.q * P.N + n0) * 2;
 #pragma unroll
@@ -979,7 +999,19 @@ __device__ __forceinline__ void gemm_tile_pair_int4(const GemmParams& P, u32x4_t
         if (rd < ROUNDS) __syncthreads();
     }
 
-    if (h == 0) {
+    if (h == 0 && P.epilogue == MOE_EPILOGUE_SWIGLU) {
+        // this lane's 4 columns are (gate, gate, up, up) of 2 output columns; y has N / 2 columns
+        const int NO = P.N >> 1;
+        const rsrc_t ro = make_rsrc(P.y + row0 * (int64_t)NO, (int64_t)rows * NO * 2);
+        const int vo = (4 * q * NO + ((n0 + col0) >> 1)) * 2;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                __builtin_amdgcn_raw_buffer_store_b32(
+                    pack_bf16_rne(swiglu(acc[mt][0][r], acc[mt][2][r]), swiglu(acc[mt][1][r], acc[mt][3][r])), ro, vo,
+                    (16 * mt + r) * NO * 2, 0);
+    } else if (h == 0) {
         // epilogue through a buffer resource that ends after the tile's last valid row: stores to
         // padded rows fall outside it and are dropped
         const rsrc_t ry = make_rsrc(P.y + row0 * (int64_t)P.N, (int64_t)rows * P.N * 2);
@@ -1198,6 +1230,7 @@ static int launch_gemm_fmt(const moe_grouped_args* a, hipStream_t stream) {
     P.gl = a->group_list;
     P.y = static_cast<uint16_t*>(a->y);
     P.M = a->M; P.K = (int)a->K; P.N = (int)a->N; P.G = (int)a->G; P.scale_rows = (int)a->scale_rows;
+    P.epilogue = a->epilogue;
     // Decode-like batches (on average at most 24 rows per expert; group_list itself stays on the
     // device) are HBM bound: use the small-tile kernel.  An expert with more than 32 rows then
     // costs one pass over its weights per 32 rows.

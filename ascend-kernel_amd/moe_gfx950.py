@@ -14,6 +14,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libmoe_gfx950.so")
 
 MOE_OK = 0
+EPILOGUE_NONE, EPILOGUE_SWIGLU = 0, 1
 FMT_FP4_REF, FMT_FP8_REF, FMT_INT8, FMT_INT4, FMT_FP4_B32, FMT_BF16, FMT_FP4_B16 = range(7)
 ERR_NULL_POINTER, ERR_BAD_FORMAT, ERR_BAD_SHAPE, ERR_BAD_ALIGNMENT, ERR_TOO_LARGE, ERR_LAUNCH, ERR_NO_DEVICE = (
     -1, -2, -3, -4, -5, -6, -7)
@@ -33,7 +34,7 @@ class GroupedArgs(ctypes.Structure):
     _fields_ = [("x", ctypes.c_void_p), ("weight", ctypes.c_void_p), ("scale", ctypes.c_void_p),
                 ("offset", ctypes.c_void_p), ("group_list", ctypes.c_void_p), ("y", ctypes.c_void_p),
                 ("M", ctypes.c_int64), ("K", ctypes.c_int64), ("N", ctypes.c_int64), ("G", ctypes.c_int64),
-                ("scale_rows", ctypes.c_int64), ("format", ctypes.c_int32), ("reserved", ctypes.c_int32)]
+                ("scale_rows", ctypes.c_int64), ("format", ctypes.c_int32), ("epilogue", ctypes.c_int32)]
 
 
 class DequantArgs(ctypes.Structure):
@@ -103,9 +104,9 @@ def dequant_fp4_bf16(codes_ptr: int, scale_ptr: int, out_ptr: int, rows: int, co
 
 
 def grouped_args(fmt: int, x_ptr: int, w_ptr: int, scale_ptr, offset_ptr, gl_ptr: int, y_ptr: int, M: int, K: int,
-                 N: int, G: int, scale_rows: int = 1) -> GroupedArgs:
+                 N: int, G: int, scale_rows: int = 1, epilogue: int = EPILOGUE_NONE) -> GroupedArgs:
     return GroupedArgs(x_ptr, w_ptr, scale_ptr or None, offset_ptr or None, gl_ptr, y_ptr, M, K, N, G, scale_rows,
-                       fmt, 0)
+                       fmt, epilogue)
 
 
 def grouped_gemm(args: GroupedArgs, stream: int = 0) -> None:

@@ -373,6 +373,21 @@ def main():
                     kernel="moe::grouped_gemm_kernel<int4>",
                     per_launch={n: dict(us=t * 1e6, TFLOPs=f / t / 1e12, frac=f / t / 1e12 / PEAK_BF16_TFLOPS)
                                 for n, t, f in zip(wl["names"], t_each, wl["flops"])})
+    # gate_up with the SwiGLU activation fused into its epilogue (same tensors; the weight columns are then read as
+    # groups of (gate, gate, up, up)): writes [M, N/2] instead of [M, N] and spares a separate activation pass
+    fused = None
+    if not args.no_extra:
+        gu = ops[0]
+        xg, wg, sg, _, glg, yg = gu.keep
+        y_half = torch.empty(yg.shape[0], yg.shape[1] // 2, dtype=torch.bfloat16, device="cuda")
+        a = mg.grouped_args(mg.format_from_compute_type("int4"), xg.data_ptr(), wg.data_ptr(), sg.data_ptr(), 0,
+                            glg.data_ptr(), y_half.data_ptr(), xg.shape[0], xg.shape[1], yg.shape[1], glg.shape[0],
+                            xg.shape[1] // 128, epilogue=mg.EPILOGUE_SWIGLU)
+        t_plain, t_fused = time_launches(
+            torch, [gu, lambda: mg.grouped_gemm(a, torch.cuda.current_stream().cuda_stream)], args.steps, 1)
+        fused = dict(us=t_fused * 1e6, plain_us=t_plain * 1e6, TFLOPs=wl["flops"][0] / t_fused / 1e12,
+                     y_bytes_saved=int(yg.numel()))   # bf16 [M, N] -> [M, N/2]
+        del y_half
     del wl, ops
     torch.cuda.empty_cache()
 
@@ -388,6 +403,7 @@ def main():
     }
     if not args.no_extra:
         result["workloads"] = run_extra(torch, mg, gen, max(args.steps, 20), args.warmup)
+        result["workloads"]["gate_up_swiglu_fused"] = fused
         torch.cuda.empty_cache()
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(torch, 0)

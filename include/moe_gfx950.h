@@ -98,6 +98,18 @@ typedef enum moe_weight_format {
     MOE_FMT_COUNT = 7
 } moe_weight_format;
 
+/* What the grouped GEMM writes.  MOE_EPILOGUE_SWIGLU fuses the activation that sits between the
+ * gate_up and the down projection of an MoE layer into the GEMM (no counterpart in the reference,
+ * whose caller runs it as a separate op on the [M, N] result): the weight's columns come in groups
+ * of 4 = (gate 2j, gate 2j+1, up 2j, up 2j+1) and y is bf16 [M, N/2] with
+ *     y[m, 2j + e] = silu(z[m, 4j + e]) * z[m, 4j + 2 + e],  e = 0, 1,
+ * z the fp32 accumulators of x . dequant(W) and silu(v) = v / (1 + exp(-v)).  Grouped GEMM only,
+ * on the N-contiguous containers (MOE_FMT_FP4_REF, MOE_FMT_FP8_REF, MOE_FMT_INT8, MOE_FMT_INT4). */
+typedef enum moe_epilogue {
+    MOE_EPILOGUE_NONE = 0,
+    MOE_EPILOGUE_SWIGLU = 1
+} moe_epilogue;
+
 /* Arguments of both grouped ops.  x, y are row-major bf16; group_list is the
  * cumulative int64 [G] device tensor of the reference (rows [gl[g-1], gl[g]) belong
  * to expert g, gl[-1] = 0; rows at or beyond gl[G-1] are not written;
@@ -108,11 +120,11 @@ typedef struct moe_grouped_args {
     const void *scale;         /* NULL only for MOE_FMT_BF16                        */
     const void *offset;        /* read by MOE_FMT_INT8 only; may be NULL otherwise  */
     const int64_t *group_list; /* device int64 [G], cumulative                      */
-    void *y;                   /* bf16 [M, N]                                       */
+    void *y;                   /* bf16 [M, N]  ([M, N/2] with MOE_EPILOGUE_SWIGLU)  */
     int64_t M, K, N, G;
     int64_t scale_rows;        /* scale.shape[-2]; used by FP4_REF (K/16) and INT4  */
     int32_t format;            /* moe_weight_format                                 */
-    int32_t reserved;          /* must be 0                                         */
+    int32_t epilogue;          /* moe_epilogue; MOE_EPILOGUE_NONE (0) for the reference's ops */
 } moe_grouped_args;
 
 /* codes uint8 [rows, cols/2] (even element in the low nibble), scale bf16

@@ -178,3 +178,19 @@ def grouped_gemm(fmt: int, x_bits, w, scale, offset, group_list, *, round_bf16: 
     if rc:
         raise RuntimeError(f"orc_grouped_gemm rc={rc}")
     return (y16, y32) if want_f32 else y16
+
+
+def swiglu_interleaved(z: np.ndarray) -> np.ndarray:
+    """fp32 accumulators [M, N] whose columns come in groups of 4 = (gate 2j, gate 2j+1, up 2j, up 2j+1)
+    -> bf16 bits [M, N/2], out[:, 2j+e] = silu(z[:, 4j+e]) * z[:, 4j+2+e] with silu(v) = v / (1 + exp(-v)),
+    evaluated in float64 and rounded once.  The fused activation has no counterpart in the reference
+    (its caller applies the activation to grouped_gemm's output as a separate op); this is the
+    definition the GPU epilogue is checked against, pinned to torch.nn.functional.silu in
+    tests/test_oracle.py."""
+    z = np.asarray(z, dtype=np.float64)
+    M, N = z.shape
+    assert N % 4 == 0
+    q = z.reshape(M, N // 4, 4)
+    gate, up = q[:, :, 0:2], q[:, :, 2:4]
+    out = (gate / (1.0 + np.exp(-gate)) * up).reshape(M, N // 2)
+    return f32_to_bf16_bits(out.astype(np.float32))

@@ -300,6 +300,20 @@ def test_routing_topk_against_torch_topk_and_softmax():
     assert list(ids[0]) == [4, 0, 1]
 
 
+def test_swiglu_interleaved_against_torch_silu_and_explicit_columns():
+    rng = np.random.default_rng(31)
+    z = (rng.standard_normal((5, 16)) * 3).astype(np.float32)
+    got = oracle.bf16_bits_to_f32(oracle.swiglu_interleaved(z))
+    zt = torch.from_numpy(z).double()
+    gate = torch.stack([zt[:, 0::4], zt[:, 1::4]], dim=2).reshape(5, 8)     # gate 2j, 2j+1 of every group of 4
+    up = torch.stack([zt[:, 2::4], zt[:, 3::4]], dim=2).reshape(5, 8)
+    ref = (torch.nn.functional.silu(gate) * up).float().to(torch.bfloat16).float().numpy()
+    assert np.array_equal(got, ref)
+    # one group by hand: columns (g0, g1, u0, u1) = (1, -2, 3, 4)
+    one = oracle.bf16_bits_to_f32(oracle.swiglu_interleaved(np.array([[1.0, -2.0, 3.0, 4.0]], dtype=np.float32)))
+    assert np.allclose(one, [[1.0 / (1.0 + np.exp(-1.0)) * 3.0, -2.0 / (1.0 + np.exp(2.0)) * 4.0]], rtol=2 ** -8)
+
+
 # ---------------------------------------------------------------- grouped_gemm
 @pytest.mark.parametrize("group_list", [[2, 3, 4, 256], [12, 25, 44, 48], [1, 2, 3, 4], [0, 0, 5, 5], [3, 3, 3, 3]])
 def test_grouped_gemm_against_torch_fp64(group_list):
