@@ -15,7 +15,7 @@
 // ALL rows of the tile, so each weight element is dequantized exactly once per tile.
 // x tiles go through a double-buffered, XOR-swizzled LDS tile shared by the 4 waves.
 // (Prefill on the int4 container uses a variant with 8 wavefronts and LDS-direct loads, see
-// gemm_tile_pair_int4.)
+// gemm_tile_pair.)
 //
 // MFMA: v_mfma_f32_16x16x32_bf16.  Lane l = 16*q + i holds, for A, row i and
 // k = 8q..8q+7 of the 16x32 block; for B, column i and the same k; for the result,
@@ -759,18 +759,29 @@ __device__ __forceinline__ void lds_load16(rsrc_t r, const u32x4_t* dst, int vof
 // 0x00..0x0f, which read as OCP e4m3 are exactly q / 512 -- v_cvt_pk_f32_fp8 converts two at
 // once -- and one fma per element applies 512 * scale and the zero point:
 // q s - 8 s = (q - 8) s exactly.
+//
+// The same routine serves the reference's pre-shuffled fp4 container: its 64 x 128-byte tile is
+// brought in by the same loads, a lane's 8 k rows of its 2 bytes are two 16-byte LDS reads, each
+// byte pair decodes to 4 floats with v_cvt_scalef32_pk_f32_fp4 and takes one multiply by the
+// column's scale of that 16-k block (4 scale rows per step instead of 2).
 // ---------------------------------------------------------------------------------
 constexpr int PAIR_CAPB = 10;                         // x stages hold 160 rows
 constexpr int PAIR_MT_MAX = 10;
 constexpr int PAIR_A_UNITS = 16 * PAIR_CAPB * 8;      // 16-byte units of one x stage
 constexpr int PAIR_B_UNITS = 64 * 8;                  // packed int4 tile of one k step: 64 rows of 128 bytes
-constexpr int PAIR_SC_UNITS = 64;                     // 2 scale rows (one per sub-step) of 256 bf16
 constexpr int PAIR_STAGES = 5;
-constexpr int PAIR_LDS_UNITS = PAIR_STAGES * (PAIR_A_UNITS + PAIR_B_UNITS + PAIR_SC_UNITS);
+// scale rows of 256 bf16 per k step: int4 one per 32-k sub-step (groups are multiples of 32), the
+// reference fp4 container one per 16 k
+template <int FMT>
+constexpr int pair_sc_rows() { return FMT == MOE_FMT_FP4_REF ? 4 : 2; }
+template <int FMT>
+constexpr int pair_lds_units() { return PAIR_STAGES * (PAIR_A_UNITS + PAIR_B_UNITS + 32 * pair_sc_rows<FMT>()); }
 
-template <int MT>
-__device__ __forceinline__ void gemm_tile_pair_int4(const GemmParams& P, u32x4_t* smem, int g, int64_t row0, int rows, int n0) {
-    constexpr int BK = 64, S = PAIR_STAGES;
+template <int FMT, int MT>
+__device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* smem, int g, int64_t row0, int rows, int n0) {
+    static_assert(FMT == MOE_FMT_INT4 || FMT == MOE_FMT_FP4_REF, "the k-split tile routine decodes int4 and the reference fp4 container");
+    constexpr bool FP4 = FMT == MOE_FMT_FP4_REF;
+    constexpr int BK = 64, S = PAIR_STAGES, SC_ROWS = pair_sc_rows<FMT>(), PAIR_SC_UNITS = 32 * SC_ROWS;
     u32x4_t* lds_a = smem;
     u32x4_t* lds_b = lds_a + S * PAIR_A_UNITS;
     u32x4_t* lds_s = lds_b + S * PAIR_B_UNITS;
@@ -814,9 +825,11 @@ __device__ __forceinline__ void gemm_tile_pair_int4(const GemmParams& P, u32x4_t
     }
     const int cb = 8 * wv * (P.N >> 1) + (n0 >> 1);
     const int kb_step = BK * (P.N >> 1);
-    const int cs = n0 * 2 + (wv & 3) * 128;    // scales: bytes [128 (wv & 3), +128) of row wv >> 2, 8 lanes
+    // scales of a step: int4 2 rows of 512 bytes, 128 bytes (8 lanes) per wavefront: bytes [128 (wv & 3), +128) of
+    // row wv >> 2; fp4 4 rows (one per 16 k), 256 bytes (16 lanes) per wavefront: bytes [256 (wv & 1), +256) of row wv >> 1
+    const int cs = FP4 ? n0 * 2 + (wv & 1) * 256 : n0 * 2 + (wv & 3) * 128;
     const int lane16 = lane * 16;
-    const bool s_lane = lane < 8;
+    const bool s_lane = lane < (FP4 ? 16 : 8);
     // m-th load of group kt (stage kt+4 of x, packed tile and scales), into LDS stage ST
     auto issue = [&](int m, int kt, int ST) {
         if (m < NA) {
@@ -824,8 +837,8 @@ __device__ __forceinline__ void gemm_tile_pair_int4(const GemmParams& P, u32x4_t
         } else if (m == NA) {
             lds_load16(rw, lds_b + ST * PAIR_B_UNITS + wv * 64, vb, cb + (kt + 4) * kb_step);
         } else {
-            const int grow = scale_row((uint32_t)((kt + 4) * 2 + (wv >> 2)));
-            if (s_lane) lds_load16(rs, lds_s + ST * PAIR_SC_UNITS + wv * 8, lane16, grow * (P.N * 2) + cs);
+            const int grow = FP4 ? (kt + 4) * 4 + (wv >> 1) : scale_row((uint32_t)((kt + 4) * 2 + (wv >> 2)));
+            if (s_lane) lds_load16(rs, lds_s + ST * PAIR_SC_UNITS + wv * (PAIR_SC_UNITS / 8), lane16, grow * (P.N * 2) + cs);
         }
     };
     auto issue_group = [&](int kt, int ST) {
@@ -866,11 +879,25 @@ __device__ __forceinline__ void gemm_tile_pair_int4(const GemmParams& P, u32x4_t
     uint32_t r[8];
     u32x2_t sc;
     auto read_raw = [&](int st) {
-        const uint32_t* t32 = reinterpret_cast<const uint32_t*>(lds_b + st * PAIR_B_UNITS);
         const uint16_t* sc16 = reinterpret_cast<const uint16_t*>(lds_s + st * PAIR_SC_UNITS);
+        if constexpr (FP4) {
+            // Reference pre-shuffle (grouped_gemm/test/python/test_group_gemm_fp4.py:129-142): the tile row
+            // 32 j + 8 i' + p holds, in its 32-byte run q', the 8 k rows 16 i' + 8 j + [0, 8) (one dword each)
+            // of byte columns 16 p + 4 q' + [0, 4).  This lane's 8 k are 32 h + 8 q + [0, 8) and its two
+            // bytes start at byte column 64 (cw >> 1) + 4 i + 2 (cw & 1): p = 4 (cw >> 1) + (i >> 2), q' = i & 3.
+            const int trow = 32 * (q & 1) + 8 * (2 * h + (q >> 1)) + 4 * (cw >> 1) + (i >> 2);
+            const int swz = 4 * ((trow >> 3) & 1);   // the halves of the rows with odd (row >> 3) are swapped (see vb)
+            const u32x4_t* tb = lds_b + st * PAIR_B_UNITS + trow * 8;
+            const u32x4_t lo4 = tb[(2 * (i & 3)) ^ swz], hi4 = tb[(2 * (i & 3) + 1) ^ swz];
 #pragma unroll
-        for (int j = 0; j < 8; ++j) r[j] = t32[((32 * h + 8 * q + j) * 8 + unit) * 4 + (d & 3)];
-        sc = *reinterpret_cast<const u32x2_t*>(sc16 + 256 * h + col0);
+            for (int j = 0; j < 4; ++j) { r[j] = lo4[j]; r[4 + j] = hi4[j]; }
+            sc = *reinterpret_cast<const u32x2_t*>(sc16 + 256 * (2 * h + (q >> 1)) + col0);
+        } else {
+            const uint32_t* t32 = reinterpret_cast<const uint32_t*>(lds_b + st * PAIR_B_UNITS);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) r[j] = t32[((32 * h + 8 * q + j) * 8 + unit) * 4 + (d & 3)];
+            sc = *reinterpret_cast<const u32x2_t*>(sc16 + 256 * h + col0);
+        }
     };
     read_raw(0);
 
@@ -881,8 +908,13 @@ __device__ __forceinline__ void gemm_tile_pair_int4(const GemmParams& P, u32x4_t
         // ---- decode phase: this wavefront's sub-step of the packed stage -> bf[0..3]
         float m[4], z[4];
         const float s0 = bf16_lo(sc[0]), s1 = bf16_hi(sc[0]), s2 = bf16_lo(sc[1]), s3 = bf16_hi(sc[1]);
-        m[0] = s0 * 512.f; m[1] = s1 * 512.f; m[2] = s2 * 512.f; m[3] = s3 * 512.f;
-        z[0] = -8.f * s0; z[1] = -8.f * s1; z[2] = -8.f * s2; z[3] = -8.f * s3;
+        if constexpr (FP4) {
+            m[0] = s0; m[1] = s1; m[2] = s2; m[3] = s3;
+            z[0] = z[1] = z[2] = z[3] = 0.f;
+        } else {
+            m[0] = s0 * 512.f; m[1] = s1 * 512.f; m[2] = s2 * 512.f; m[3] = s3 * 512.f;
+            z[0] = -8.f * s0; z[1] = -8.f * s1; z[2] = -8.f * s2; z[3] = -8.f * s3;
+        }
         // Written stage by stage over two row pairs at a time so that consecutive instructions are
         // independent (a VALU result is not available to the very next instruction); the fences
         // keep the scheduler from folding the stages back into per-element chains.
@@ -904,6 +936,21 @@ __device__ __forceinline__ void gemm_tile_pair_int4(const GemmParams& P, u32x4_t
             float wa[2][4], wb[2][4];
 #pragma unroll
             for (int p = 0; p < 2; ++p) pr[p] = __builtin_amdgcn_perm(r[2 * (p0 + p) + 1], r[2 * (p0 + p)], sel);   // a.b0 a.b1 b.b0 b.b1
+            if constexpr (FP4) {
+                // e2m1: each byte of pr is two columns of one k row; exact decode, one multiply by the
+                // column's scale, RNE to bf16 (W = bf16(e2m1 * scale) as the reference's antiquant phase)
+#pragma unroll
+                for (int p = 0; p < 2; ++p) {
+                    const f32x2_t a01 = e2m1_pair_to_f32<0>(pr[p]), a23 = e2m1_pair_to_f32<1>(pr[p]);
+                    const f32x2_t b01 = e2m1_pair_to_f32<2>(pr[p]), b23 = e2m1_pair_to_f32<3>(pr[p]);
+                    bf[0][p0 + p] = pack_bf16_rne(a01[0] * m[0], b01[0] * m[0]);
+                    bf[1][p0 + p] = pack_bf16_rne(a01[1] * m[1], b01[1] * m[1]);
+                    bf[2][p0 + p] = pack_bf16_rne(a23[0] * m[2], b23[0] * m[2]);
+                    bf[3][p0 + p] = pack_bf16_rne(a23[1] * m[3], b23[1] * m[3]);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+                continue;
+            }
 #pragma unroll
             for (int p = 0; p < 2; ++p) { lo[p] = pr[p] & mask; hi[p] = pr[p] >> 4; }
             __builtin_amdgcn_sched_barrier(0);
@@ -1052,7 +1099,8 @@ enum { GK_GENERAL = 0, GK_SKINNY = 1, GK_PAIR = 2 };
 
 template <int FMT, int KIND>
 struct KernelCfg {
-    static_assert(KIND != GK_PAIR || FMT == MOE_FMT_INT4, "the k-split tile routine decodes int4 only");
+    static_assert(KIND != GK_PAIR || FMT == MOE_FMT_INT4 || FMT == MOE_FMT_FP4_REF,
+                  "the k-split tile routine decodes int4 and the reference fp4 container");
     static constexpr int WAVES = KIND == GK_PAIR ? 8 : 4;
     static constexpr int BN = GM_BN;                                             // columns per tile
     static constexpr int WG_PER_CU = KIND == GK_SKINNY ? GM_SKINNY_WAVES : 1;
@@ -1062,7 +1110,7 @@ struct KernelCfg {
     // 16-byte LDS units of the tile routine (the tile prefix array follows them)
     static constexpr int lds_units() {
         if constexpr (KIND == GK_PAIR)
-            return PAIR_LDS_UNITS;
+            return pair_lds_units<FMT>();
         else
             return 2 * 16 * CAPB * (BTraits<FMT>::BK / 8) + 2 * BTraits<FMT>::B_LDS_UNITS;
     }
@@ -1072,7 +1120,7 @@ template <int FMT, int MT, int KIND>
 __device__ __forceinline__ void run_tile(const GemmParams& P, u32x4_t* smem, int g, int64_t row0, int rows, int n0) {
     using C = KernelCfg<FMT, KIND>;
     if constexpr (KIND == GK_PAIR)
-        gemm_tile_pair_int4<MT>(P, smem, g, row0, rows, n0);
+        gemm_tile_pair<FMT, MT>(P, smem, g, row0, rows, n0);
     else
         gemm_tile<FMT, MT, C::CAPB>(P, smem, smem + 2 * 16 * C::CAPB * (BTraits<FMT>::BK / 8), g, row0, rows, n0);
 }
@@ -1231,9 +1279,10 @@ static int launch_gemm_fmt(const moe_grouped_args* a, hipStream_t stream) {
     P.y = static_cast<uint16_t*>(a->y);
     P.M = a->M; P.K = (int)a->K; P.N = (int)a->N; P.G = (int)a->G; P.scale_rows = (int)a->scale_rows;
     P.epilogue = a->epilogue;
-    // int4: the k-split kernel at every batch size (measured faster than the small-tile kernel down to
-    // decode batches of 1-2 rows per expert: 243 vs 344 us at 128 rows over 256 experts, 7168 x 2048).
-    if constexpr (FMT == MOE_FMT_INT4) {
+    // int4 and the reference fp4 container: the k-split kernel at every batch size (measured faster than
+    // the small-tile kernel down to decode batches of 1-2 rows per expert: int4 243 vs 344 us at 128 rows
+    // over 256 experts, 7168 x 2048; fp4 476 vs 519 us at 512 rows).
+    if constexpr (FMT == MOE_FMT_INT4 || FMT == MOE_FMT_FP4_REF) {
         return launch_gemm_kind<FMT, GK_PAIR>(P, a, stream);
     } else {
         // Decode-like batches (on average at most 24 rows per expert; group_list itself stays on the
