@@ -98,6 +98,16 @@ def _check_accumulator_moves(src: str) -> None:
 
     for m in re.finditer(r"^(\w*grouped_gemm_kernel\w*):", text, re.M):
         lines = text[m.end():text.index("s_endpgm", m.end())].split("\n")
+        # Only the MFMAs of inline asm are invisible to the compiler; those it emitted itself (builtins)
+        # get their wait states from it and are ordinary instructions here: rename them.
+        in_asm = False
+        for i, l in enumerate(lines):
+            if "#ASMSTART" in l:
+                in_asm = True
+            elif "#ASMEND" in l:
+                in_asm = False
+            elif not in_asm and l.strip().startswith("v_mfma"):
+                lines[i] = l.replace("v_mfma", "v_builtin_mfma", 1)
         labels = {mm.group(1): i for i, l in enumerate(lines) if (mm := re.match(r"^(\.LBB\d+_\d+):", l))}
         loops = []
         for i, l in enumerate(lines):

@@ -777,7 +777,13 @@ constexpr int pair_sc_rows() { return FMT == MOE_FMT_FP4_REF ? 4 : 2; }
 template <int FMT>
 constexpr int pair_lds_units() { return PAIR_STAGES * (PAIR_A_UNITS + PAIR_B_UNITS + 32 * pair_sc_rows<FMT>()); }
 
-template <int FMT, int MT>
+// EXACT selects the arithmetic of the GEMV op (grouped_soft_gemv/op_kernel/gemv_impl.h:147-199: the
+// dequantized weights stay fp32): the B fragments then hold the codes themselves, which are exact in
+// bf16, every MFMA covers k of one scale group only and its result is multiplied by that group's fp32
+// scale on the way into the accumulators.  The fp4 container has a scale per 16 k, half an MFMA: the x
+// fragment is split into its lanes q < 2 and q >= 2 (the other half zeroed) and each half takes its
+// own MFMA.  These MFMAs are compiler-visible builtins (their results feed ordinary VALU code).
+template <int FMT, int MT, bool EXACT = false>
 __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* smem, int g, int64_t row0, int rows, int n0) {
     static_assert(FMT == MOE_FMT_INT4 || FMT == MOE_FMT_FP4_REF, "the k-split tile routine decodes int4 and the reference fp4 container");
     constexpr bool FP4 = FMT == MOE_FMT_FP4_REF;
@@ -861,9 +867,13 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-        for (int t = 0; t < 4; ++t)
-            asm volatile("v_mov_b32 %0, 0\n\tv_mov_b32 %1, 0\n\tv_mov_b32 %2, 0\n\tv_mov_b32 %3, 0"
-                         : "=v"(acc[mt][t][0]), "=v"(acc[mt][t][1]), "=v"(acc[mt][t][2]), "=v"(acc[mt][t][3]));
+        for (int t = 0; t < 4; ++t) {
+            if constexpr (EXACT)
+                acc[mt][t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+            else
+                asm volatile("v_mov_b32 %0, 0\n\tv_mov_b32 %1, 0\n\tv_mov_b32 %2, 0\n\tv_mov_b32 %3, 0"
+                             : "=v"(acc[mt][t][0]), "=v"(acc[mt][t][1]), "=v"(acc[mt][t][2]), "=v"(acc[mt][t][3]));
+        }
     u32x4_t bf[4], afr[4];
     constexpr int RING = 3;
     constexpr int R = RING < MT ? RING : MT;   // x fragments read ahead of their MFMAs
@@ -877,7 +887,7 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
 
     // this lane's packed dwords and scales of its sub-step of LDS stage st
     uint32_t r[8];
-    u32x2_t sc;
+    u32x2_t sc, sc2 = {0u, 0u};   // sc2: with EXACT, the fp4 scales of the second 16 k of the sub-step
     auto read_raw = [&](int st) {
         const uint16_t* sc16 = reinterpret_cast<const uint16_t*>(lds_s + st * PAIR_SC_UNITS);
         if constexpr (FP4) {
@@ -891,7 +901,12 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
             const u32x4_t lo4 = tb[(2 * (i & 3)) ^ swz], hi4 = tb[(2 * (i & 3) + 1) ^ swz];
 #pragma unroll
             for (int j = 0; j < 4; ++j) { r[j] = lo4[j]; r[4 + j] = hi4[j]; }
-            sc = *reinterpret_cast<const u32x2_t*>(sc16 + 256 * (2 * h + (q >> 1)) + col0);
+            if constexpr (EXACT) {
+                sc = *reinterpret_cast<const u32x2_t*>(sc16 + 256 * (2 * h) + col0);
+                sc2 = *reinterpret_cast<const u32x2_t*>(sc16 + 256 * (2 * h + 1) + col0);
+            } else {
+                sc = *reinterpret_cast<const u32x2_t*>(sc16 + 256 * (2 * h + (q >> 1)) + col0);
+            }
         } else {
             const uint32_t* t32 = reinterpret_cast<const uint32_t*>(lds_b + st * PAIR_B_UNITS);
 #pragma unroll
@@ -908,7 +923,13 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
         // ---- decode phase: this wavefront's sub-step of the packed stage -> bf[0..3]
         float m[4], z[4];
         const float s0 = bf16_lo(sc[0]), s1 = bf16_hi(sc[0]), s2 = bf16_lo(sc[1]), s3 = bf16_hi(sc[1]);
-        if constexpr (FP4) {
+        // with EXACT: the scales of the step being multiplied (sc is refilled during the MFMA phase)
+        const float sa[4] = {s0, s1, s2, s3};
+        const float sb[4] = {bf16_lo(sc2[0]), bf16_hi(sc2[0]), bf16_lo(sc2[1]), bf16_hi(sc2[1])};
+        if constexpr (EXACT) {
+            m[0] = m[1] = m[2] = m[3] = FP4 ? 1.f : 512.f;
+            z[0] = z[1] = z[2] = z[3] = FP4 ? 0.f : -8.f;
+        } else if constexpr (FP4) {
             m[0] = s0; m[1] = s1; m[2] = s2; m[3] = s3;
             z[0] = z[1] = z[2] = z[3] = 0.f;
         } else {
@@ -943,10 +964,17 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
                 for (int p = 0; p < 2; ++p) {
                     const f32x2_t a01 = e2m1_pair_to_f32<0>(pr[p]), a23 = e2m1_pair_to_f32<1>(pr[p]);
                     const f32x2_t b01 = e2m1_pair_to_f32<2>(pr[p]), b23 = e2m1_pair_to_f32<3>(pr[p]);
-                    bf[0][p0 + p] = pack_bf16_rne(a01[0] * m[0], b01[0] * m[0]);
-                    bf[1][p0 + p] = pack_bf16_rne(a01[1] * m[1], b01[1] * m[1]);
-                    bf[2][p0 + p] = pack_bf16_rne(a23[0] * m[2], b23[0] * m[2]);
-                    bf[3][p0 + p] = pack_bf16_rne(a23[1] * m[3], b23[1] * m[3]);
+                    if constexpr (EXACT) {
+                        bf[0][p0 + p] = pack_bf16_rne(a01[0], b01[0]);
+                        bf[1][p0 + p] = pack_bf16_rne(a01[1], b01[1]);
+                        bf[2][p0 + p] = pack_bf16_rne(a23[0], b23[0]);
+                        bf[3][p0 + p] = pack_bf16_rne(a23[1], b23[1]);
+                    } else {
+                        bf[0][p0 + p] = pack_bf16_rne(a01[0] * m[0], b01[0] * m[0]);
+                        bf[1][p0 + p] = pack_bf16_rne(a01[1] * m[1], b01[1] * m[1]);
+                        bf[2][p0 + p] = pack_bf16_rne(a23[0] * m[2], b23[0] * m[2]);
+                        bf[3][p0 + p] = pack_bf16_rne(a23[1] * m[3], b23[1] * m[3]);
+                    }
                 }
                 __builtin_amdgcn_sched_barrier(0);
                 continue;
@@ -1000,8 +1028,35 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
             if (mt + R < MT) afr[(mt + R) & 3] = la[a_lds_unit<BK>(16 * (mt + R) + i, 4 * h + q)];
+            if constexpr (EXACT) {
+                const f32x4_t zero = {0.f, 0.f, 0.f, 0.f};
+                if constexpr (FP4) {
+                    const uint32_t mlo = q < 2 ? 0xffffffffu : 0u;
+                    u32x4_t xlo, xhi;
 #pragma unroll
-            for (int t = 0; t < 4; ++t) mfma_16x16x32_v(acc[mt][t], afr[mt & 3], bf[t]);
+                    for (int j = 0; j < 4; ++j) { xlo[j] = afr[mt & 3][j] & mlo; xhi[j] = afr[mt & 3][j] & ~mlo; }
+#pragma unroll
+                    for (int t = 0; t < 4; ++t) {
+                        const f32x4_t dlo = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                            __builtin_bit_cast(bf16x8_t, xlo), __builtin_bit_cast(bf16x8_t, bf[t]), zero, 0, 0, 0);
+                        const f32x4_t dhi = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                            __builtin_bit_cast(bf16x8_t, xhi), __builtin_bit_cast(bf16x8_t, bf[t]), zero, 0, 0, 0);
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) acc[mt][t][e] = fmaf(dhi[e], sb[t], fmaf(dlo[e], sa[t], acc[mt][t][e]));
+                    }
+                } else {
+#pragma unroll
+                    for (int t = 0; t < 4; ++t) {
+                        const f32x4_t dd = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                            __builtin_bit_cast(bf16x8_t, afr[mt & 3]), __builtin_bit_cast(bf16x8_t, bf[t]), zero, 0, 0, 0);
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) acc[mt][t][e] = fmaf(dd[e], sa[t], acc[mt][t][e]);
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int t = 0; t < 4; ++t) mfma_16x16x32_v(acc[mt][t], afr[mt & 3], bf[t]);
+            }
 #pragma unroll
             for (int m = (mt * NI + MT - 1) / MT; m < ((mt + 1) * NI + MT - 1) / MT; ++m) issue(m, kt, sl);
             if (mt == 0) read_raw(sn);
@@ -1095,21 +1150,26 @@ __device__ __forceinline__ void expert_chunks(int m, int& chunks, int& bpc) {
 //   GK_SKINNY   the same tile routine with tiles of at most 32 rows and several workgroups per CU
 //               (decode-sized batches are HBM bound: more weight bytes in flight)
 //   GK_PAIR     int4 prefill: 8 wavefronts, k range split between the two wavefronts of a SIMD
-enum { GK_GENERAL = 0, GK_SKINNY = 1, GK_PAIR = 2 };
+//   GK_PAIR_EXACT  GK_PAIR with the GEMV op's arithmetic (weights not rounded to bf16), tiles of at most 32 rows
+enum { GK_GENERAL = 0, GK_SKINNY = 1, GK_PAIR = 2, GK_PAIR_EXACT = 3 };
+constexpr int PAIR_EXACT_MT_MAX = 2;
 
 template <int FMT, int KIND>
 struct KernelCfg {
-    static_assert(KIND != GK_PAIR || FMT == MOE_FMT_INT4 || FMT == MOE_FMT_FP4_REF,
+    static constexpr bool PAIR = KIND == GK_PAIR || KIND == GK_PAIR_EXACT;
+    static_assert(!PAIR || FMT == MOE_FMT_INT4 || FMT == MOE_FMT_FP4_REF,
                   "the k-split tile routine decodes int4 and the reference fp4 container");
-    static constexpr int WAVES = KIND == GK_PAIR ? 8 : 4;
+    static constexpr int WAVES = PAIR ? 8 : 4;
     static constexpr int BN = GM_BN;                                             // columns per tile
     static constexpr int WG_PER_CU = KIND == GK_SKINNY ? GM_SKINNY_WAVES : 1;
-    static constexpr int CAPB = KIND == GK_SKINNY ? GM_SKINNY_BLOCKS : KIND == GK_PAIR ? PAIR_CAPB : GM_MT_MAX;
-    static constexpr int fmt_mt_max() { return KIND == GK_PAIR ? PAIR_MT_MAX : BTraits<FMT>::MT_MAX; }
+    static constexpr int CAPB = KIND == GK_SKINNY ? GM_SKINNY_BLOCKS : PAIR ? PAIR_CAPB : GM_MT_MAX;
+    static constexpr int fmt_mt_max() {
+        return KIND == GK_PAIR ? PAIR_MT_MAX : KIND == GK_PAIR_EXACT ? PAIR_EXACT_MT_MAX : BTraits<FMT>::MT_MAX;
+    }
     static constexpr int MTM = CAPB < fmt_mt_max() ? CAPB : fmt_mt_max();        // row blocks per tile
     // 16-byte LDS units of the tile routine (the tile prefix array follows them)
     static constexpr int lds_units() {
-        if constexpr (KIND == GK_PAIR)
+        if constexpr (PAIR)
             return pair_lds_units<FMT>();
         else
             return 2 * 16 * CAPB * (BTraits<FMT>::BK / 8) + 2 * BTraits<FMT>::B_LDS_UNITS;
@@ -1119,8 +1179,8 @@ struct KernelCfg {
 template <int FMT, int MT, int KIND>
 __device__ __forceinline__ void run_tile(const GemmParams& P, u32x4_t* smem, int g, int64_t row0, int rows, int n0) {
     using C = KernelCfg<FMT, KIND>;
-    if constexpr (KIND == GK_PAIR)
-        gemm_tile_pair<FMT, MT>(P, smem, g, row0, rows, n0);
+    if constexpr (C::PAIR)
+        gemm_tile_pair<FMT, MT, KIND == GK_PAIR_EXACT>(P, smem, g, row0, rows, n0);
     else
         gemm_tile<FMT, MT, C::CAPB>(P, smem, smem + 2 * 16 * C::CAPB * (BTraits<FMT>::BK / 8), g, row0, rows, n0);
 }
@@ -1268,8 +1328,7 @@ static int launch_gemm_kind(const GemmParams& P, const moe_grouped_args* a, hipS
     return hipGetLastError() == hipSuccess ? MOE_OK : MOE_ERR_LAUNCH;
 }
 
-template <int FMT>
-static int launch_gemm_fmt(const moe_grouped_args* a, hipStream_t stream) {
+static GemmParams gemm_params(const moe_grouped_args* a) {
     GemmParams P;
     P.x = static_cast<const uint16_t*>(a->x);
     P.w = static_cast<const uint8_t*>(a->weight);
@@ -1279,6 +1338,12 @@ static int launch_gemm_fmt(const moe_grouped_args* a, hipStream_t stream) {
     P.y = static_cast<uint16_t*>(a->y);
     P.M = a->M; P.K = (int)a->K; P.N = (int)a->N; P.G = (int)a->G; P.scale_rows = (int)a->scale_rows;
     P.epilogue = a->epilogue;
+    return P;
+}
+
+template <int FMT>
+static int launch_gemm_fmt(const moe_grouped_args* a, hipStream_t stream) {
+    const GemmParams P = gemm_params(a);
     // int4 and the reference fp4 container: the k-split kernel at every batch size (measured faster than
     // the small-tile kernel down to decode batches of 1-2 rows per expert: int4 243 vs 344 us at 128 rows
     // over 256 experts, 7168 x 2048; fp4 476 vs 519 us at 512 rows).
@@ -1290,6 +1355,15 @@ static int launch_gemm_fmt(const moe_grouped_args* a, hipStream_t stream) {
         // costs one pass over its weights per 32 rows.
         if (a->M <= 24 * a->G) return launch_gemm_kind<FMT, GK_SKINNY>(P, a, stream);
         return launch_gemm_kind<FMT, GK_GENERAL>(P, a, stream);
+    }
+}
+
+int launch_gemm_exact(const moe_grouped_args* a, hipStream_t stream) {
+    const GemmParams P = gemm_params(a);
+    switch (a->format) {
+        case MOE_FMT_FP4_REF: return launch_gemm_kind<MOE_FMT_FP4_REF, GK_PAIR_EXACT>(P, a, stream);
+        case MOE_FMT_INT4: return launch_gemm_kind<MOE_FMT_INT4, GK_PAIR_EXACT>(P, a, stream);
+        default: return MOE_ERR_BAD_FORMAT;
     }
 }
 

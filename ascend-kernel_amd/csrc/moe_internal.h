@@ -10,6 +10,9 @@ int launch_dequant_fp4_bf16(const moe_dequant_args* a, hipStream_t stream);
 int launch_grouped_gemv(const moe_grouped_args* a, hipStream_t stream, bool gemm_rounding = false);
 // True when the GEMV launcher is the faster path for a grouped GEMM call of this shape.
 bool gemv_preferred(const moe_grouped_args* a);
+// grouped GEMV on the fp4 / int4 N-contiguous containers by the k-split GEMM kernel run with the GEMV
+// op's arithmetic; MOE_ERR_TOO_LARGE when the expert count does not fit its LDS
+int launch_gemm_exact(const moe_grouped_args* a, hipStream_t stream);
 int launch_grouped_gemm(const moe_grouped_args* a, hipStream_t stream);
 int launch_prepack_fp4_ref(const moe_prepack_fp4_args* a, hipStream_t stream);
 int launch_route(const moe_route_args* a, hipStream_t stream);

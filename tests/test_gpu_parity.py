@@ -263,6 +263,22 @@ def test_gemv_fp4_b32_row_counts_up_to_and_beyond_16(K, N, fmt):
     assert (got[gl[-1]:] == 0x7FC0).all()
 
 
+@pytest.mark.parametrize("fmt,K,N,group", [("fp4", 1024, 256, 16), ("fp4", 7168, 512, 16), ("fp4", 64, 256, 16),
+                                           ("int4", 1024, 256, 128), ("int4", 7168, 512, 128), ("int4", 192, 256, 32),
+                                           ("int4", 256, 256, 64)])
+def test_gemv_n_contiguous_row_counts_up_to_and_beyond_32(fmt, K, N, group):
+    """The GEMV op on the reference fp4 container and on int4 runs on the matrix cores with weights that are
+    not rounded to bf16 (the codes go through the MFMA, the fp32 scales are applied to its results), in
+    tiles of up to 32 rows of an expert; K = 64 is a single k step."""
+    _say(f"gemv {fmt} rows K={K} N={N} group={group}")
+    counts = [1, 0, 4, 5, 16, 17, 32, 33, 70, 0, 3]
+    gl = list(np.cumsum(counts))
+    case = H.make_case(fmt, len(gl), K, N, gl, seed=K + N + group, extra_rows=2, group=group)
+    got = H.run_cabi(case, H.upload(case), "gemv")
+    H.assert_close(got, H.oracle_out(case, gemv=True), rows=slice(0, gl[-1]), what=f"gemv {fmt} rows K={K} N={N}")
+    assert (got[gl[-1]:] == 0x7FC0).all()
+
+
 def test_gemv_reference_fp8_test_shape_via_module():
     """test_group_soft_gemv_fp8.py:37-88: G=4, M=4, K=512, N=1536, x = ones, expected value
     from fp32 (un-rounded) weights, rtol 0.02."""
