@@ -279,6 +279,20 @@ def test_gemv_n_contiguous_row_counts_up_to_and_beyond_32(fmt, K, N, group):
     assert (got[gl[-1]:] == 0x7FC0).all()
 
 
+@pytest.mark.parametrize("fmt", ["fp4", "int4"])
+def test_gemv_n_contiguous_more_experts_than_the_matrix_core_kernel_takes(fmt):
+    """The k-split kernel keeps a tile table of G + 1 entries in LDS; beyond its capacity the GEMV op
+    falls back to the vector kernel."""
+    _say(f"gemv {fmt} G=2100")
+    G = 2100
+    rng = np.random.default_rng(11)
+    counts = rng.integers(0, 3, G)
+    gl = list(np.cumsum(counts))
+    case = H.make_case(fmt, G, 128, 256, gl, seed=12, group=32 if fmt == "int4" else 16)
+    got = H.run_cabi(case, H.upload(case), "gemv")
+    H.assert_close(got, H.oracle_out(case, gemv=True), what=f"gemv {fmt} G={G}")
+
+
 def test_gemv_reference_fp8_test_shape_via_module():
     """test_group_soft_gemv_fp8.py:37-88: G=4, M=4, K=512, N=1536, x = ones, expected value
     from fp32 (un-rounded) weights, rtol 0.02."""
