@@ -4,8 +4,8 @@
 //
 // Replaces grouped_matmul_antiquant (grouped_gemm/op_kernel/grouped_matmul_antiquant.h:225-364,
 // grouped_matmul.h:147-463).  The reference decodes each weight slab to a bf16 copy in
-// global memory and then runs a bf16 matmul on it; here the packed weights go
-// HBM -> registers -> bf16 MFMA fragments directly and never touch LDS or HBM again.
+// global memory and then runs a bf16 matmul on it; here the packed weights are decoded
+// in registers straight into bf16 MFMA fragments and never go back to HBM.
 //
 // Work decomposition.  A tile is (expert, chunk of <= 192 rows, 256 columns).  The
 // tile list is derived inside the kernel from the device-resident cumulative
@@ -14,8 +14,8 @@
 // L2.  A workgroup has 4 wavefronts; every wavefront owns 64 of the 256 columns for
 // ALL rows of the tile, so each weight element is dequantized exactly once per tile.
 // x tiles go through a double-buffered, XOR-swizzled LDS tile shared by the 4 waves.
-// (Prefill on the int4 container uses a variant with 8 wavefronts and LDS-direct loads, see
-// gemm_tile_pair.)
+// (The int4 container and the reference's pre-shuffled fp4 container use a tile routine with 8
+// wavefronts and LDS-direct loads instead, see gemm_tile_pair.)
 //
 // MFMA: v_mfma_f32_16x16x32_bf16.  Lane l = 16*q + i holds, for A, row i and
 // k = 8q..8q+7 of the 16x32 block; for B, column i and the same k; for the result,
@@ -102,10 +102,7 @@ struct BCtx {
     const uint16_t* og;
     const float* s8;     // fp8: scale blocks of the expert
     int K, N, n0;
-    uint32_t gmul;       // int4: floor(2^32 / (group/32)) + 1 turns sub-step -> scale row into a
-                         // multiply (exact below 2^16 sub-steps); 0 when the group is 32
     int i, q, w;         // lane & 15, lane >> 4, wavefront (scalar)
-    uint32_t mlo, mhi;   // 0x0f0f / 0xf0f0, opaque to the optimizer (int4 decode)
 };
 
 // Each weight container provides
@@ -119,175 +116,24 @@ struct BCtx {
 template <int FMT>
 struct BTraits;
 
-// ------------------------------------------------------------------ int4, [K, N/2]
-// Lane (i, q) of wavefront w owns the 4 columns 128(w>>1) + 8i + 4(w&1) + [0,4), i.e. half
-// of the dword holding the 8 columns 128(w>>1) + 8i + [0,8) of each of its 8 k rows
-// (wavefronts 2p and 2p+1 use the two halves of the same dwords).  MFMA t gets nibble t
-// of that half.
-// The packed 64(k) x 128 B tile of a k step goes HBM -> registers -> LDS with two
-// coalesced 16-byte loads per thread (the vector-memory address unit handles a 16-byte
-// load in the time of a 4-byte one), and each lane then picks its dwords from LDS.  In
-// LDS the two 64-byte halves of the rows with odd (row >> 3) are swapped, so that the
-// four q groups of a wavefront read from both halves of the banks.
-// Decode: byte b of (v & 0x0f0f) is nibble 2b, byte b of (v & 0xf0f0) is
-// 16 * nibble 2b+1; v_cvt_f32_ubyteN turns either into fp32 and one fma applies
-// scale (or scale/16) and the zero point: q*s - 8s = (q - 8)*s exactly (<= 12 significant
-// bits), so the bf16 weight equals RNE_bf16((q - 8) * scale).
-template <>
-struct BTraits<MOE_FMT_INT4> {
-    static constexpr int BK = 64, NS = 2;
-    static constexpr bool DOUBLE_RAW = false;
-    static constexpr int MT_MAX = 10;  // 160 rows: the largest tile that keeps every value in registers
-    static constexpr int B_LDS_UNITS = 64 * 8;  // 16-byte units of one packed tile in LDS (0: no LDS staging)
-    static constexpr int B_LOADS = 2;           // 16-byte global loads per thread per k step
-    struct Raw {
-        uint32_t r[2][8];
-        u32x2_t sc[2];
-    };
-    __device__ static __forceinline__ int a_chunk(int s, int q) { return 4 * s + q; }
-    __device__ static __forceinline__ int col(const BCtx& c, int t) {
-        return 128 * (c.w >> 1) + 8 * c.i + 4 * (c.w & 1) + t;
-    }
-    __device__ static __forceinline__ void init(BCtx& c) {
-        const int tid = 64 * c.w + 16 * c.q + c.i;
-        c.vw = (tid >> 3) * (c.N >> 1) + (tid & 7) * 16;   // staging: row tid>>3 (+32), chunk tid&7
-        c.vs = col(c, 0) * 2;
-    }
-    // global -> registers: rows (tid >> 3) + 32h of the tile of the step starting at k0
-    __device__ static __forceinline__ void stage_load(u32x4_t breg[B_LOADS], const BCtx& c, int k0) {
-        const int nb = c.N >> 1;
-#pragma unroll
-        for (int h = 0; h < B_LOADS; ++h) breg[h] = ldg_b128(c.rw, c.vw, (k0 + 32 * h) * nb + (c.n0 >> 1));
-    }
-    // registers -> LDS tile
-    __device__ static __forceinline__ void stage_store(u32x4_t* tile, const u32x4_t breg[B_LOADS], const BCtx& c) {
-        const int tid = 64 * c.w + 16 * c.q + c.i;
-        const int r = tid >> 3, ch = tid & 7;
-#pragma unroll
-        for (int h = 0; h < B_LOADS; ++h) tile[(r + 32 * h) * 8 + (ch ^ (4 * ((r >> 3) & 1)))] = breg[h];
-    }
-    // LDS tile -> this lane's dwords of sub-step s
-    __device__ static __forceinline__ void load_sub(Raw& raw, const BCtx& c, int, int s, const u32x4_t* tile) {
-        const uint32_t* t32 = reinterpret_cast<const uint32_t*>(tile);
-        const int d = 16 * (c.w >> 1) + c.i;  // dword of the row
-        const int unit = (d >> 2) ^ (4 * (c.q & 1));
-#pragma unroll
-        for (int j = 0; j < 8; ++j) raw.r[s][j] = t32[((32 * s + 8 * c.q + j) * 8 + unit) * 4 + (d & 3)];
-    }
-    // The scales of sub-step s of the step starting at k0 come straight from global memory, a
-    // full step ahead.  A 32-k sub-step never straddles a scale group (group % 32 == 0).
-    __device__ static __forceinline__ void load_scale(Raw& raw, const BCtx& c, int k0, int s) {
-        const uint32_t sub = (uint32_t)((k0 >> 5) + s);
-        const int grow = c.gmul ? (int)__umulhi(sub, c.gmul) : (int)sub;
-        raw.sc[s] = ldg_b64(c.rs, c.vs, (grow * c.N + c.n0) * 2);
-    }
-    // The nibble masks come from BCtx as values the compiler cannot see through; with literal
-    // masks it folds them into every extraction and spends an extra instruction per element
-    // instead of using v_cvt_f32_ubyte0 / ubyte1 directly.
-    __device__ static __forceinline__ float ubyte0(uint32_t v) { return (float)(v & 0xffu); }
-    __device__ static __forceinline__ float ubyte1(uint32_t v) { return (float)((v >> 8) & 0xffu); }
-    struct Dq {
-        float m[4], z[4];        // multiplier and zero-point term of the 4 columns
-        uint32_t al, ah, bl, bh; // masked halves of the two k rows of the current pair
-        __device__ __forceinline__ void init_tile(const BCtx&) {}
-        __device__ __forceinline__ void prep(const Raw& raw, const BCtx&, int s) {
-            const uint32_t sa = pinned(raw.sc[s][0]), sb = pinned(raw.sc[s][1]);
-            const float s0 = bf16_lo(sa), s1 = bf16_hi(sa), s2 = bf16_lo(sb), s3 = bf16_hi(sb);
-            m[0] = s0; m[1] = s1 * 0.0625f; m[2] = s2; m[3] = s3 * 0.0625f;  // odd nibbles arrive times 16
-            z[0] = -8.f * s0; z[1] = -8.f * s1; z[2] = -8.f * s2; z[3] = -8.f * s3;
-        }
-        __device__ __forceinline__ void unit(const Raw& raw, const BCtx& c, int s, int p, int t, u32x4_t out[4]) {
-            if (t == 0) {
-                const int sh = 16 * (c.w & 1);
-                const uint32_t a = pinned(raw.r[s][2 * p]) >> sh, b = raw.r[s][2 * p + 1] >> sh;
-                al = a & c.mlo; ah = a & c.mhi; bl = b & c.mlo; bh = b & c.mhi;
-            }
-            const uint32_t ua = pinned((t & 1) ? ah : al), ub = (t & 1) ? bh : bl;
-            const float fa = (t & 2) ? ubyte1(ua) : ubyte0(ua), fb = (t & 2) ? ubyte1(ub) : ubyte0(ub);
-            out[t][p] = pinned(pack_bf16_rne(fmaf(fa, m[t], z[t]), fmaf(fb, m[t], z[t])));
-        }
-    };
-};
-
-// ---------------------------------------------- reference "fp4": pre-shuffled [K, N/2]
-// Inside tile (a = k/64, 256-column block) destination row R = j<<5 | i'<<3 | p holds
-// k = 64a + 16i' + 8j + [0,8) for columns 32p + [0,32); bytes 32q' + 4r + [0,4) of
-// that row are the 8 columns 32p + 8q' + [0,8) at k offset r.  So the 8 k rows a lane
-// needs for its 8-column group are 32 contiguous bytes.
-template <>
-struct BTraits<MOE_FMT_FP4_REF> {
-    static constexpr int BK = 64, NS = 2;
-    static constexpr int B_LDS_UNITS = 0, B_LOADS = 1;
-    static constexpr bool DOUBLE_RAW = false;
-    static constexpr int MT_MAX = 11;
-    struct Raw {
-        u32x4_t r[2][2];
-        u32x2_t sc[2];
-    };
-    __device__ static __forceinline__ void stage_load(u32x4_t*, const BCtx&, int) {}
-    __device__ static __forceinline__ void stage_store(u32x4_t*, const u32x4_t*, const BCtx&) {}
-    __device__ static __forceinline__ void load_scale(Raw&, const BCtx&, int, int) {}
-    __device__ static __forceinline__ int a_chunk(int s, int q) { return 4 * s + q; }
-    __device__ static __forceinline__ int col(const BCtx& c, int t) {
-        return 128 * (c.w >> 1) + 8 * c.i + 4 * (c.w & 1) + t;
-    }
-    __device__ static __forceinline__ void init(BCtx& c) {
-        const int c8 = 16 * (c.w >> 1) + c.i, p = c8 >> 2, qq = c8 & 3;
-        // row of sub-step 0; sub-step s adds 16 rows (i' = 2s + (q >> 1))
-        const int R0 = ((c.q & 1) << 5) | ((c.q >> 1) << 3) | p;
-        c.vw = R0 * (c.N >> 1) + 32 * qq;
-        c.vs = ((c.q >> 1) * c.N + col(c, 0)) * 2;  // scale group of 16 k: (k0 + 32s)/16 + (q >> 1)
-    }
-    __device__ static __forceinline__ void load_sub(Raw& raw, const BCtx& c, int k0, int s, const u32x4_t*) {
-        const int nb = c.N >> 1;
-        const int so = (k0 + 16 * s) * nb + (c.n0 >> 1);
-        raw.r[s][0] = ldg_b128(c.rw, c.vw, so);
-        raw.r[s][1] = ldg_b128(c.rw, c.vw, so + 16);
-        raw.sc[s] = ldg_b64(c.rs, c.vs, (((k0 + 32 * s) >> 4) * c.N + c.n0) * 2);
-    }
-    struct Dq {
-        float sc[4];
-        f32x2_t va, vb;  // decoded pair of the current byte for the two k rows
-        __device__ __forceinline__ void init_tile(const BCtx&) {}
-        __device__ __forceinline__ void prep(const Raw& raw, const BCtx&, int s) {
-            sc[0] = bf16_lo(raw.sc[s][0]); sc[1] = bf16_hi(raw.sc[s][0]);
-            sc[2] = bf16_lo(raw.sc[s][1]); sc[3] = bf16_hi(raw.sc[s][1]);
-        }
-        __device__ __forceinline__ void unit(const Raw& raw, const BCtx& c, int s, int p, int t, u32x4_t out[4]) {
-            if ((t & 1) == 0) {
-                const int sh = 16 * (c.w & 1);
-                const int j = 2 * p;
-                const uint32_t a = pinned(raw.r[s][j >> 2][j & 3]) >> sh, b = raw.r[s][(j + 1) >> 2][(j + 1) & 3] >> sh;
-                if (t == 0) { va = e2m1_pair_to_f32<0>(a); vb = e2m1_pair_to_f32<0>(b); }
-                else        { va = e2m1_pair_to_f32<1>(a); vb = e2m1_pair_to_f32<1>(b); }
-            }
-            out[t][p] = pinned(pack_bf16_rne(pinned(va[t & 1]) * sc[t], vb[t & 1] * sc[t]));
-        }
-    };
-};
-
 // ------------------------------------------------------- int8 / reference fp8, [K, N]
 // Lane (i, q) loads the dword with columns 64w + 4i + [0,4) of each of its 8 k rows.
 template <int FMT>
 struct BTraitsByte {
     static constexpr int BK = 64, NS = 2;
-    static constexpr int B_LDS_UNITS = 0, B_LOADS = 1;
     static constexpr bool DOUBLE_RAW = false;
     static constexpr int MT_MAX = 11;
     struct Raw {
         uint32_t r[2][8];
         float s8[2];  // fp8: scale of the 128x128 block of each sub-step
     };
-    __device__ static __forceinline__ void stage_load(u32x4_t*, const BCtx&, int) {}
-    __device__ static __forceinline__ void stage_store(u32x4_t*, const u32x4_t*, const BCtx&) {}
-    __device__ static __forceinline__ void load_scale(Raw&, const BCtx&, int, int) {}
     __device__ static __forceinline__ int a_chunk(int s, int q) { return 4 * s + q; }
     __device__ static __forceinline__ int col(const BCtx& c, int t) { return 64 * c.w + 4 * c.i + t; }
     __device__ static __forceinline__ void init(BCtx& c) {
         c.vw = 8 * c.q * c.N + col(c, 0);
         c.vs = 0;
     }
-    __device__ static __forceinline__ void load_sub(Raw& raw, const BCtx& c, int k0, int s, const u32x4_t*) {
+    __device__ static __forceinline__ void load_sub(Raw& raw, const BCtx& c, int k0, int s) {
 #pragma unroll
         for (int j = 0; j < 8; ++j) raw.r[s][j] = ldg_b32(c.rw, c.vw, (k0 + 32 * s + j) * c.N + c.n0);
         if (FMT == MOE_FMT_FP8_REF) {
@@ -341,7 +187,6 @@ struct BTraits<MOE_FMT_FP8_REF> : BTraitsByte<MOE_FMT_FP8_REF> {
 template <int BLK>
 struct BTraitsFp4K {
     static constexpr int BK = 128, NS = 4;
-    static constexpr int B_LDS_UNITS = 0, B_LOADS = 1;
     // One 16-byte load per t serves all 4 sub-steps, so the registers cannot be reloaded
     // sub-step by sub-step: a whole step is loaded into a second register set (load_sub
     // ignores its sub-step argument and is called once per step).
@@ -352,16 +197,13 @@ struct BTraitsFp4K {
         u32x4_t r[4];
         uint32_t sc[4];   // block 32: the scale as fp32 bits; block 16: the two bf16 scales, unpacked where used
     };
-    __device__ static __forceinline__ void stage_load(u32x4_t*, const BCtx&, int) {}
-    __device__ static __forceinline__ void stage_store(u32x4_t*, const u32x4_t*, const BCtx&) {}
-    __device__ static __forceinline__ void load_scale(Raw&, const BCtx&, int, int) {}
     __device__ static __forceinline__ int a_chunk(int s, int q) { return 4 * q + s; }
     __device__ static __forceinline__ int col(const BCtx& c, int t) { return 64 * c.w + 16 * t + c.i; }
     __device__ static __forceinline__ void init(BCtx& c) {
         c.vw = (64 * c.w + c.i) * (c.K >> 1) + 16 * c.q;
         c.vs = ((64 * c.w + c.i) * (c.K / BLK) + SPB * c.q) * 2;
     }
-    __device__ static __forceinline__ void load_sub(Raw& raw, const BCtx& c, int k0, int, const u32x4_t*) {
+    __device__ static __forceinline__ void load_sub(Raw& raw, const BCtx& c, int k0, int) {
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
             raw.r[t] = ldg_b128(c.rw, c.vw, (c.n0 + 16 * t) * (c.K >> 1) + (k0 >> 1));
@@ -397,22 +239,18 @@ struct BTraits<MOE_FMT_FP4_B16> : BTraitsFp4K<16> {};
 template <>
 struct BTraits<MOE_FMT_BF16> {
     static constexpr int BK = 64, NS = 2;
-    static constexpr int B_LDS_UNITS = 0, B_LOADS = 1;
     static constexpr bool DOUBLE_RAW = false;
     static constexpr int MT_MAX = 11;
     struct Raw {
         u32x4_t r[4][2];
     };
-    __device__ static __forceinline__ void stage_load(u32x4_t*, const BCtx&, int) {}
-    __device__ static __forceinline__ void stage_store(u32x4_t*, const u32x4_t*, const BCtx&) {}
-    __device__ static __forceinline__ void load_scale(Raw&, const BCtx&, int, int) {}
     __device__ static __forceinline__ int a_chunk(int s, int q) { return 2 * q + s; }
     __device__ static __forceinline__ int col(const BCtx& c, int t) { return 64 * c.w + 16 * t + c.i; }
     __device__ static __forceinline__ void init(BCtx& c) {
         c.vw = (64 * c.w + c.i) * c.K * 2 + 32 * c.q;
         c.vs = 0;
     }
-    __device__ static __forceinline__ void load_sub(Raw& raw, const BCtx& c, int k0, int s, const u32x4_t*) {
+    __device__ static __forceinline__ void load_sub(Raw& raw, const BCtx& c, int k0, int s) {
 #pragma unroll
         for (int t = 0; t < 4; ++t) raw.r[t][s] = ldg_b128(c.rw, c.vw, ((c.n0 + 16 * t) * c.K + k0) * 2 + 16 * s);
     }
@@ -442,24 +280,9 @@ __device__ __forceinline__ void make_ctx(BCtx& c, const GemmParams& P, int g, in
     const int tid = threadIdx.x, lane = tid & 63;
     c.K = P.K; c.N = P.N; c.n0 = n0;
     c.i = lane & 15; c.q = lane >> 4; c.w = __builtin_amdgcn_readfirstlane(tid >> 6);
-    c.gmul = 0; c.sg = nullptr; c.og = nullptr; c.s8 = nullptr;
-    c.mlo = 0x0f0fu; c.mhi = 0xf0f0u;
-    asm volatile("" : "+s"(c.mlo), "+s"(c.mhi));
+    c.sg = nullptr; c.og = nullptr; c.s8 = nullptr;
     const int64_t KN = (int64_t)P.K * P.N;
     switch (FMT) {
-        case MOE_FMT_INT4:
-            c.rw = make_rsrc(P.w + g * (KN >> 1), KN >> 1);
-            c.rs = make_rsrc(static_cast<const uint16_t*>(P.scale) + (int64_t)g * P.scale_rows * P.N,
-                             (int64_t)P.scale_rows * P.N * 2);
-            {
-                const uint32_t per = (uint32_t)((P.K / P.scale_rows) >> 5);  // sub-steps per scale group
-                c.gmul = per == 1 ? 0u : 0xffffffffu / per + 1u;
-            }
-            break;
-        case MOE_FMT_FP4_REF:
-            c.rw = make_rsrc(P.w + g * (KN >> 1), KN >> 1);
-            c.rs = make_rsrc(static_cast<const uint16_t*>(P.scale) + g * (KN >> 4), KN >> 3);
-            break;
         case MOE_FMT_INT8:
             c.rw = make_rsrc(P.w + g * KN, KN);
             c.rs = c.rw;
@@ -491,8 +314,7 @@ template <int FMT, int MT>
 __device__ __forceinline__ void store_tile(const GemmParams& P, const BCtx& c, f32x4_t (&acc)[MT][4], int64_t row0, int rows,
                                            int n0) {
     using T = BTraits<FMT>;
-    constexpr bool N_CONTIG = (FMT == MOE_FMT_INT4 || FMT == MOE_FMT_FP4_REF || FMT == MOE_FMT_INT8 ||
-                               FMT == MOE_FMT_FP8_REF);
+    constexpr bool N_CONTIG = FMT == MOE_FMT_INT8 || FMT == MOE_FMT_FP8_REF;
     // through a buffer resource that ends after the tile's last valid row: stores to padded
     // rows fall outside it and are dropped
     if (N_CONTIG && P.epilogue == MOE_EPILOGUE_SWIGLU) {
@@ -531,8 +353,7 @@ __device__ __forceinline__ void store_tile(const GemmParams& P, const BCtx& c, f
 }
 
 template <int FMT, int MT, int CAPB>
-__device__ __forceinline__ void gemm_tile(const GemmParams& P, u32x4_t* lds_a, u32x4_t* lds_b, int g, int64_t row0,
-                                          int rows, int n0) {
+__device__ __forceinline__ void gemm_tile(const GemmParams& P, u32x4_t* lds_a, int g, int64_t row0, int rows, int n0) {
     using T = BTraits<FMT>;
     constexpr int BK = T::BK, NS = T::NS;
     constexpr int CPR = BK / 8;               // 16-byte chunks per tile row
@@ -581,10 +402,8 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& P, u32x4_t* lds_a, u
     //  * weights: while the MFMAs of sub-step f run, the fragments of sub-step f+1 are
     //    decoded, one unit (two elements of one column) at a time between MFMAs; as soon as
     //    a sub-step's packed registers have been decoded they are refilled with the same
-    //    sub-step of the next k step -- straight from global memory a full step ahead
-    //    (formats whose loads span a whole step keep a second register set), or, for the
-    //    staged formats, from the LDS copy of the next step's packed tile, which itself was
-    //    fetched with wide loads one step earlier and written before the last barrier;
+    //    sub-step of the next k step, straight from global memory a full step ahead
+    //    (formats whose loads span a whole step keep a second register set);
     //  * x: fragments come from LDS through a ring of 4 register sets, read RING
     //    fragments ahead of their MFMAs; the x tile of step kt+1 travels through registers
     //    into the other LDS buffer.
@@ -594,28 +413,11 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& P, u32x4_t* lds_a, u
     constexpr int SLOTS = 4 * MT;   // MFMAs per sub-step
     constexpr int UNITS = 17;       // prep + 16 decode units per sub-step
 
-    constexpr bool STAGED = T::B_LDS_UNITS > 0;   // packed weights travel through LDS like the x tile
-    u32x4_t breg[T::B_LOADS], breg2[T::B_LOADS];
-    auto btile = [&](int kt) { return lds_b + (kt & 1) * T::B_LDS_UNITS; };
-
     __syncthreads();  // previous tile's readers are done with both buffers
     load_a(0);
-    if (STAGED) {
-        T::stage_load(breg, c, 0);
-        T::stage_store(btile(0), breg, c);
-        T::stage_load(breg, c, BK);
-    }
     store_a(0);
-    if (STAGED) {
-        __syncthreads();
-        T::stage_store(btile(1), breg, c);
-        T::stage_load(breg, c, 2 * BK);
-    }
 #pragma unroll
-    for (int s = 0; s < (T::DOUBLE_RAW ? 1 : NS); ++s) {
-        T::load_sub(raw, c, 0, s, btile(0));
-        T::load_scale(raw, c, 0, s);
-    }
+    for (int s = 0; s < (T::DOUBLE_RAW ? 1 : NS); ++s) T::load_sub(raw, c, 0, s);
     u32x4_t bf[2][4];
     dq.prep(raw, c, 0);
 #pragma unroll
@@ -623,25 +425,18 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& P, u32x4_t* lds_a, u
 #pragma unroll
         for (int t = 0; t < 4; ++t) dq.unit(raw, c, 0, p, t, bf[0]);
     __syncthreads();
-    // raw[0] <- sub-step 0 of step 1 (direct formats: loaded a full step ahead; staged: read at the
-    // top of each step from the tile written during the previous one)
-    if (!STAGED) {
-        if (T::DOUBLE_RAW)
-            T::load_sub(raw_next, c, BK, 0, nullptr);
-        else
-            T::load_sub(raw, c, BK, 0, nullptr);
-    }
-    T::load_scale(raw, c, BK, 0);
+    // raw[0] <- sub-step 0 of step 1, a full step ahead
+    if (T::DOUBLE_RAW)
+        T::load_sub(raw_next, c, BK, 0);
+    else
+        T::load_sub(raw, c, BK, 0);
 
-    // One k step.  Staged formats fetch their packed tile two steps before it is written to
-    // LDS (three before it is used): `bload` receives tile kt+3, `bstore` (loaded during the
-    // previous step) is written as tile kt+2 at the end of this step.
-    // Global loads of the next tiles are issued one per MFMA slot at the start of the first
-    // sub-step, the LDS writes one per slot at the end of the last one, so that neither sits
-    // between the barrier and the first MFMA or between the last MFMA and the barrier.
-    constexpr int NW = PASSES + (STAGED ? 1 : 0);   // write slots: one per x pass, one for the packed tile
+    // One k step.  The global loads of the next x tile are issued one per MFMA slot at the start
+    // of the first sub-step, the LDS writes one per slot at the end of the last one, so that
+    // neither sits between the barrier and the first MFMA or between the last MFMA and the barrier.
+    constexpr int NW = PASSES;   // write slots: one per x pass
     static_assert(NW + 1 <= SLOTS, "not enough MFMA slots to spread the tile transfers over");
-    auto step = [&](int kt, u32x4_t* bload, const u32x4_t* bstore) {
+    auto step = [&](int kt) {
         const u32x4_t* la = lds_a + (kt & 1) * ABUF;
         u32x4_t afr[4];
         auto read_a = [&](int f) {
@@ -661,16 +456,8 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& P, u32x4_t* lds_a, u
                 const int mt = slot >> 2, t = slot & 3, f = s * MT + mt;
                 if (t == 0 && f + RING < F) read_a(f + RING);
                 mfma_16x16x32(acc[mt][t], afr[f & 3], bcur[t]);
-                if (s == 0) {
-                    // fetch: x tile of step kt+1, packed tile of step kt+3, then this lane's
-                    // dwords of sub-step 0 of step kt+1 from the LDS tile written last step
-                    if (slot < PASSES)
-                        areg[slot] = ldg_b128(rx, vx, (slot * RPP * P.K + (kt + 1) * BK) * 2);
-                    else if (STAGED && slot == PASSES)
-                        T::stage_load(bload, c, (kt + 3) * BK);
-                    else if (STAGED && slot == PASSES + 1)
-                        T::load_sub(raw, c, (kt + 1) * BK, 0, btile(kt + 1));
-                }
+                // fetch the x tile of step kt+1
+                if (s == 0 && slot < PASSES) areg[slot] = ldg_b128(rx, vx, (slot * RPP * P.K + (kt + 1) * BK) * 2);
                 // decode units u with floor(u * SLOTS / UNITS) == slot
 #pragma unroll
                 for (int u = (slot * UNITS + SLOTS - 1) / SLOTS; u < ((slot + 1) * UNITS + SLOTS - 1) / SLOTS; ++u) {
@@ -681,35 +468,22 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& P, u32x4_t* lds_a, u
                 }
                 if (slot == ((UNITS - 1) * SLOTS) / UNITS) {
                     // everything of sub-step sn has been decoded: refill its registers
-                    T::load_scale(raw, c, (kt + (sn == 0 ? 2 : 1)) * BK, sn);
-                    if (STAGED) {
-                        if (sn != 0) T::load_sub(raw, c, (kt + 1) * BK, sn, btile(kt + 1));
-                    } else if (T::DOUBLE_RAW) {
-                        if (sn == 0) T::load_sub(raw_next, c, (kt + 2) * BK, 0, nullptr);
+                    if (T::DOUBLE_RAW) {
+                        if (sn == 0) T::load_sub(raw_next, c, (kt + 2) * BK, 0);
                     } else {
-                        T::load_sub(raw, c, (kt + (sn == 0 ? 2 : 1)) * BK, sn, nullptr);
+                        T::load_sub(raw, c, (kt + (sn == 0 ? 2 : 1)) * BK, sn);
                     }
                 }
                 if (s == NS - 1 && slot >= SLOTS - NW) {
                     const int wi = slot - (SLOTS - NW);
-                    if (wi < PASSES)
-                        lds_a[((kt + 1) & 1) * ABUF + a_lds_unit<BK>(ar + RPP * wi, ac)] = areg[wi];
-                    else if (wi == PASSES)
-                        T::stage_store(btile(kt + 2), bstore, c);
+                    lds_a[((kt + 1) & 1) * ABUF + a_lds_unit<BK>(ar + RPP * wi, ac)] = areg[wi];
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
         __syncthreads();
     };
-    if (STAGED) {
-        for (int kt = 0; kt < nk; kt += 2) {
-            step(kt, breg2, breg);
-            if (kt + 1 < nk) step(kt + 1, breg, breg2);
-        }
-    } else {
-        for (int kt = 0; kt < nk; ++kt) step(kt, breg, breg);
-    }
+    for (int kt = 0; kt < nk; ++kt) step(kt);
     // the accumulators were last written by MFMAs the compiler cannot see: wait out their latency
     asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
 
@@ -728,7 +502,7 @@ __device__ __forceinline__ void lds_load16(rsrc_t r, const u32x4_t* dst, int vof
 }
 
 // ---------------------------------------------------------------------------------
-// Prefill tile routine for int4 with two wavefronts per SIMD that split the k range.
+// Tile routine for int4 and the reference fp4 container with two wavefronts per SIMD that split the k range.
 //
 // A single wavefront issues at most one instruction every ~5 cycles whatever its kind, and an
 // MFMA holds the SIMD's vector issue port for about 8 of its 16 cycles: with one wavefront
@@ -1149,7 +923,7 @@ __device__ __forceinline__ void expert_chunks(int m, int& chunks, int& bpc) {
 //   GK_GENERAL  4 wavefronts of 64 columns, one workgroup per CU, tiles of up to 192 rows
 //   GK_SKINNY   the same tile routine with tiles of at most 32 rows and several workgroups per CU
 //               (decode-sized batches are HBM bound: more weight bytes in flight)
-//   GK_PAIR     int4 prefill: 8 wavefronts, k range split between the two wavefronts of a SIMD
+//   GK_PAIR     int4 / reference fp4: 8 wavefronts, k range split between the two wavefronts of a SIMD
 //   GK_PAIR_EXACT  GK_PAIR with the GEMV op's arithmetic (weights not rounded to bf16), tiles of at most 32 rows
 enum { GK_GENERAL = 0, GK_SKINNY = 1, GK_PAIR = 2, GK_PAIR_EXACT = 3 };
 constexpr int PAIR_EXACT_MT_MAX = 2;
@@ -1164,7 +938,10 @@ struct KernelCfg {
     static constexpr int WG_PER_CU = KIND == GK_SKINNY ? GM_SKINNY_WAVES : 1;
     static constexpr int CAPB = KIND == GK_SKINNY ? GM_SKINNY_BLOCKS : PAIR ? PAIR_CAPB : GM_MT_MAX;
     static constexpr int fmt_mt_max() {
-        return KIND == GK_PAIR ? PAIR_MT_MAX : KIND == GK_PAIR_EXACT ? PAIR_EXACT_MT_MAX : BTraits<FMT>::MT_MAX;
+        if constexpr (PAIR)
+            return KIND == GK_PAIR ? PAIR_MT_MAX : PAIR_EXACT_MT_MAX;
+        else
+            return BTraits<FMT>::MT_MAX;
     }
     static constexpr int MTM = CAPB < fmt_mt_max() ? CAPB : fmt_mt_max();        // row blocks per tile
     // 16-byte LDS units of the tile routine (the tile prefix array follows them)
@@ -1172,7 +949,7 @@ struct KernelCfg {
         if constexpr (PAIR)
             return pair_lds_units<FMT>();
         else
-            return 2 * 16 * CAPB * (BTraits<FMT>::BK / 8) + 2 * BTraits<FMT>::B_LDS_UNITS;
+            return 2 * 16 * CAPB * (BTraits<FMT>::BK / 8);
     }
 };
 
@@ -1182,7 +959,7 @@ __device__ __forceinline__ void run_tile(const GemmParams& P, u32x4_t* smem, int
     if constexpr (C::PAIR)
         gemm_tile_pair<FMT, MT, KIND == GK_PAIR_EXACT>(P, smem, g, row0, rows, n0);
     else
-        gemm_tile<FMT, MT, C::CAPB>(P, smem, smem + 2 * 16 * C::CAPB * (BTraits<FMT>::BK / 8), g, row0, rows, n0);
+        gemm_tile<FMT, MT, C::CAPB>(P, smem, g, row0, rows, n0);
 }
 
 template <int FMT, int KIND>
