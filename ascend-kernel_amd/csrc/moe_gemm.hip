@@ -177,6 +177,14 @@ struct BTraits<MOE_FMT_FP8_REF> : BTraitsByte<MOE_FMT_FP8_REF> {
             const float sc = raw.s8[s] * 256.f;
             out[t][p] = pinned(pack_bf16_rne(v[0] * sc, v[1] * sc));
         }
+        // GEMV arithmetic: the codes themselves (worth 2^-8 of their value, exact in bf16); the block
+        // scale is applied to the sums of each 128-k block
+        __device__ __forceinline__ void unit_exact(const Raw& raw, const BCtx&, int s, int p, int t, u32x4_t out[4]) {
+            const uint32_t a = pinned(raw.r[s][2 * p]), b = raw.r[s][2 * p + 1];
+            const uint32_t sel = (uint32_t)t | 0x0c00u | ((uint32_t)(4 + t) << 16) | 0x0c000000u;
+            const f32x2_t v = e4m3_ref_pair_over_256(__builtin_amdgcn_perm(b, a, sel));
+            out[t][p] = pinned(pack_bf16_rne(v[0], v[1]));
+        }
     };
 };
 
@@ -352,8 +360,13 @@ __device__ __forceinline__ void store_tile(const GemmParams& P, const BCtx& c, f
         }
 }
 
-template <int FMT, int MT, int CAPB>
+// EXACT (reference fp8 container only) selects the arithmetic of the GEMV op, whose dequantized weights
+// stay fp32 (grouped_soft_gemv/op_kernel/gemv_impl.h:147-199): the B fragments hold the e4m3 values
+// themselves (exact in bf16), the sums of every 128-k scale block are kept apart and multiplied by the
+// block's fp32 scale when the block ends.  Its MFMAs are compiler builtins (their results feed VALU code).
+template <int FMT, int MT, int CAPB, bool EXACT = false>
 __device__ __forceinline__ void gemm_tile(const GemmParams& P, u32x4_t* lds_a, int g, int64_t row0, int rows, int n0) {
+    static_assert(!EXACT || FMT == MOE_FMT_FP8_REF, "un-rounded weights: reference fp8 container only");
     using T = BTraits<FMT>;
     constexpr int BK = T::BK, NS = T::NS;
     constexpr int CPR = BK / 8;               // 16-byte chunks per tile row
@@ -379,6 +392,13 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& P, u32x4_t* lds_a, i
     for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
         for (int t = 0; t < 4; ++t) acc[mt][t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    // EXACT: sums of the current 128-k scale block and that block's scale (times the 2^8 the decode leaves out)
+    f32x4_t part[EXACT ? MT : 1][4];
+    float sblk = 0.f;
+#pragma unroll
+    for (int mt = 0; mt < (EXACT ? MT : 1); ++mt)
+#pragma unroll
+        for (int t = 0; t < 4; ++t) part[mt][t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
     u32x4_t areg[PASSES];
     typename T::Raw raw, raw_next;
@@ -423,7 +443,10 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& P, u32x4_t* lds_a, i
 #pragma unroll
     for (int p = 0; p < 4; ++p)
 #pragma unroll
-        for (int t = 0; t < 4; ++t) dq.unit(raw, c, 0, p, t, bf[0]);
+        for (int t = 0; t < 4; ++t) {
+            if constexpr (EXACT) dq.unit_exact(raw, c, 0, p, t, bf[0]);
+            else dq.unit(raw, c, 0, p, t, bf[0]);
+        }
     __syncthreads();
     // raw[0] <- sub-step 0 of step 1, a full step ahead
     if (T::DOUBLE_RAW)
@@ -439,6 +462,8 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& P, u32x4_t* lds_a, i
     auto step = [&](int kt) {
         const u32x4_t* la = lds_a + (kt & 1) * ABUF;
         u32x4_t afr[4];
+        if constexpr (EXACT)
+            if ((kt & 1) == 0) sblk = c.s8[(kt >> 1) * (c.N >> 7) + ((c.n0 + 64 * c.w) >> 7)] * 256.f;
         auto read_a = [&](int f) {
             afr[f & 3] = la[a_lds_unit<BK>(16 * (f % MT) + c.i, T::a_chunk(f / MT, c.q))];
         };
@@ -455,7 +480,11 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& P, u32x4_t* lds_a, i
             for (int slot = 0; slot < SLOTS; ++slot) {
                 const int mt = slot >> 2, t = slot & 3, f = s * MT + mt;
                 if (t == 0 && f + RING < F) read_a(f + RING);
-                mfma_16x16x32(acc[mt][t], afr[f & 3], bcur[t]);
+                if constexpr (EXACT)
+                    part[mt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, afr[f & 3]),
+                                                                          __builtin_bit_cast(bf16x8_t, bcur[t]), part[mt][t], 0, 0, 0);
+                else
+                    mfma_16x16x32(acc[mt][t], afr[f & 3], bcur[t]);
                 // fetch the x tile of step kt+1
                 if (s == 0 && slot < PASSES) areg[slot] = ldg_b128(rx, vx, (slot * RPP * P.K + (kt + 1) * BK) * 2);
                 // decode units u with floor(u * SLOTS / UNITS) == slot
@@ -463,6 +492,8 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& P, u32x4_t* lds_a, i
                 for (int u = (slot * UNITS + SLOTS - 1) / SLOTS; u < ((slot + 1) * UNITS + SLOTS - 1) / SLOTS; ++u) {
                     if (u == 0)
                         dq.prep(raw, c, sn);
+                    else if constexpr (EXACT)
+                        dq.unit_exact(raw, c, sn, (u - 1) >> 2, (u - 1) & 3, bnxt);
                     else
                         dq.unit(raw, c, sn, (u - 1) >> 2, (u - 1) & 3, bnxt);
                 }
@@ -479,6 +510,18 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& P, u32x4_t* lds_a, i
                     lds_a[((kt + 1) & 1) * ABUF + a_lds_unit<BK>(ar + RPP * wi, ac)] = areg[wi];
                 }
                 __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+        if constexpr (EXACT) {
+            if (kt & 1) {   // a 128-k scale block ends with every second 64-k step
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+                    for (int t = 0; t < 4; ++t) {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) acc[mt][t][e] = fmaf(part[mt][t][e], sblk, acc[mt][t][e]);
+                        part[mt][t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+                    }
             }
         }
         __syncthreads();
@@ -925,18 +968,20 @@ __device__ __forceinline__ void expert_chunks(int m, int& chunks, int& bpc) {
 //               (decode-sized batches are HBM bound: more weight bytes in flight)
 //   GK_PAIR     int4 / reference fp4: 8 wavefronts, k range split between the two wavefronts of a SIMD
 //   GK_PAIR_EXACT  GK_PAIR with the GEMV op's arithmetic (weights not rounded to bf16), tiles of at most 32 rows
-enum { GK_GENERAL = 0, GK_SKINNY = 1, GK_PAIR = 2, GK_PAIR_EXACT = 3 };
+//   GK_SKINNY_EXACT  GK_SKINNY with the GEMV op's arithmetic (reference fp8 container)
+enum { GK_GENERAL = 0, GK_SKINNY = 1, GK_PAIR = 2, GK_PAIR_EXACT = 3, GK_SKINNY_EXACT = 4 };
 constexpr int PAIR_EXACT_MT_MAX = 2;
 
 template <int FMT, int KIND>
 struct KernelCfg {
     static constexpr bool PAIR = KIND == GK_PAIR || KIND == GK_PAIR_EXACT;
+    static constexpr bool SKINNY = KIND == GK_SKINNY || KIND == GK_SKINNY_EXACT;
     static_assert(!PAIR || FMT == MOE_FMT_INT4 || FMT == MOE_FMT_FP4_REF,
                   "the k-split tile routine decodes int4 and the reference fp4 container");
     static constexpr int WAVES = PAIR ? 8 : 4;
     static constexpr int BN = GM_BN;                                             // columns per tile
-    static constexpr int WG_PER_CU = KIND == GK_SKINNY ? GM_SKINNY_WAVES : 1;
-    static constexpr int CAPB = KIND == GK_SKINNY ? GM_SKINNY_BLOCKS : PAIR ? PAIR_CAPB : GM_MT_MAX;
+    static constexpr int WG_PER_CU = SKINNY ? GM_SKINNY_WAVES : 1;
+    static constexpr int CAPB = SKINNY ? GM_SKINNY_BLOCKS : PAIR ? PAIR_CAPB : GM_MT_MAX;
     static constexpr int fmt_mt_max() {
         if constexpr (PAIR)
             return KIND == GK_PAIR ? PAIR_MT_MAX : PAIR_EXACT_MT_MAX;
@@ -959,7 +1004,7 @@ __device__ __forceinline__ void run_tile(const GemmParams& P, u32x4_t* smem, int
     if constexpr (C::PAIR)
         gemm_tile_pair<FMT, MT, KIND == GK_PAIR_EXACT>(P, smem, g, row0, rows, n0);
     else
-        gemm_tile<FMT, MT, C::CAPB>(P, smem, g, row0, rows, n0);
+        gemm_tile<FMT, MT, C::CAPB, KIND == GK_SKINNY_EXACT>(P, smem, g, row0, rows, n0);
 }
 
 template <int FMT, int KIND>
@@ -1140,6 +1185,7 @@ int launch_gemm_exact(const moe_grouped_args* a, hipStream_t stream) {
     switch (a->format) {
         case MOE_FMT_FP4_REF: return launch_gemm_kind<MOE_FMT_FP4_REF, GK_PAIR_EXACT>(P, a, stream);
         case MOE_FMT_INT4: return launch_gemm_kind<MOE_FMT_INT4, GK_PAIR_EXACT>(P, a, stream);
+        case MOE_FMT_FP8_REF: return launch_gemm_kind<MOE_FMT_FP8_REF, GK_SKINNY_EXACT>(P, a, stream);
         default: return MOE_ERR_BAD_FORMAT;
     }
 }

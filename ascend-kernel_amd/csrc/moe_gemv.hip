@@ -720,14 +720,16 @@ int launch_grouped_gemv(const moe_grouped_args* a, hipStream_t stream, bool gemm
             if (a->K % GF_KSTEP != 0) return gemm_rounding ? MOE_ERR_BAD_SHAPE : launch_kmajor<MOE_FMT_FP4_B16>(a, stream);
             return gemm_rounding ? launch_fp4_mfma<true, 16>(a, stream) : launch_fp4_mfma<false, 16>(a, stream);
         case MOE_FMT_FP4_REF:
-        case MOE_FMT_INT4: {
-            // the k-split matrix-core kernel with this op's arithmetic (fp32 weights); the vector kernel
-            // only where the expert count does not fit that kernel's tile table in LDS
+        case MOE_FMT_INT4:
+        case MOE_FMT_FP8_REF: {
+            // the matrix-core GEMM kernels run with this op's arithmetic (fp32 weights); the vector kernel
+            // only where the expert count does not fit those kernels' tile table in LDS
             const int rc = launch_gemm_exact(a, stream);
             if (rc != MOE_ERR_TOO_LARGE) return rc;
-            return a->format == MOE_FMT_INT4 ? launch_nmajor<MOE_FMT_INT4>(a, stream) : launch_nmajor<MOE_FMT_FP4_REF>(a, stream);
+            return a->format == MOE_FMT_INT4      ? launch_nmajor<MOE_FMT_INT4>(a, stream)
+                   : a->format == MOE_FMT_FP4_REF ? launch_nmajor<MOE_FMT_FP4_REF>(a, stream)
+                                                  : launch_nmajor<MOE_FMT_FP8_REF>(a, stream);
         }
-        case MOE_FMT_FP8_REF: return launch_nmajor<MOE_FMT_FP8_REF>(a, stream);
         default: return MOE_ERR_BAD_FORMAT;
     }
 }

@@ -265,11 +265,12 @@ def test_gemv_fp4_b32_row_counts_up_to_and_beyond_16(K, N, fmt):
 
 @pytest.mark.parametrize("fmt,K,N,group", [("fp4", 1024, 256, 16), ("fp4", 7168, 512, 16), ("fp4", 64, 256, 16),
                                            ("int4", 1024, 256, 128), ("int4", 7168, 512, 128), ("int4", 192, 256, 32),
-                                           ("int4", 256, 256, 64)])
+                                           ("int4", 256, 256, 64), ("fp8", 1024, 256, 128), ("fp8", 7168, 512, 128),
+                                           ("fp8", 128, 256, 128)])
 def test_gemv_n_contiguous_row_counts_up_to_and_beyond_32(fmt, K, N, group):
-    """The GEMV op on the reference fp4 container and on int4 runs on the matrix cores with weights that are
-    not rounded to bf16 (the codes go through the MFMA, the fp32 scales are applied to its results), in
-    tiles of up to 32 rows of an expert; K = 64 is a single k step."""
+    """The GEMV op on the reference fp4 / fp8 containers and on int4 runs on the matrix cores with weights
+    that are not rounded to bf16 (the codes go through the MFMA, the fp32 scales are applied to its
+    results), in tiles of up to 32 rows of an expert; K = 64 (fp8: 128) is a single scale block."""
     _say(f"gemv {fmt} rows K={K} N={N} group={group}")
     counts = [1, 0, 4, 5, 16, 17, 32, 33, 70, 0, 3]
     gl = list(np.cumsum(counts))
@@ -279,7 +280,7 @@ def test_gemv_n_contiguous_row_counts_up_to_and_beyond_32(fmt, K, N, group):
     assert (got[gl[-1]:] == 0x7FC0).all()
 
 
-@pytest.mark.parametrize("fmt", ["fp4", "int4"])
+@pytest.mark.parametrize("fmt", ["fp4", "int4", "fp8"])
 def test_gemv_n_contiguous_more_experts_than_the_matrix_core_kernel_takes(fmt):
     """The k-split kernel keeps a tile table of G + 1 entries in LDS; beyond its capacity the GEMV op
     falls back to the vector kernel."""
@@ -288,7 +289,7 @@ def test_gemv_n_contiguous_more_experts_than_the_matrix_core_kernel_takes(fmt):
     rng = np.random.default_rng(11)
     counts = rng.integers(0, 3, G)
     gl = list(np.cumsum(counts))
-    case = H.make_case(fmt, G, 128, 256, gl, seed=12, group=32 if fmt == "int4" else 16)
+    case = H.make_case(fmt, G, 128, 256, gl, seed=12, group=32 if fmt == "int4" else 128 if fmt == "fp8" else 16)
     got = H.run_cabi(case, H.upload(case), "gemv")
     H.assert_close(got, H.oracle_out(case, gemv=True), what=f"gemv {fmt} G={G}")
 
