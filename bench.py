@@ -283,6 +283,28 @@ def run_extra(torch, mg, gen, iters, warmup):
                                              separate_gemm_us=t_s * 1e6, speedup_vs_separate=(t_d + t_s) / t_f,
                                              gemv_op_us=t_v * 1e6, gemv_op_frac_hbm=nbytes / t_v / 1e9 / PEAK_HBM_GBS,
                                              max_abs_diff_fused_vs_separate=diff)
+    del w, s, wd, y2, y3, fused, sep, gemv
+
+    # the same decode batch on the reference's own containers (N-contiguous: pre-shuffled fp4 with per-16
+    # scales, fp8 with 128 x 128 block scales) and on int4 group-128, through both ops
+    ref = {}
+    for fmt, wshape, sshape, srows, wbytes in (
+            ("fp4", (G, K, N // 2), (G, K // 16, N), K // 16, N * K // 2 + (K // 16) * N * 2),
+            ("int4", (G, K, N // 2), (G, K // 128, N), K // 128, N * K // 2 + (K // 128) * N * 2),
+            ("fp8", (G, K, N), (G, K // 128, N // 128), K // 128, N * K + (K // 128) * (N // 128) * 4)):
+        w = torch.randint(0, 255, wshape, dtype=torch.uint8, device="cuda")
+        if fmt == "fp8":
+            s = torch.rand(sshape, device="cuda") * 1e-2 + 1e-3
+        else:
+            s = bf16_uniform(torch, sshape, 2.0 ** -8, 2.0 ** -2)
+        w = w.view(torch.int8) if fmt == "fp4" else w
+        ops = [Op(mg, torch, kind, fmt, x, w, s, None, gl, y, scale_rows=srows) for kind in ("gemv", "gemm")]
+        t_v, t_m = time_launches(torch, ops, max(iters // 2, 5), warmup)
+        nbytes = A * wbytes + M * K * 2 + M * N * 2
+        ref[fmt] = dict(bytes=nbytes, gemv_op_us=t_v * 1e6, gemv_op_frac_hbm=nbytes / t_v / 1e9 / PEAK_HBM_GBS,
+                        gemm_op_us=t_m * 1e6, gemm_op_frac_hbm=nbytes / t_m / 1e9 / PEAK_HBM_GBS)
+        del w, s, ops
+    out["decode_256e_reference_containers"] = dict(active_experts=A, rows=M, **ref)
     return out
 
 
