@@ -585,14 +585,18 @@ __device__ __forceinline__ void lds_load16(rsrc_t r, const u32x4_t* dst, int vof
 constexpr int PAIR_CAPB = 10;                         // x stages hold 160 rows
 constexpr int PAIR_MT_MAX = 10;
 constexpr int PAIR_A_UNITS = 16 * PAIR_CAPB * 8;      // 16-byte units of one x stage
-constexpr int PAIR_B_UNITS = 64 * 8;                  // packed int4 tile of one k step: 64 rows of 128 bytes
-constexpr int PAIR_STAGES = 5;
+// packed tile of one k step: 64 rows of 128 bytes (4-bit codes) or of 256 bytes (int8)
+template <int FMT>
+constexpr int pair_b_units() { return FMT == MOE_FMT_INT8 ? 64 * 16 : 64 * 8; }
+// ring depth: what fits into LDS next to the x stages
+template <int FMT>
+constexpr int pair_stages() { return FMT == MOE_FMT_INT8 ? 4 : 5; }
 // scale rows of 256 bf16 per k step: int4 one per 32-k sub-step (groups are multiples of 32), the
 // reference fp4 container one per 16 k
 template <int FMT>
-constexpr int pair_sc_rows() { return FMT == MOE_FMT_FP4_REF ? 4 : 2; }
+constexpr int pair_sc_rows() { return FMT == MOE_FMT_FP4_REF ? 4 : FMT == MOE_FMT_INT8 ? 0 : 2; }
 template <int FMT>
-constexpr int pair_lds_units() { return PAIR_STAGES * (PAIR_A_UNITS + PAIR_B_UNITS + 32 * pair_sc_rows<FMT>()); }
+constexpr int pair_lds_units() { return pair_stages<FMT>() * (PAIR_A_UNITS + pair_b_units<FMT>() + 32 * pair_sc_rows<FMT>()); }
 
 // EXACT selects the arithmetic of the GEMV op (grouped_soft_gemv/op_kernel/gemv_impl.h:147-199: the
 // dequantized weights stay fp32): the B fragments then hold the codes themselves, which are exact in
@@ -602,9 +606,13 @@ constexpr int pair_lds_units() { return PAIR_STAGES * (PAIR_A_UNITS + PAIR_B_UNI
 // own MFMA.  These MFMAs are compiler-visible builtins (their results feed ordinary VALU code).
 template <int FMT, int MT, bool EXACT = false>
 __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* smem, int g, int64_t row0, int rows, int n0) {
-    static_assert(FMT == MOE_FMT_INT4 || FMT == MOE_FMT_FP4_REF, "the k-split tile routine decodes int4 and the reference fp4 container");
-    constexpr bool FP4 = FMT == MOE_FMT_FP4_REF;
-    constexpr int BK = 64, S = PAIR_STAGES, SC_ROWS = pair_sc_rows<FMT>(), PAIR_SC_UNITS = 32 * SC_ROWS;
+    static_assert(FMT == MOE_FMT_INT4 || FMT == MOE_FMT_FP4_REF || FMT == MOE_FMT_INT8,
+                  "the k-split tile routine decodes int4, int8 and the reference fp4 container");
+    static_assert(!EXACT || FMT != MOE_FMT_INT8, "the GEMV op has no int8 container");
+    constexpr bool FP4 = FMT == MOE_FMT_FP4_REF, I8 = FMT == MOE_FMT_INT8;
+    constexpr int BK = 64, S = pair_stages<FMT>(), SC_ROWS = pair_sc_rows<FMT>(), PAIR_SC_UNITS = 32 * SC_ROWS;
+    constexpr int PAIR_B_UNITS = pair_b_units<FMT>();
+    constexpr int AHEAD = S - 1;   // a step's loads fill the stage of step kt + AHEAD
     u32x4_t* lds_a = smem;
     u32x4_t* lds_b = lds_a + S * PAIR_A_UNITS;
     u32x4_t* lds_s = lds_b + S * PAIR_B_UNITS;
@@ -617,14 +625,15 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
     // wavefront in the lower slot (wv < 4); measured, the pair runs 20 % faster when that one takes
     // the role whose barrier sits inside the decode phase
     const int h = 1 - (wv >> 2);
-    const int col0 = 128 * (cw >> 1) + 8 * i + 4 * (cw & 1);  // this lane's 4 columns (MFMA t = column col0 + t)
+    // this lane's 4 columns (MFMA t = column col0 + t): half of a dword of 8 4-bit codes, or a dword of 4 bytes
+    const int col0 = I8 ? 64 * cw + 4 * i : 128 * (cw >> 1) + 8 * i + 4 * (cw & 1);
     const int nk = P.K / BK;
 
     const int64_t KN = (int64_t)P.K * P.N;
-    const rsrc_t rw = make_rsrc(P.w + g * (KN >> 1), KN >> 1);
+    const rsrc_t rw = I8 ? make_rsrc(P.w + g * KN, KN) : make_rsrc(P.w + g * (KN >> 1), KN >> 1);
     const rsrc_t rs = make_rsrc(static_cast<const uint16_t*>(P.scale) + (int64_t)g * P.scale_rows * P.N,
                                 (int64_t)P.scale_rows * P.N * 2);
-    const uint32_t per = (uint32_t)((P.K / P.scale_rows) >> 5);      // 32-k sub-steps per scale group
+    const uint32_t per = I8 ? 1u : (uint32_t)((P.K / P.scale_rows) >> 5);      // 32-k sub-steps per scale group
     const uint32_t gmul = per == 1 ? 0u : 0xffffffffu / per + 1u;   // sub-step -> scale row as a multiply
     auto scale_row = [&](uint32_t sub) { return gmul ? (int)__umulhi(sub, gmul) : (int)sub; };
     // x rows through a buffer resource that ends after the last valid row (padded rows read as
@@ -635,9 +644,14 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
     // packed tile: instruction wv brings rows 8 wv + (lane >> 3) into the 1 KB block wv of the stage;
     // the two 64-byte halves of the rows with odd (row >> 3) are swapped, so that the four q groups
     // of a wavefront read from both halves of the banks
-    const int vb = (lane >> 3) * (P.N >> 1) + (((lane & 7) ^ (4 * (wv & 1))) * 16);
+    // int8 (rows of 256 bytes): instruction e of wavefront wv brings rows 8 wv + 4 e + (lane >> 4); the
+    // 64-byte quarters of a row are permuted by (row >> 3) & 3 = wv & 3, so that the four q groups read
+    // from different quarters of the banks
+    const int vb = I8 ? (lane >> 4) * P.N + (((lane & 15) ^ (4 * (wv & 3))) * 16)
+                      : (lane >> 3) * (P.N >> 1) + (((lane & 7) ^ (4 * (wv & 1))) * 16);
     constexpr int NA = (2 * MT + 7) / 8;   // x load instructions per wavefront per step
-    constexpr int NI = NA + 2;             // + one packed-tile instruction + an eighth of the scales
+    constexpr int NB = I8 ? 2 : 1;         // packed-tile instructions
+    constexpr int NI = NA + NB + (SC_ROWS ? 1 : 0);   // + an eighth of the step's scales
     int ja[NA], ca[NA];
 #pragma unroll
     for (int m = 0; m < NA; ++m) {
@@ -646,21 +660,23 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
         ja[m] = j * 64;
         ca[m] = 8 * j * P.K * 2;
     }
-    const int cb = 8 * wv * (P.N >> 1) + (n0 >> 1);
-    const int kb_step = BK * (P.N >> 1);
+    const int cb = I8 ? 8 * wv * P.N + n0 : 8 * wv * (P.N >> 1) + (n0 >> 1);
+    const int kb_step = I8 ? BK * P.N : BK * (P.N >> 1);
     // scales of a step: int4 2 rows of 512 bytes, 128 bytes (8 lanes) per wavefront: bytes [128 (wv & 3), +128) of
     // row wv >> 2; fp4 4 rows (one per 16 k), 256 bytes (16 lanes) per wavefront: bytes [256 (wv & 1), +256) of row wv >> 1
     const int cs = FP4 ? n0 * 2 + (wv & 1) * 256 : n0 * 2 + (wv & 3) * 128;
     const int lane16 = lane * 16;
     const bool s_lane = lane < (FP4 ? 16 : 8);
-    // m-th load of group kt (stage kt+4 of x, packed tile and scales), into LDS stage ST
+    // m-th load of group kt (stage kt+AHEAD of x, packed tile and scales), into LDS stage ST
     auto issue = [&](int m, int kt, int ST) {
         if (m < NA) {
-            lds_load16(rx, lds_a + ST * PAIR_A_UNITS + ja[m], va, ca[m] + (kt + 4) * (BK * 2));
-        } else if (m == NA) {
-            lds_load16(rw, lds_b + ST * PAIR_B_UNITS + wv * 64, vb, cb + (kt + 4) * kb_step);
+            lds_load16(rx, lds_a + ST * PAIR_A_UNITS + ja[m], va, ca[m] + (kt + AHEAD) * (BK * 2));
+        } else if (m < NA + NB) {
+            const int e = m - NA;
+            lds_load16(rw, lds_b + ST * PAIR_B_UNITS + wv * (PAIR_B_UNITS / 8) + e * 64, vb,
+                       cb + (I8 ? 4 * e * P.N : 0) + (kt + AHEAD) * kb_step);
         } else {
-            const int grow = FP4 ? (kt + 4) * 4 + (wv >> 1) : scale_row((uint32_t)((kt + 4) * 2 + (wv >> 2)));
+            const int grow = FP4 ? (kt + AHEAD) * 4 + (wv >> 1) : scale_row((uint32_t)((kt + AHEAD) * 2 + (wv >> 2)));
             if (s_lane) lds_load16(rs, lds_s + ST * PAIR_SC_UNITS + wv * (PAIR_SC_UNITS / 8), lane16, grow * (P.N * 2) + cs);
         }
     };
@@ -695,16 +711,28 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
     constexpr int RING = 3;
     constexpr int R = RING < MT ? RING : MT;   // x fragments read ahead of their MFMAs
 
-    // groups -4 .. -1: stages 0 .. 3; stages 0 and 1 must have landed before the first barrier
-    issue_group(-4, 0);
-    issue_group(-3, 1);
-    issue_group(-2, 2);
-    issue_group(-1, 3);
-    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(2 * NI) : "memory");
+    // int8: per-channel scale and offset of this lane's 4 columns, fixed for the tile (ordinary loads,
+    // older than every ring load: the counted waits below cover them)
+    float ch_s[4] = {0.f, 0.f, 0.f, 0.f}, ch_o[4] = {0.f, 0.f, 0.f, 0.f};
+    u32x2_t ch_sb = {0u, 0u}, ch_ob = {0u, 0u};
+    if constexpr (I8) {
+        ch_sb = *reinterpret_cast<const u32x2_t*>(static_cast<const uint16_t*>(P.scale) + (int64_t)g * P.N + n0 + col0);
+        ch_ob = *reinterpret_cast<const u32x2_t*>(P.offset + (int64_t)g * P.N + n0 + col0);
+    }
+    // groups -AHEAD .. -1: stages 0 .. AHEAD-1; stages 0 and 1 must have landed before the first barrier
+    // (WAITN: the loads of the S - 3 youngest groups may still be in flight at a barrier)
+    constexpr int WAITN = (S - 3) * NI;
+#pragma unroll
+    for (int st0 = 0; st0 < AHEAD; ++st0) issue_group(st0 - AHEAD, st0);
+    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(WAITN) : "memory");
+    if constexpr (I8) {
+        ch_s[0] = bf16_lo(ch_sb[0]); ch_s[1] = bf16_hi(ch_sb[0]); ch_s[2] = bf16_lo(ch_sb[1]); ch_s[3] = bf16_hi(ch_sb[1]);
+        ch_o[0] = bf16_lo(ch_ob[0]); ch_o[1] = bf16_hi(ch_ob[0]); ch_o[2] = bf16_lo(ch_ob[1]); ch_o[3] = bf16_hi(ch_ob[1]);
+    }
 
     // this lane's packed dwords and scales of its sub-step of LDS stage st
     uint32_t r[8];
-    u32x2_t sc, sc2 = {0u, 0u};   // sc2: with EXACT, the fp4 scales of the second 16 k of the sub-step
+    u32x2_t sc = {0u, 0u}, sc2 = {0u, 0u};   // sc2: with EXACT, the fp4 scales of the second 16 k of the sub-step
     auto read_raw = [&](int st) {
         const uint16_t* sc16 = reinterpret_cast<const uint16_t*>(lds_s + st * PAIR_SC_UNITS);
         if constexpr (FP4) {
@@ -724,6 +752,12 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
             } else {
                 sc = *reinterpret_cast<const u32x2_t*>(sc16 + 256 * (2 * h + (q >> 1)) + col0);
             }
+        } else if constexpr (I8) {
+            // dword 16 cw + i of each of this lane's 8 k rows; the quarter of the row it lies in is
+            // permuted by (row >> 3) & 3 = q (see vb)
+            const uint32_t* t32 = reinterpret_cast<const uint32_t*>(lds_b + st * PAIR_B_UNITS);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) r[j] = t32[(32 * h + 8 * q + j) * 64 + 16 * (cw ^ q) + i];
         } else {
             const uint32_t* t32 = reinterpret_cast<const uint32_t*>(lds_b + st * PAIR_B_UNITS);
 #pragma unroll
@@ -733,7 +767,7 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
     };
     read_raw(0);
 
-    // One data step; st = step mod 5 is its LDS stage, sn the next one, sl the stage this step's loads
+    // One data step; st = step mod S is its LDS stage, sn the next one, sl the stage this step's loads
     // go to (wave-uniform).
     auto step = [&](int kt, int st, int sn, int sl) {
         const u32x4_t* la = lds_a + st * PAIR_A_UNITS;
@@ -763,11 +797,27 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
                     // barrier kt-1 for the wavefronts that own sub-step 1, half way through their decode
                     // (not in the tile's first step: the barrier of the prologue stands for it); x stage
                     // kt is visible behind it
-                    if (kt > 0) asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(2 * NI) : "memory");
+                    if (kt > 0) asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(WAITN) : "memory");
                 }
                 // first x fragments of the MFMA phase, read under the rest of the decode
 #pragma unroll
                 for (int f = 0; f < R; ++f) afr[f & 3] = la[a_lds_unit<BK>(16 * f + i, 4 * h + q)];
+            }
+            if constexpr (I8) {
+                // byte t of the dwords of k rows 2p, 2p+1 -> (q + offset) * scale as two rounded fp32
+                // operations -> bf16 pair along k
+#pragma unroll
+                for (int p = 0; p < 2; ++p) {
+                    const uint32_t a = r[2 * (p0 + p)], b = r[2 * (p0 + p) + 1];
+#pragma unroll
+                    for (int t = 0; t < 4; ++t) {
+                        const float qa = (float)(int)(int8_t)(a >> (8 * t)), qb = (float)(int)(int8_t)(b >> (8 * t));
+                        bf[t][p0 + p] = pack_bf16_rne(__fmul_rn(__fadd_rn(qa, ch_o[t]), ch_s[t]),
+                                                      __fmul_rn(__fadd_rn(qb, ch_o[t]), ch_s[t]));
+                    }
+                }
+                __builtin_amdgcn_sched_barrier(0);
+                continue;
             }
             uint32_t pr[2], lo[2], hi[2];
             f32x2_t a02[2], b02[2], a13[2], b13[2];
@@ -880,7 +930,7 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
             __builtin_amdgcn_sched_barrier(0);
         }
         __builtin_amdgcn_s_setprio(0);
-        if (h == 0) asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(2 * NI) : "memory");   // barrier kt
+        if (h == 0) asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(WAITN) : "memory");   // barrier kt
     };
     for (int kt = 0, st = 0, sl = S - 1; kt < nk; ++kt) {
         const int sn = st == S - 1 ? 0 : st + 1;
@@ -888,7 +938,7 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
         st = sn;
         sl = sl == S - 1 ? 0 : sl + 1;
     }
-    if (h == 1) asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(2 * NI) : "memory");       // barrier nk-1
+    if (h == 1) asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(WAITN) : "memory");       // barrier nk-1
     // drain this wavefront's loads (they target stages past K and are never read); the
     // accumulators were last written by MFMAs the compiler cannot see: wait out their latency
     asm volatile("s_waitcnt vmcnt(0)\n\ts_nop 15\n\ts_nop 15\n\ts_barrier" ::: "memory");
@@ -976,8 +1026,8 @@ template <int FMT, int KIND>
 struct KernelCfg {
     static constexpr bool PAIR = KIND == GK_PAIR || KIND == GK_PAIR_EXACT;
     static constexpr bool SKINNY = KIND == GK_SKINNY || KIND == GK_SKINNY_EXACT;
-    static_assert(!PAIR || FMT == MOE_FMT_INT4 || FMT == MOE_FMT_FP4_REF,
-                  "the k-split tile routine decodes int4 and the reference fp4 container");
+    static_assert(!PAIR || FMT == MOE_FMT_INT4 || FMT == MOE_FMT_FP4_REF || FMT == MOE_FMT_INT8,
+                  "the k-split tile routine decodes int4, int8 and the reference fp4 container");
     static constexpr int WAVES = PAIR ? 8 : 4;
     static constexpr int BN = GM_BN;                                             // columns per tile
     static constexpr int WG_PER_CU = SKINNY ? GM_SKINNY_WAVES : 1;
@@ -1176,7 +1226,10 @@ static int launch_gemm_fmt(const moe_grouped_args* a, hipStream_t stream) {
         // device) are HBM bound: use the small-tile kernel.  An expert with more than 32 rows then
         // costs one pass over its weights per 32 rows.
         if (a->M <= 24 * a->G) return launch_gemm_kind<FMT, GK_SKINNY>(P, a, stream);
-        return launch_gemm_kind<FMT, GK_GENERAL>(P, a, stream);
+        // int8 prefill: the k-split kernel too (its ring is one stage shorter for the 16 KB tiles, which
+        // is enough where the steps are long; at decode sizes the small-tile kernel is faster)
+        if constexpr (FMT == MOE_FMT_INT8) return launch_gemm_kind<FMT, GK_PAIR>(P, a, stream);
+        else return launch_gemm_kind<FMT, GK_GENERAL>(P, a, stream);
     }
 }
 
