@@ -46,12 +46,29 @@ __device__ __forceinline__ uint32_t e2m1_pair_scaled_bf16(uint32_t word, float s
 // the sign moved from bit 14 to bit 15 is an fp16 worth 2^-8 of the e4m3 value, subnormals
 // included (preCastFP8Weight, grouped_gemm/op_kernel/antiquant_impl.h:87-129, does the same);
 // fp16 -> fp32 is exact, so callers fold the 2^8 into their scale and round once.
-__device__ __forceinline__ f32x2_t e4m3_ref_pair_over_256(uint32_t pair) {
-    typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t e4m3_ref_pair_over_256_fp16(uint32_t pair) {
     uint32_t h = pair << 7;
     h += h & 0x40004000u;
-    const half2_t v = __builtin_bit_cast(half2_t, h);
+    return h;   // two fp16
+}
+__device__ __forceinline__ f32x2_t e4m3_ref_pair_over_256(uint32_t pair) {
+    typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+    const half2_t v = __builtin_bit_cast(half2_t, e4m3_ref_pair_over_256_fp16(pair));
     return f32x2_t{(float)v[0], (float)v[1]};
+}
+
+// fp32(low / high fp16 of h2) * s in one instruction (v_fma_mix_f32 converts the fp16 operand on the way
+// in; the product is rounded to fp32 once, exactly as a conversion followed by a multiply).  The addend
+// is -0.0 so that the sign of a zero product survives.
+__device__ __forceinline__ float fp16_lo_times(uint32_t h2, float s, float neg_zero) {
+    float r;
+    asm("v_fma_mix_f32 %0, %1, %2, %3 op_sel_hi:[1,0,0]" : "=v"(r) : "v"(h2), "v"(s), "v"(neg_zero));
+    return r;
+}
+__device__ __forceinline__ float fp16_hi_times(uint32_t h2, float s, float neg_zero) {
+    float r;
+    asm("v_fma_mix_f32 %0, %1, %2, %3 op_sel:[1,0,0] op_sel_hi:[1,0,0]" : "=v"(r) : "v"(h2), "v"(s), "v"(neg_zero));
+    return r;
 }
 
 __device__ __forceinline__ float wave_reduce_sum(float v) {

@@ -173,9 +173,11 @@ struct BTraits<MOE_FMT_FP8_REF> : BTraitsByte<MOE_FMT_FP8_REF> {
         __device__ __forceinline__ void unit(const Raw& raw, const BCtx&, int s, int p, int t, u32x4_t out[4]) {
             const uint32_t a = pinned(raw.r[s][2 * p]), b = raw.r[s][2 * p + 1];
             const uint32_t sel = (uint32_t)t | 0x0c00u | ((uint32_t)(4 + t) << 16) | 0x0c000000u;   // [a.byte t, 0, b.byte t, 0]
-            const f32x2_t v = e4m3_ref_pair_over_256(__builtin_amdgcn_perm(b, a, sel));
+            const uint32_t h2 = e4m3_ref_pair_over_256_fp16(__builtin_amdgcn_perm(b, a, sel));
             const float sc = raw.s8[s] * 256.f;
-            out[t][p] = pinned(pack_bf16_rne(v[0] * sc, v[1] * sc));
+            float nz = -0.0f;
+            asm volatile("" : "+v"(nz));   // kept in a register: not an inline constant
+            out[t][p] = pinned(pack_bf16_rne(fp16_lo_times(h2, sc, nz), fp16_hi_times(h2, sc, nz)));
         }
         // GEMV arithmetic: the codes themselves (worth 2^-8 of their value, exact in bf16); the block
         // scale is applied to the sums of each 128-k block
@@ -585,18 +587,19 @@ __device__ __forceinline__ void lds_load16(rsrc_t r, const u32x4_t* dst, int vof
 constexpr int PAIR_CAPB = 10;                         // x stages hold 160 rows
 constexpr int PAIR_MT_MAX = 10;
 constexpr int PAIR_A_UNITS = 16 * PAIR_CAPB * 8;      // 16-byte units of one x stage
-// packed tile of one k step: 64 rows of 128 bytes (4-bit codes) or of 256 bytes (int8)
+// packed tile of one k step: 64 rows of 128 bytes (4-bit codes) or of 256 bytes (int8, fp8)
 template <int FMT>
-constexpr int pair_b_units() { return FMT == MOE_FMT_INT8 ? 64 * 16 : 64 * 8; }
+constexpr int pair_b_units() { return (FMT == MOE_FMT_INT8 || FMT == MOE_FMT_FP8_REF) ? 64 * 16 : 64 * 8; }
 // ring depth: what fits into LDS next to the x stages
 template <int FMT>
-constexpr int pair_stages() { return FMT == MOE_FMT_INT8 ? 4 : 5; }
-// scale rows of 256 bf16 per k step: int4 one per 32-k sub-step (groups are multiples of 32), the
-// reference fp4 container one per 16 k
+constexpr int pair_stages() { return (FMT == MOE_FMT_INT8 || FMT == MOE_FMT_FP8_REF) ? 4 : 5; }
+// 16-byte units of scales per k step: rows of 256 bf16, int4 one per 32-k sub-step (groups are multiples
+// of 32), the reference fp4 container one per 16 k; fp8 one unit per wavefront holding the fp32 scale of
+// its 128 x 128 block; int8 none (per-channel scales stay in registers)
 template <int FMT>
-constexpr int pair_sc_rows() { return FMT == MOE_FMT_FP4_REF ? 4 : FMT == MOE_FMT_INT8 ? 0 : 2; }
+constexpr int pair_sc_units() { return FMT == MOE_FMT_FP4_REF ? 128 : FMT == MOE_FMT_INT4 ? 64 : FMT == MOE_FMT_FP8_REF ? 8 : 0; }
 template <int FMT>
-constexpr int pair_lds_units() { return pair_stages<FMT>() * (PAIR_A_UNITS + pair_b_units<FMT>() + 32 * pair_sc_rows<FMT>()); }
+constexpr int pair_lds_units() { return pair_stages<FMT>() * (PAIR_A_UNITS + pair_b_units<FMT>() + pair_sc_units<FMT>()); }
 
 // EXACT selects the arithmetic of the GEMV op (grouped_soft_gemv/op_kernel/gemv_impl.h:147-199: the
 // dequantized weights stay fp32): the B fragments then hold the codes themselves, which are exact in
@@ -606,11 +609,12 @@ constexpr int pair_lds_units() { return pair_stages<FMT>() * (PAIR_A_UNITS + pai
 // own MFMA.  These MFMAs are compiler-visible builtins (their results feed ordinary VALU code).
 template <int FMT, int MT, bool EXACT = false>
 __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* smem, int g, int64_t row0, int rows, int n0) {
-    static_assert(FMT == MOE_FMT_INT4 || FMT == MOE_FMT_FP4_REF || FMT == MOE_FMT_INT8,
-                  "the k-split tile routine decodes int4, int8 and the reference fp4 container");
-    static_assert(!EXACT || FMT != MOE_FMT_INT8, "the GEMV op has no int8 container");
-    constexpr bool FP4 = FMT == MOE_FMT_FP4_REF, I8 = FMT == MOE_FMT_INT8;
-    constexpr int BK = 64, S = pair_stages<FMT>(), SC_ROWS = pair_sc_rows<FMT>(), PAIR_SC_UNITS = 32 * SC_ROWS;
+    static_assert(FMT == MOE_FMT_INT4 || FMT == MOE_FMT_FP4_REF || FMT == MOE_FMT_INT8 || FMT == MOE_FMT_FP8_REF,
+                  "the k-split tile routine decodes int4, int8 and the reference fp4 / fp8 containers");
+    static_assert(!EXACT || FMT == MOE_FMT_INT4 || FMT == MOE_FMT_FP4_REF, "un-rounded weights: int4 and reference fp4 only");
+    constexpr bool FP4 = FMT == MOE_FMT_FP4_REF, I8 = FMT == MOE_FMT_INT8, F8 = FMT == MOE_FMT_FP8_REF;
+    constexpr bool B8 = I8 || F8;   // one byte per weight: tiles of 64 rows x 256 bytes
+    constexpr int BK = 64, S = pair_stages<FMT>(), PAIR_SC_UNITS = pair_sc_units<FMT>();
     constexpr int PAIR_B_UNITS = pair_b_units<FMT>();
     constexpr int AHEAD = S - 1;   // a step's loads fill the stage of step kt + AHEAD
     u32x4_t* lds_a = smem;
@@ -626,14 +630,18 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
     // the role whose barrier sits inside the decode phase
     const int h = 1 - (wv >> 2);
     // this lane's 4 columns (MFMA t = column col0 + t): half of a dword of 8 4-bit codes, or a dword of 4 bytes
-    const int col0 = I8 ? 64 * cw + 4 * i : 128 * (cw >> 1) + 8 * i + 4 * (cw & 1);
+    const int col0 = B8 ? 64 * cw + 4 * i : 128 * (cw >> 1) + 8 * i + 4 * (cw & 1);
     const int nk = P.K / BK;
 
     const int64_t KN = (int64_t)P.K * P.N;
-    const rsrc_t rw = I8 ? make_rsrc(P.w + g * KN, KN) : make_rsrc(P.w + g * (KN >> 1), KN >> 1);
+    const rsrc_t rw = B8 ? make_rsrc(P.w + g * KN, KN) : make_rsrc(P.w + g * (KN >> 1), KN >> 1);
     const rsrc_t rs = make_rsrc(static_cast<const uint16_t*>(P.scale) + (int64_t)g * P.scale_rows * P.N,
                                 (int64_t)P.scale_rows * P.N * 2);
-    const uint32_t per = I8 ? 1u : (uint32_t)((P.K / P.scale_rows) >> 5);      // 32-k sub-steps per scale group
+    // fp8: the expert's fp32 block scales [K/128, N/128]; this wavefront's 128-column block
+    const rsrc_t rs8 = make_rsrc(static_cast<const float*>(P.scale) + (int64_t)g * (P.K >> 7) * (P.N >> 7),
+                                 (int64_t)(P.K >> 7) * (P.N >> 7) * 4);
+    const int cs8 = ((n0 + 64 * cw) >> 7) * 4;
+    const uint32_t per = B8 ? 1u : (uint32_t)((P.K / P.scale_rows) >> 5);      // 32-k sub-steps per scale group
     const uint32_t gmul = per == 1 ? 0u : 0xffffffffu / per + 1u;   // sub-step -> scale row as a multiply
     auto scale_row = [&](uint32_t sub) { return gmul ? (int)__umulhi(sub, gmul) : (int)sub; };
     // x rows through a buffer resource that ends after the last valid row (padded rows read as
@@ -644,14 +652,14 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
     // packed tile: instruction wv brings rows 8 wv + (lane >> 3) into the 1 KB block wv of the stage;
     // the two 64-byte halves of the rows with odd (row >> 3) are swapped, so that the four q groups
     // of a wavefront read from both halves of the banks
-    // int8 (rows of 256 bytes): instruction e of wavefront wv brings rows 8 wv + 4 e + (lane >> 4); the
+    // int8 / fp8 (rows of 256 bytes): instruction e of wavefront wv brings rows 8 wv + 4 e + (lane >> 4); the
     // 64-byte quarters of a row are permuted by (row >> 3) & 3 = wv & 3, so that the four q groups read
     // from different quarters of the banks
-    const int vb = I8 ? (lane >> 4) * P.N + (((lane & 15) ^ (4 * (wv & 3))) * 16)
+    const int vb = B8 ? (lane >> 4) * P.N + (((lane & 15) ^ (4 * (wv & 3))) * 16)
                       : (lane >> 3) * (P.N >> 1) + (((lane & 7) ^ (4 * (wv & 1))) * 16);
     constexpr int NA = (2 * MT + 7) / 8;   // x load instructions per wavefront per step
-    constexpr int NB = I8 ? 2 : 1;         // packed-tile instructions
-    constexpr int NI = NA + NB + (SC_ROWS ? 1 : 0);   // + an eighth of the step's scales
+    constexpr int NB = B8 ? 2 : 1;         // packed-tile instructions
+    constexpr int NI = NA + NB + (PAIR_SC_UNITS ? 1 : 0);   // + an eighth of the step's scales
     int ja[NA], ca[NA];
 #pragma unroll
     for (int m = 0; m < NA; ++m) {
@@ -660,8 +668,8 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
         ja[m] = j * 64;
         ca[m] = 8 * j * P.K * 2;
     }
-    const int cb = I8 ? 8 * wv * P.N + n0 : 8 * wv * (P.N >> 1) + (n0 >> 1);
-    const int kb_step = I8 ? BK * P.N : BK * (P.N >> 1);
+    const int cb = B8 ? 8 * wv * P.N + n0 : 8 * wv * (P.N >> 1) + (n0 >> 1);
+    const int kb_step = B8 ? BK * P.N : BK * (P.N >> 1);
     // scales of a step: int4 2 rows of 512 bytes, 128 bytes (8 lanes) per wavefront: bytes [128 (wv & 3), +128) of
     // row wv >> 2; fp4 4 rows (one per 16 k), 256 bytes (16 lanes) per wavefront: bytes [256 (wv & 1), +256) of row wv >> 1
     const int cs = FP4 ? n0 * 2 + (wv & 1) * 256 : n0 * 2 + (wv & 3) * 128;
@@ -674,7 +682,12 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
         } else if (m < NA + NB) {
             const int e = m - NA;
             lds_load16(rw, lds_b + ST * PAIR_B_UNITS + wv * (PAIR_B_UNITS / 8) + e * 64, vb,
-                       cb + (I8 ? 4 * e * P.N : 0) + (kt + AHEAD) * kb_step);
+                       cb + (B8 ? 4 * e * P.N : 0) + (kt + AHEAD) * kb_step);
+        } else if constexpr (F8) {
+            // the block scale of the stage's 128-k block, 4 bytes by lane 0 (past K: reads as 0, unused)
+            if (lane == 0)
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rs8, MOE_LDS_PTR(lds_s + ST * PAIR_SC_UNITS + wv), 4, 0,
+                                                         ((kt + AHEAD) >> 1) * (P.N >> 7) * 4 + cs8, 0, 0);
         } else {
             const int grow = FP4 ? (kt + AHEAD) * 4 + (wv >> 1) : scale_row((uint32_t)((kt + AHEAD) * 2 + (wv >> 2)));
             if (s_lane) lds_load16(rs, lds_s + ST * PAIR_SC_UNITS + wv * (PAIR_SC_UNITS / 8), lane16, grow * (P.N * 2) + cs);
@@ -752,12 +765,13 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
             } else {
                 sc = *reinterpret_cast<const u32x2_t*>(sc16 + 256 * (2 * h + (q >> 1)) + col0);
             }
-        } else if constexpr (I8) {
+        } else if constexpr (B8) {
             // dword 16 cw + i of each of this lane's 8 k rows; the quarter of the row it lies in is
             // permuted by (row >> 3) & 3 = q (see vb)
             const uint32_t* t32 = reinterpret_cast<const uint32_t*>(lds_b + st * PAIR_B_UNITS);
 #pragma unroll
             for (int j = 0; j < 8; ++j) r[j] = t32[(32 * h + 8 * q + j) * 64 + 16 * (cw ^ q) + i];
+            if constexpr (F8) sc[0] = *reinterpret_cast<const uint32_t*>(lds_s + st * PAIR_SC_UNITS + wv);
         } else {
             const uint32_t* t32 = reinterpret_cast<const uint32_t*>(lds_b + st * PAIR_B_UNITS);
 #pragma unroll
@@ -802,6 +816,25 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
                 // first x fragments of the MFMA phase, read under the rest of the decode
 #pragma unroll
                 for (int f = 0; f < R; ++f) afr[f & 3] = la[a_lds_unit<BK>(16 * f + i, 4 * h + q)];
+            }
+            if constexpr (F8) {
+                // byte t of the dwords of k rows 2p, 2p+1, decoded as a pair through fp16 (see
+                // e4m3_ref_pair_over_256); the 2^8 goes into the block scale
+                const float scl = __uint_as_float(sc[0]) * 256.f;
+                float nz = -0.0f;
+                asm volatile("" : "+v"(nz));   // kept in a register: not an inline constant
+#pragma unroll
+                for (int p = 0; p < 2; ++p) {
+                    const uint32_t a = r[2 * (p0 + p)], b = r[2 * (p0 + p) + 1];
+#pragma unroll
+                    for (int t = 0; t < 4; ++t) {
+                        const uint32_t sel8 = (uint32_t)t | 0x0c00u | ((uint32_t)(4 + t) << 16) | 0x0c000000u;   // [a.byte t, 0, b.byte t, 0]
+                        const uint32_t h2 = e4m3_ref_pair_over_256_fp16(__builtin_amdgcn_perm(b, a, sel8));
+                        bf[t][p0 + p] = pack_bf16_rne(fp16_lo_times(h2, scl, nz), fp16_hi_times(h2, scl, nz));
+                    }
+                }
+                __builtin_amdgcn_sched_barrier(0);
+                continue;
             }
             if constexpr (I8) {
                 // byte t of the dwords of k rows 2p, 2p+1 -> (q + offset) * scale as two rounded fp32
@@ -1026,8 +1059,8 @@ template <int FMT, int KIND>
 struct KernelCfg {
     static constexpr bool PAIR = KIND == GK_PAIR || KIND == GK_PAIR_EXACT;
     static constexpr bool SKINNY = KIND == GK_SKINNY || KIND == GK_SKINNY_EXACT;
-    static_assert(!PAIR || FMT == MOE_FMT_INT4 || FMT == MOE_FMT_FP4_REF || FMT == MOE_FMT_INT8,
-                  "the k-split tile routine decodes int4, int8 and the reference fp4 container");
+    static_assert(!PAIR || FMT == MOE_FMT_INT4 || FMT == MOE_FMT_FP4_REF || FMT == MOE_FMT_INT8 || FMT == MOE_FMT_FP8_REF,
+                  "the k-split tile routine decodes int4, int8 and the reference fp4 / fp8 containers");
     static constexpr int WAVES = PAIR ? 8 : 4;
     static constexpr int BN = GM_BN;                                             // columns per tile
     static constexpr int WG_PER_CU = SKINNY ? GM_SKINNY_WAVES : 1;
@@ -1226,9 +1259,9 @@ static int launch_gemm_fmt(const moe_grouped_args* a, hipStream_t stream) {
         // device) are HBM bound: use the small-tile kernel.  An expert with more than 32 rows then
         // costs one pass over its weights per 32 rows.
         if (a->M <= 24 * a->G) return launch_gemm_kind<FMT, GK_SKINNY>(P, a, stream);
-        // int8 prefill: the k-split kernel too (its ring is one stage shorter for the 16 KB tiles, which
+        // int8 / fp8 prefill: the k-split kernel too (its ring is one stage shorter for the 16 KB tiles, which
         // is enough where the steps are long; at decode sizes the small-tile kernel is faster)
-        if constexpr (FMT == MOE_FMT_INT8) return launch_gemm_kind<FMT, GK_PAIR>(P, a, stream);
+        if constexpr (FMT == MOE_FMT_INT8 || FMT == MOE_FMT_FP8_REF) return launch_gemm_kind<FMT, GK_PAIR>(P, a, stream);
         else return launch_gemm_kind<FMT, GK_GENERAL>(P, a, stream);
     }
 }
