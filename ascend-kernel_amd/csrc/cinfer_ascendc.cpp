@@ -6,8 +6,8 @@
 // Differences from the reference adapters (grouped_gemm/src/grouped_gemm.cpp:122-161,
 // grouped_soft_gemv/src/grouped_soft_gemv.cpp:123-155): shapes, dtypes, devices and
 // contiguity are validated before the launch; no workspace is allocated or cached;
-// computeType accepts "int8", "int4", "fp4_b32" and "bf16" besides "fp4" and "fp8";
-// dequant_fp4 is an extra entry point.  Every failure raises RuntimeError, as the
+// computeType accepts "int8", "int4", "fp4_b32", "fp4_b16" and "bf16" besides "fp4" and "fp8";
+// dequant_fp4, the fp4 weight preparation, routing and the fused-SwiGLU GEMM are extra entry points.  Every failure raises RuntimeError, as the
 // reference does.
 #include <c10/core/DeviceGuard.h>
 #include <c10/hip/HIPStream.h>
@@ -42,7 +42,7 @@ int parse_format(const char* computeType) {
     const int fmt = moe_format_from_compute_type(computeType);
     if (fmt < 0)
         fail(std::string("Invalid compute type: ") + (computeType ? computeType : "(null)") +
-             ". Supported: \"fp4\", \"fp8\", \"int8\", \"int4\", \"fp4_b32\", \"bf16\"");
+             ". Supported: \"fp4\", \"fp8\", \"int8\", \"int4\", \"fp4_b32\", \"fp4_b16\", \"bf16\"");
     return fmt;
 }
 
