@@ -14,8 +14,9 @@
 // L2.  A workgroup has 4 wavefronts; every wavefront owns 64 of the 256 columns for
 // ALL rows of the tile, so each weight element is dequantized exactly once per tile.
 // x tiles go through a double-buffered, XOR-swizzled LDS tile shared by the 4 waves.
-// (The int4 container and the reference's pre-shuffled fp4 container use a tile routine with 8
-// wavefronts and LDS-direct loads instead, see gemm_tile_pair.)
+// (That is gemm_tile, used by the K-contiguous containers.  The N-contiguous ones -- int4, int8 and
+// the reference's fp4 and fp8 containers -- use a tile routine with 8 wavefronts and LDS-direct loads
+// instead, see gemm_tile_pair.)
 //
 // MFMA: v_mfma_f32_16x16x32_bf16.  Lane l = 16*q + i holds, for A, row i and
 // k = 8q..8q+7 of the 16x32 block; for B, column i and the same k; for the result,
@@ -98,9 +99,6 @@ __device__ __forceinline__ V pinned(V v) {
 struct BCtx {
     rsrc_t rw, rs;       // weight / scale slab of the expert
     int vw, vs;          // per-lane byte offsets into them (constant over the tile)
-    const uint16_t* sg;  // int8: scale / offset rows of the expert
-    const uint16_t* og;
-    const float* s8;     // fp8: scale blocks of the expert
     int K, N, n0;
     int i, q, w;         // lane & 15, lane >> 4, wavefront (scalar)
 };
@@ -115,80 +113,6 @@ struct BCtx {
 //   col        output column (relative to n0) of MFMA t in this lane
 template <int FMT>
 struct BTraits;
-
-// ------------------------------------------------------- int8 / reference fp8, [K, N]
-// Lane (i, q) loads the dword with columns 64w + 4i + [0,4) of each of its 8 k rows.
-template <int FMT>
-struct BTraitsByte {
-    static constexpr int BK = 64, NS = 2;
-    static constexpr bool DOUBLE_RAW = false;
-    static constexpr int MT_MAX = 11;
-    struct Raw {
-        uint32_t r[2][8];
-        float s8[2];  // fp8: scale of the 128x128 block of each sub-step
-    };
-    __device__ static __forceinline__ int a_chunk(int s, int q) { return 4 * s + q; }
-    __device__ static __forceinline__ int col(const BCtx& c, int t) { return 64 * c.w + 4 * c.i + t; }
-    __device__ static __forceinline__ void init(BCtx& c) {
-        c.vw = 8 * c.q * c.N + col(c, 0);
-        c.vs = 0;
-    }
-    __device__ static __forceinline__ void load_sub(Raw& raw, const BCtx& c, int k0, int s) {
-#pragma unroll
-        for (int j = 0; j < 8; ++j) raw.r[s][j] = ldg_b32(c.rw, c.vw, (k0 + 32 * s + j) * c.N + c.n0);
-        if (FMT == MOE_FMT_FP8_REF) {
-            // the prefetch may point past K: clamp the block row (value unused then)
-            const int kb = min(k0 >> 7, (c.K >> 7) - 1);
-            raw.s8[s] = c.s8[kb * (c.N >> 7) + ((c.n0 + 64 * c.w) >> 7)];
-        }
-    }
-};
-
-template <>
-struct BTraits<MOE_FMT_INT8> : BTraitsByte<MOE_FMT_INT8> {
-    struct Dq {
-        float sc[4], of[4];  // per-channel scale and offset of this lane's 4 columns, fixed for the tile
-        __device__ __forceinline__ void init_tile(const BCtx& c) {
-            const u32x2_t s = *reinterpret_cast<const u32x2_t*>(c.sg + c.n0 + col(c, 0));
-            const u32x2_t o = *reinterpret_cast<const u32x2_t*>(c.og + c.n0 + col(c, 0));
-            sc[0] = bf16_lo(s[0]); sc[1] = bf16_hi(s[0]); sc[2] = bf16_lo(s[1]); sc[3] = bf16_hi(s[1]);
-            of[0] = bf16_lo(o[0]); of[1] = bf16_hi(o[0]); of[2] = bf16_lo(o[1]); of[3] = bf16_hi(o[1]);
-        }
-        __device__ __forceinline__ void prep(const Raw&, const BCtx&, int) {}
-        __device__ __forceinline__ void unit(const Raw& raw, const BCtx&, int s, int p, int t, u32x4_t out[4]) {
-            const uint32_t a = pinned(raw.r[s][2 * p]), b = raw.r[s][2 * p + 1];
-            const float qa = (float)(int)(int8_t)(a >> (8 * t)), qb = (float)(int)(int8_t)(b >> (8 * t));
-            // (q + offset) * scale as two rounded fp32 operations
-            out[t][p] = pinned(pack_bf16_rne(__fmul_rn(__fadd_rn(qa, of[t]), sc[t]), __fmul_rn(__fadd_rn(qb, of[t]), sc[t])));
-        }
-    };
-};
-
-template <>
-struct BTraits<MOE_FMT_FP8_REF> : BTraitsByte<MOE_FMT_FP8_REF> {
-    struct Dq {
-        __device__ __forceinline__ void init_tile(const BCtx&) {}
-        __device__ __forceinline__ void prep(const Raw&, const BCtx&, int) {}
-        // both k rows of a pair at once (see e4m3_ref_pair_over_256): the 2^8 goes into the block scale
-        __device__ __forceinline__ void unit(const Raw& raw, const BCtx&, int s, int p, int t, u32x4_t out[4]) {
-            const uint32_t a = pinned(raw.r[s][2 * p]), b = raw.r[s][2 * p + 1];
-            const uint32_t sel = (uint32_t)t | 0x0c00u | ((uint32_t)(4 + t) << 16) | 0x0c000000u;   // [a.byte t, 0, b.byte t, 0]
-            const uint32_t h2 = e4m3_ref_pair_over_256_fp16(__builtin_amdgcn_perm(b, a, sel));
-            const float sc = raw.s8[s] * 256.f;
-            float nz = -0.0f;
-            asm volatile("" : "+v"(nz));   // kept in a register: not an inline constant
-            out[t][p] = pinned(pack_bf16_rne(fp16_lo_times(h2, sc, nz), fp16_hi_times(h2, sc, nz)));
-        }
-        // GEMV arithmetic: the codes themselves (worth 2^-8 of their value, exact in bf16); the block
-        // scale is applied to the sums of each 128-k block
-        __device__ __forceinline__ void unit_exact(const Raw& raw, const BCtx&, int s, int p, int t, u32x4_t out[4]) {
-            const uint32_t a = pinned(raw.r[s][2 * p]), b = raw.r[s][2 * p + 1];
-            const uint32_t sel = (uint32_t)t | 0x0c00u | ((uint32_t)(4 + t) << 16) | 0x0c000000u;
-            const f32x2_t v = e4m3_ref_pair_over_256(__builtin_amdgcn_perm(b, a, sel));
-            out[t][p] = pinned(pack_bf16_rne(v[0], v[1]));
-        }
-    };
-};
 
 // ------------------------------------------- fp4 block-32 / block-16, [N, K/2]
 // K-contiguous: MFMA t, lane (i, q) owns column 64w + 16t + i and loads the 16 bytes
@@ -290,20 +214,8 @@ __device__ __forceinline__ void make_ctx(BCtx& c, const GemmParams& P, int g, in
     const int tid = threadIdx.x, lane = tid & 63;
     c.K = P.K; c.N = P.N; c.n0 = n0;
     c.i = lane & 15; c.q = lane >> 4; c.w = __builtin_amdgcn_readfirstlane(tid >> 6);
-    c.sg = nullptr; c.og = nullptr; c.s8 = nullptr;
     const int64_t KN = (int64_t)P.K * P.N;
     switch (FMT) {
-        case MOE_FMT_INT8:
-            c.rw = make_rsrc(P.w + g * KN, KN);
-            c.rs = c.rw;
-            c.sg = static_cast<const uint16_t*>(P.scale) + (int64_t)g * P.N;
-            c.og = P.offset + (int64_t)g * P.N;
-            break;
-        case MOE_FMT_FP8_REF:
-            c.rw = make_rsrc(P.w + g * KN, KN);
-            c.rs = c.rw;
-            c.s8 = static_cast<const float*>(P.scale) + (int64_t)g * (P.K >> 7) * (P.N >> 7);
-            break;
         case MOE_FMT_FP4_B32:
             c.rw = make_rsrc(P.w + g * (KN >> 1), KN >> 1);
             c.rs = make_rsrc(static_cast<const uint16_t*>(P.scale) + g * (KN >> 5), KN >> 4);
@@ -324,23 +236,9 @@ template <int FMT, int MT>
 __device__ __forceinline__ void store_tile(const GemmParams& P, const BCtx& c, f32x4_t (&acc)[MT][4], int64_t row0, int rows,
                                            int n0) {
     using T = BTraits<FMT>;
-    constexpr bool N_CONTIG = FMT == MOE_FMT_INT8 || FMT == MOE_FMT_FP8_REF;
     // through a buffer resource that ends after the tile's last valid row: stores to padded
-    // rows fall outside it and are dropped
-    if (N_CONTIG && P.epilogue == MOE_EPILOGUE_SWIGLU) {
-        // this lane's 4 columns are (gate, gate, up, up) of 2 output columns; y has N / 2 columns
-        const int NO = P.N >> 1;
-        const rsrc_t ro = make_rsrc(P.y + row0 * (int64_t)NO, (int64_t)rows * NO * 2);
-        const int vo = (4 * c.q * NO + ((n0 + T::col(c, 0)) >> 1)) * 2;
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-            for (int r = 0; r < 4; ++r)
-                __builtin_amdgcn_raw_buffer_store_b32(
-                    pack_bf16_rne(swiglu(acc[mt][0][r], acc[mt][2][r]), swiglu(acc[mt][1][r], acc[mt][3][r])), ro, vo,
-                    (16 * mt + r) * NO * 2, 0);
-        return;
-    }
+    // rows fall outside it and are dropped (the containers of this routine are K-contiguous: a lane's
+    // 4 accumulators of a row are 16 columns apart)
     const rsrc_t ry = make_rsrc(P.y + row0 * (int64_t)P.N, (int64_t)rows * P.N * 2);
     const int vy = (4 * c.q * P.N + n0) * 2;
 #pragma unroll
@@ -348,27 +246,15 @@ __device__ __forceinline__ void store_tile(const GemmParams& P, const BCtx& c, f
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
             const int so = (16 * mt + r) * P.N * 2;
-            if (N_CONTIG) {
-                u32x2_t v;
-                v[0] = pack_bf16_rne(acc[mt][0][r], acc[mt][1][r]);
-                v[1] = pack_bf16_rne(acc[mt][2][r], acc[mt][3][r]);
-                __builtin_amdgcn_raw_buffer_store_b64(v, ry, vy + T::col(c, 0) * 2, so, 0);
-            } else {
 #pragma unroll
-                for (int t = 0; t < 4; ++t)
-                    __builtin_amdgcn_raw_buffer_store_b16((uint16_t)(pack_bf16_rne(acc[mt][t][r], 0.f) & 0xffffu), ry,
-                                                          vy + T::col(c, t) * 2, so, 0);
-            }
+            for (int t = 0; t < 4; ++t)
+                __builtin_amdgcn_raw_buffer_store_b16((uint16_t)(pack_bf16_rne(acc[mt][t][r], 0.f) & 0xffffu), ry,
+                                                      vy + T::col(c, t) * 2, so, 0);
         }
 }
 
-// EXACT (reference fp8 container only) selects the arithmetic of the GEMV op, whose dequantized weights
-// stay fp32 (grouped_soft_gemv/op_kernel/gemv_impl.h:147-199): the B fragments hold the e4m3 values
-// themselves (exact in bf16), the sums of every 128-k scale block are kept apart and multiplied by the
-// block's fp32 scale when the block ends.  Its MFMAs are compiler builtins (their results feed VALU code).
-template <int FMT, int MT, int CAPB, bool EXACT = false>
+template <int FMT, int MT, int CAPB>
 __device__ __forceinline__ void gemm_tile(const GemmParams& P, u32x4_t* lds_a, int g, int64_t row0, int rows, int n0) {
-    static_assert(!EXACT || FMT == MOE_FMT_FP8_REF, "un-rounded weights: reference fp8 container only");
     using T = BTraits<FMT>;
     constexpr int BK = T::BK, NS = T::NS;
     constexpr int CPR = BK / 8;               // 16-byte chunks per tile row
@@ -394,13 +280,6 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& P, u32x4_t* lds_a, i
     for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
         for (int t = 0; t < 4; ++t) acc[mt][t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-    // EXACT: sums of the current 128-k scale block and that block's scale (times the 2^8 the decode leaves out)
-    f32x4_t part[EXACT ? MT : 1][4];
-    float sblk = 0.f;
-#pragma unroll
-    for (int mt = 0; mt < (EXACT ? MT : 1); ++mt)
-#pragma unroll
-        for (int t = 0; t < 4; ++t) part[mt][t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
     u32x4_t areg[PASSES];
     typename T::Raw raw, raw_next;
@@ -445,10 +324,7 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& P, u32x4_t* lds_a, i
 #pragma unroll
     for (int p = 0; p < 4; ++p)
 #pragma unroll
-        for (int t = 0; t < 4; ++t) {
-            if constexpr (EXACT) dq.unit_exact(raw, c, 0, p, t, bf[0]);
-            else dq.unit(raw, c, 0, p, t, bf[0]);
-        }
+        for (int t = 0; t < 4; ++t) dq.unit(raw, c, 0, p, t, bf[0]);
     __syncthreads();
     // raw[0] <- sub-step 0 of step 1, a full step ahead
     if (T::DOUBLE_RAW)
@@ -464,8 +340,6 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& P, u32x4_t* lds_a, i
     auto step = [&](int kt) {
         const u32x4_t* la = lds_a + (kt & 1) * ABUF;
         u32x4_t afr[4];
-        if constexpr (EXACT)
-            if ((kt & 1) == 0) sblk = c.s8[(kt >> 1) * (c.N >> 7) + ((c.n0 + 64 * c.w) >> 7)] * 256.f;
         auto read_a = [&](int f) {
             afr[f & 3] = la[a_lds_unit<BK>(16 * (f % MT) + c.i, T::a_chunk(f / MT, c.q))];
         };
@@ -482,11 +356,7 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& P, u32x4_t* lds_a, i
             for (int slot = 0; slot < SLOTS; ++slot) {
                 const int mt = slot >> 2, t = slot & 3, f = s * MT + mt;
                 if (t == 0 && f + RING < F) read_a(f + RING);
-                if constexpr (EXACT)
-                    part[mt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, afr[f & 3]),
-                                                                          __builtin_bit_cast(bf16x8_t, bcur[t]), part[mt][t], 0, 0, 0);
-                else
-                    mfma_16x16x32(acc[mt][t], afr[f & 3], bcur[t]);
+                mfma_16x16x32(acc[mt][t], afr[f & 3], bcur[t]);
                 // fetch the x tile of step kt+1
                 if (s == 0 && slot < PASSES) areg[slot] = ldg_b128(rx, vx, (slot * RPP * P.K + (kt + 1) * BK) * 2);
                 // decode units u with floor(u * SLOTS / UNITS) == slot
@@ -494,8 +364,6 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& P, u32x4_t* lds_a, i
                 for (int u = (slot * UNITS + SLOTS - 1) / SLOTS; u < ((slot + 1) * UNITS + SLOTS - 1) / SLOTS; ++u) {
                     if (u == 0)
                         dq.prep(raw, c, sn);
-                    else if constexpr (EXACT)
-                        dq.unit_exact(raw, c, sn, (u - 1) >> 2, (u - 1) & 3, bnxt);
                     else
                         dq.unit(raw, c, sn, (u - 1) >> 2, (u - 1) & 3, bnxt);
                 }
@@ -512,18 +380,6 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& P, u32x4_t* lds_a, i
                     lds_a[((kt + 1) & 1) * ABUF + a_lds_unit<BK>(ar + RPP * wi, ac)] = areg[wi];
                 }
                 __builtin_amdgcn_sched_barrier(0);
-            }
-        }
-        if constexpr (EXACT) {
-            if (kt & 1) {   // a 128-k scale block ends with every second 64-k step
-#pragma unroll
-                for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-                    for (int t = 0; t < 4; ++t) {
-#pragma unroll
-                        for (int e = 0; e < 4; ++e) acc[mt][t][e] = fmaf(part[mt][t][e], sblk, acc[mt][t][e]);
-                        part[mt][t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-                    }
             }
         }
         __syncthreads();
@@ -547,7 +403,8 @@ __device__ __forceinline__ void lds_load16(rsrc_t r, const u32x4_t* dst, int vof
 }
 
 // ---------------------------------------------------------------------------------
-// Tile routine for int4 and the reference fp4 container with two wavefronts per SIMD that split the k range.
+// Tile routine for the N-contiguous containers (int4, int8, reference fp4 / fp8) with two wavefronts per
+// SIMD that split the k range.
 //
 // A single wavefront issues at most one instruction every ~5 cycles whatever its kind, and an
 // MFMA holds the SIMD's vector issue port for about 8 of its 16 cycles: with one wavefront
@@ -611,7 +468,7 @@ template <int FMT, int MT, bool EXACT = false>
 __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* smem, int g, int64_t row0, int rows, int n0) {
     static_assert(FMT == MOE_FMT_INT4 || FMT == MOE_FMT_FP4_REF || FMT == MOE_FMT_INT8 || FMT == MOE_FMT_FP8_REF,
                   "the k-split tile routine decodes int4, int8 and the reference fp4 / fp8 containers");
-    static_assert(!EXACT || FMT == MOE_FMT_INT4 || FMT == MOE_FMT_FP4_REF, "un-rounded weights: int4 and reference fp4 only");
+    static_assert(!EXACT || FMT != MOE_FMT_INT8, "the GEMV op has no int8 container");
     constexpr bool FP4 = FMT == MOE_FMT_FP4_REF, I8 = FMT == MOE_FMT_INT8, F8 = FMT == MOE_FMT_FP8_REF;
     constexpr bool B8 = I8 || F8;   // one byte per weight: tiles of 64 rows x 256 bytes
     constexpr int BK = 64, S = pair_stages<FMT>(), PAIR_SC_UNITS = pair_sc_units<FMT>();
@@ -789,7 +646,8 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
         float m[4], z[4];
         const float s0 = bf16_lo(sc[0]), s1 = bf16_hi(sc[0]), s2 = bf16_lo(sc[1]), s3 = bf16_hi(sc[1]);
         // with EXACT: the scales of the step being multiplied (sc is refilled during the MFMA phase)
-        const float sa[4] = {s0, s1, s2, s3};
+        const float f8s = __uint_as_float(sc[0]) * 256.f;   // fp8: the step's block scale (times the 2^8 the decode leaves out)
+        const float sa[4] = {F8 ? f8s : s0, F8 ? f8s : s1, F8 ? f8s : s2, F8 ? f8s : s3};
         const float sb[4] = {bf16_lo(sc2[0]), bf16_hi(sc2[0]), bf16_lo(sc2[1]), bf16_hi(sc2[1])};
         if constexpr (EXACT) {
             m[0] = m[1] = m[2] = m[3] = FP4 ? 1.f : 512.f;
@@ -830,7 +688,14 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
                     for (int t = 0; t < 4; ++t) {
                         const uint32_t sel8 = (uint32_t)t | 0x0c00u | ((uint32_t)(4 + t) << 16) | 0x0c000000u;   // [a.byte t, 0, b.byte t, 0]
                         const uint32_t h2 = e4m3_ref_pair_over_256_fp16(__builtin_amdgcn_perm(b, a, sel8));
-                        bf[t][p0 + p] = pack_bf16_rne(fp16_lo_times(h2, scl, nz), fp16_hi_times(h2, scl, nz));
+                        if constexpr (EXACT) {
+                            // the e4m3 values themselves (worth 2^-8): exact in bf16
+                            typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+                            const half2_t hv = __builtin_bit_cast(half2_t, h2);
+                            bf[t][p0 + p] = pack_bf16_rne((float)hv[0], (float)hv[1]);
+                        } else {
+                            bf[t][p0 + p] = pack_bf16_rne(fp16_lo_times(h2, scl, nz), fp16_hi_times(h2, scl, nz));
+                        }
                     }
                 }
                 __builtin_amdgcn_sched_barrier(0);
@@ -1049,16 +914,15 @@ __device__ __forceinline__ void expert_chunks(int m, int& chunks, int& bpc) {
 //   GK_GENERAL  4 wavefronts of 64 columns, one workgroup per CU, tiles of up to 192 rows
 //   GK_SKINNY   the same tile routine with tiles of at most 32 rows and several workgroups per CU
 //               (decode-sized batches are HBM bound: more weight bytes in flight)
-//   GK_PAIR     int4 / reference fp4: 8 wavefronts, k range split between the two wavefronts of a SIMD
+//   GK_PAIR     N-contiguous containers: 8 wavefronts, k range split between the two wavefronts of a SIMD
 //   GK_PAIR_EXACT  GK_PAIR with the GEMV op's arithmetic (weights not rounded to bf16), tiles of at most 32 rows
-//   GK_SKINNY_EXACT  GK_SKINNY with the GEMV op's arithmetic (reference fp8 container)
-enum { GK_GENERAL = 0, GK_SKINNY = 1, GK_PAIR = 2, GK_PAIR_EXACT = 3, GK_SKINNY_EXACT = 4 };
+enum { GK_GENERAL = 0, GK_SKINNY = 1, GK_PAIR = 2, GK_PAIR_EXACT = 3 };
 constexpr int PAIR_EXACT_MT_MAX = 2;
 
 template <int FMT, int KIND>
 struct KernelCfg {
     static constexpr bool PAIR = KIND == GK_PAIR || KIND == GK_PAIR_EXACT;
-    static constexpr bool SKINNY = KIND == GK_SKINNY || KIND == GK_SKINNY_EXACT;
+    static constexpr bool SKINNY = KIND == GK_SKINNY;
     static_assert(!PAIR || FMT == MOE_FMT_INT4 || FMT == MOE_FMT_FP4_REF || FMT == MOE_FMT_INT8 || FMT == MOE_FMT_FP8_REF,
                   "the k-split tile routine decodes int4, int8 and the reference fp4 / fp8 containers");
     static constexpr int WAVES = PAIR ? 8 : 4;
@@ -1087,7 +951,7 @@ __device__ __forceinline__ void run_tile(const GemmParams& P, u32x4_t* smem, int
     if constexpr (C::PAIR)
         gemm_tile_pair<FMT, MT, KIND == GK_PAIR_EXACT>(P, smem, g, row0, rows, n0);
     else
-        gemm_tile<FMT, MT, C::CAPB, KIND == GK_SKINNY_EXACT>(P, smem, g, row0, rows, n0);
+        gemm_tile<FMT, MT, C::CAPB>(P, smem, g, row0, rows, n0);
 }
 
 template <int FMT, int KIND>
@@ -1249,20 +1113,17 @@ static GemmParams gemm_params(const moe_grouped_args* a) {
 template <int FMT>
 static int launch_gemm_fmt(const moe_grouped_args* a, hipStream_t stream) {
     const GemmParams P = gemm_params(a);
-    // int4 and the reference fp4 container: the k-split kernel at every batch size (measured faster than
-    // the small-tile kernel down to decode batches of 1-2 rows per expert: int4 243 vs 344 us at 128 rows
-    // over 256 experts, 7168 x 2048; fp4 476 vs 519 us at 512 rows).
-    if constexpr (FMT == MOE_FMT_INT4 || FMT == MOE_FMT_FP4_REF) {
+    // The N-contiguous containers run on the k-split kernel at every batch size: measured faster than the
+    // small-tile kernel down to decode batches of 1-2 rows per expert (256 experts of 7168 x 2048: int4
+    // 243 vs 344 us at 128 rows, fp4 476 vs 519 us and fp8 610 vs 784 us at 512 rows).
+    if constexpr (FMT == MOE_FMT_INT4 || FMT == MOE_FMT_FP4_REF || FMT == MOE_FMT_FP8_REF || FMT == MOE_FMT_INT8) {
         return launch_gemm_kind<FMT, GK_PAIR>(P, a, stream);
     } else {
         // Decode-like batches (on average at most 24 rows per expert; group_list itself stays on the
         // device) are HBM bound: use the small-tile kernel.  An expert with more than 32 rows then
         // costs one pass over its weights per 32 rows.
         if (a->M <= 24 * a->G) return launch_gemm_kind<FMT, GK_SKINNY>(P, a, stream);
-        // int8 / fp8 prefill: the k-split kernel too (its ring is one stage shorter for the 16 KB tiles, which
-        // is enough where the steps are long; at decode sizes the small-tile kernel is faster)
-        if constexpr (FMT == MOE_FMT_INT8 || FMT == MOE_FMT_FP8_REF) return launch_gemm_kind<FMT, GK_PAIR>(P, a, stream);
-        else return launch_gemm_kind<FMT, GK_GENERAL>(P, a, stream);
+        return launch_gemm_kind<FMT, GK_GENERAL>(P, a, stream);
     }
 }
 
@@ -1271,7 +1132,7 @@ int launch_gemm_exact(const moe_grouped_args* a, hipStream_t stream) {
     switch (a->format) {
         case MOE_FMT_FP4_REF: return launch_gemm_kind<MOE_FMT_FP4_REF, GK_PAIR_EXACT>(P, a, stream);
         case MOE_FMT_INT4: return launch_gemm_kind<MOE_FMT_INT4, GK_PAIR_EXACT>(P, a, stream);
-        case MOE_FMT_FP8_REF: return launch_gemm_kind<MOE_FMT_FP8_REF, GK_SKINNY_EXACT>(P, a, stream);
+        case MOE_FMT_FP8_REF: return launch_gemm_kind<MOE_FMT_FP8_REF, GK_PAIR_EXACT>(P, a, stream);
         default: return MOE_ERR_BAD_FORMAT;
     }
 }
