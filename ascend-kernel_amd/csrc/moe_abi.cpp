@@ -69,7 +69,7 @@ const char* moe_strerror(int status) {
         case MOE_ERR_BAD_FORMAT: return "unknown weight format / computeType";
         case MOE_ERR_BAD_SHAPE: return "shape not valid for this weight format";
         case MOE_ERR_BAD_ALIGNMENT: return "size or pointer alignment not supported by the kernels";
-        case MOE_ERR_TOO_LARGE: return "M, K, N or G out of int32 range";
+        case MOE_ERR_TOO_LARGE: return "M, K, N or G out of int32 range, or more experts than the grouped GEMM supports";
         case MOE_ERR_LAUNCH: return "kernel launch failed";
         case MOE_ERR_NO_DEVICE: return "no gfx950 device";
         default: return "unknown moe_status";
@@ -104,7 +104,10 @@ int moe_dequant_fp4_bf16_validate(const moe_dequant_args* a) {
 int moe_grouped_gemm_validate(const moe_grouped_args* a) {
     // the fp4_b32 tile routine steps through K 128 at a time
     const bool fp4_k = a && (a->format == MOE_FMT_FP4_B32 || a->format == MOE_FMT_FP4_B16);
-    return validate_grouped(a, fp4_k ? 128 : 64, 256, true);
+    const int rc = validate_grouped(a, fp4_k ? 128 : 64, 256, true);
+    if (rc != MOE_OK) return rc;
+    // the GEMM kernels keep G + 1 tile counts in LDS next to their tile buffers
+    return a->G > MOE_GEMM_MAX_EXPERTS ? MOE_ERR_TOO_LARGE : MOE_OK;
 }
 
 // GEMV: N-contiguous containers are read 256 columns per wavefront step,

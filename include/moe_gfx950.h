@@ -42,6 +42,9 @@ extern "C" {
 /* hipStream_t, passed opaquely so that this header needs no HIP include. */
 typedef void *moe_stream_t;
 
+/* moe_grouped_gemm keeps a table of G + 1 tile counts in LDS next to its tile buffers. */
+#define MOE_GEMM_MAX_EXPERTS 2047
+
 typedef enum moe_status {
     MOE_OK = 0,
     MOE_ERR_NULL_POINTER = -1,   /* a required pointer is NULL                        */
@@ -50,7 +53,8 @@ typedef enum moe_status {
     MOE_ERR_BAD_ALIGNMENT = -4,  /* K/N/cols not a multiple the kernels need, or a
                                     pointer not aligned to 16 bytes                   */
     MOE_ERR_TOO_LARGE = -5,      /* M, K, N or G beyond int32 (reference limit,
-                                    grouped_matmul_antiquant_tiling.cpp:260-264)       */
+                                    grouped_matmul_antiquant_tiling.cpp:260-264), or
+                                    more experts than MOE_GEMM_MAX_EXPERTS            */
     MOE_ERR_LAUNCH = -6,         /* hipLaunchKernel reported an error                 */
     MOE_ERR_NO_DEVICE = -7       /* no gfx950 device / wrong architecture             */
 } moe_status;
