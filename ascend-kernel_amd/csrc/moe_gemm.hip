@@ -452,9 +452,13 @@ template <int FMT>
 constexpr int pair_stages() { return (FMT == MOE_FMT_INT8 || FMT == MOE_FMT_FP8_REF) ? 4 : 5; }
 // 16-byte units of scales per k step: rows of 256 bf16, int4 one per 32-k sub-step (groups are multiples
 // of 32), the reference fp4 container one per 16 k; fp8 one unit per wavefront holding the fp32 scale of
-// its 128 x 128 block; int8 none (per-channel scales stay in registers)
+// its 128 x 128 block; int8 none (per-channel scales stay in registers); the K-contiguous fp4 containers 4
+// (per-32 scales) or 8 bytes (per-16) for each of the tile's 256 weight rows
 template <int FMT>
-constexpr int pair_sc_units() { return FMT == MOE_FMT_FP4_REF ? 128 : FMT == MOE_FMT_INT4 ? 64 : FMT == MOE_FMT_FP8_REF ? 8 : 0; }
+constexpr int pair_sc_units() {
+    return (FMT == MOE_FMT_FP4_REF || FMT == MOE_FMT_FP4_B16) ? 128 : (FMT == MOE_FMT_INT4 || FMT == MOE_FMT_FP4_B32) ? 64
+           : FMT == MOE_FMT_FP8_REF ? 8 : 0;
+}
 template <int FMT>
 constexpr int pair_lds_units() { return pair_stages<FMT>() * (PAIR_A_UNITS + pair_b_units<FMT>() + pair_sc_units<FMT>()); }
 
@@ -466,10 +470,13 @@ constexpr int pair_lds_units() { return pair_stages<FMT>() * (PAIR_A_UNITS + pai
 // own MFMA.  These MFMAs are compiler-visible builtins (their results feed ordinary VALU code).
 template <int FMT, int MT, bool EXACT = false>
 __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* smem, int g, int64_t row0, int rows, int n0) {
-    static_assert(FMT == MOE_FMT_INT4 || FMT == MOE_FMT_FP4_REF || FMT == MOE_FMT_INT8 || FMT == MOE_FMT_FP8_REF,
-                  "the k-split tile routine decodes int4, int8 and the reference fp4 / fp8 containers");
-    static_assert(!EXACT || FMT != MOE_FMT_INT8, "the GEMV op has no int8 container");
+    static_assert(FMT != MOE_FMT_BF16, "the k-split tile routine decodes quantized containers");
+    static_assert(!EXACT || FMT == MOE_FMT_INT4 || FMT == MOE_FMT_FP4_REF || FMT == MOE_FMT_FP8_REF,
+                  "un-rounded weights: the N-contiguous containers of the GEMV op");
     constexpr bool FP4 = FMT == MOE_FMT_FP4_REF, I8 = FMT == MOE_FMT_INT8, F8 = FMT == MOE_FMT_FP8_REF;
+    // K-contiguous fp4 (weight [N, K/2], scales [N, K/KBLK]): the step's tile is 256 weight rows x 32 bytes
+    constexpr bool KC = FMT == MOE_FMT_FP4_B32 || FMT == MOE_FMT_FP4_B16;
+    constexpr int KBLK = FMT == MOE_FMT_FP4_B32 ? 32 : 16;
     constexpr bool B8 = I8 || F8;   // one byte per weight: tiles of 64 rows x 256 bytes
     constexpr int BK = 64, S = pair_stages<FMT>(), PAIR_SC_UNITS = pair_sc_units<FMT>();
     constexpr int PAIR_B_UNITS = pair_b_units<FMT>();
@@ -492,13 +499,14 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
 
     const int64_t KN = (int64_t)P.K * P.N;
     const rsrc_t rw = B8 ? make_rsrc(P.w + g * KN, KN) : make_rsrc(P.w + g * (KN >> 1), KN >> 1);
-    const rsrc_t rs = make_rsrc(static_cast<const uint16_t*>(P.scale) + (int64_t)g * P.scale_rows * P.N,
-                                (int64_t)P.scale_rows * P.N * 2);
+    const rsrc_t rs = KC ? make_rsrc(static_cast<const uint16_t*>(P.scale) + g * (KN / KBLK), (KN / KBLK) * 2)
+                         : make_rsrc(static_cast<const uint16_t*>(P.scale) + (int64_t)g * P.scale_rows * P.N,
+                                     (int64_t)P.scale_rows * P.N * 2);
     // fp8: the expert's fp32 block scales [K/128, N/128]; this wavefront's 128-column block
     const rsrc_t rs8 = make_rsrc(static_cast<const float*>(P.scale) + (int64_t)g * (P.K >> 7) * (P.N >> 7),
                                  (int64_t)(P.K >> 7) * (P.N >> 7) * 4);
     const int cs8 = ((n0 + 64 * cw) >> 7) * 4;
-    const uint32_t per = B8 ? 1u : (uint32_t)((P.K / P.scale_rows) >> 5);      // 32-k sub-steps per scale group
+    const uint32_t per = (B8 || KC) ? 1u : (uint32_t)((P.K / P.scale_rows) >> 5);      // 32-k sub-steps per scale group
     const uint32_t gmul = per == 1 ? 0u : 0xffffffffu / per + 1u;   // sub-step -> scale row as a multiply
     auto scale_row = [&](uint32_t sub) { return gmul ? (int)__umulhi(sub, gmul) : (int)sub; };
     // x rows through a buffer resource that ends after the last valid row (padded rows read as
@@ -512,8 +520,12 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
     // int8 / fp8 (rows of 256 bytes): instruction e of wavefront wv brings rows 8 wv + 4 e + (lane >> 4); the
     // 64-byte quarters of a row are permuted by (row >> 3) & 3 = wv & 3, so that the four q groups read
     // from different quarters of the banks
-    const int vb = B8 ? (lane >> 4) * P.N + (((lane & 15) ^ (4 * (wv & 3))) * 16)
-                      : (lane >> 3) * (P.N >> 1) + (((lane & 7) ^ (4 * (wv & 1))) * 16);
+    // K-contiguous fp4: LDS unit 64 wv + lane of the stage holds one 16-byte half of weight row
+    // n = 32 wv + (lane >> 1); the halves of the rows with odd (n >> 3) are swapped (bank spread)
+    const int kc_n = 32 * wv + (lane >> 1);
+    const int vb = KC   ? kc_n * (P.K >> 1) + 16 * ((lane & 1) ^ ((kc_n >> 3) & 1))
+                   : B8 ? (lane >> 4) * P.N + (((lane & 15) ^ (4 * (wv & 3))) * 16)
+                        : (lane >> 3) * (P.N >> 1) + (((lane & 7) ^ (4 * (wv & 1))) * 16);
     constexpr int NA = (2 * MT + 7) / 8;   // x load instructions per wavefront per step
     constexpr int NB = B8 ? 2 : 1;         // packed-tile instructions
     constexpr int NI = NA + NB + (PAIR_SC_UNITS ? 1 : 0);   // + an eighth of the step's scales
@@ -525,8 +537,12 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
         ja[m] = j * 64;
         ca[m] = 8 * j * P.K * 2;
     }
-    const int cb = B8 ? 8 * wv * P.N + n0 : 8 * wv * (P.N >> 1) + (n0 >> 1);
-    const int kb_step = B8 ? BK * P.N : BK * (P.N >> 1);
+    const int cb = KC ? n0 * (P.K >> 1) : B8 ? 8 * wv * P.N + n0 : 8 * wv * (P.N >> 1) + (n0 >> 1);
+    const int kb_step = KC ? BK / 2 : B8 ? BK * P.N : BK * (P.N >> 1);
+    // K-contiguous fp4 scales: 4 bytes per lane.  Per-16: dword 64 wv + lane = half (lane & 1) of row
+    // 32 wv + (lane >> 1); per-32: lanes < 32, dword 32 wv + lane = row 32 wv + lane
+    const int kc_vs = KBLK == 16 ? (kc_n * (P.K / 16) + 2 * (lane & 1)) * 2 : (32 * wv + lane) * (P.K / 32) * 2;
+    const int kc_cs = n0 * (P.K / KBLK) * 2;
     // scales of a step: int4 2 rows of 512 bytes, 128 bytes (8 lanes) per wavefront: bytes [128 (wv & 3), +128) of
     // row wv >> 2; fp4 4 rows (one per 16 k), 256 bytes (16 lanes) per wavefront: bytes [256 (wv & 1), +256) of row wv >> 1
     const int cs = FP4 ? n0 * 2 + (wv & 1) * 256 : n0 * 2 + (wv & 3) * 128;
@@ -540,6 +556,10 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
             const int e = m - NA;
             lds_load16(rw, lds_b + ST * PAIR_B_UNITS + wv * (PAIR_B_UNITS / 8) + e * 64, vb,
                        cb + (B8 ? 4 * e * P.N : 0) + (kt + AHEAD) * kb_step);
+        } else if constexpr (KC) {
+            if (KBLK == 16 || lane < 32)
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, MOE_LDS_PTR(lds_s + ST * PAIR_SC_UNITS + wv * (PAIR_SC_UNITS / 8)), 4,
+                                                         kc_vs, kc_cs + (kt + AHEAD) * (BK / KBLK) * 2, 0, 0);
         } else if constexpr (F8) {
             // the block scale of the stage's 128-k block, 4 bytes by lane 0 (past K: reads as 0, unused)
             if (lane == 0)
@@ -622,6 +642,19 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
             } else {
                 sc = *reinterpret_cast<const u32x2_t*>(sc16 + 256 * (2 * h + (q >> 1)) + col0);
             }
+        } else if constexpr (KC) {
+            // MFMA t takes weight row n = 64 cw + 16 t + i: its 8 codes k = 32 h + 8 q + [0, 8) are dword q of
+            // the row's half h; the scale of that block
+            const uint32_t* t32 = reinterpret_cast<const uint32_t*>(lds_b + st * PAIR_B_UNITS);
+            uint32_t s4[4];
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                const int n = 64 * cw + 16 * t + i;
+                r[t] = t32[(2 * n + (h ^ ((i >> 3) & 1))) * 4 + q];
+                s4[t] = KBLK == 16 ? sc16[4 * n + 2 * h + (q >> 1)] : sc16[2 * n + h];
+            }
+            sc[0] = s4[0] | (s4[1] << 16);
+            sc[1] = s4[2] | (s4[3] << 16);
         } else if constexpr (B8) {
             // dword 16 cw + i of each of this lane's 8 k rows; the quarter of the row it lies in is
             // permuted by (row >> 3) & 3 = q (see vb)
@@ -652,7 +685,7 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
         if constexpr (EXACT) {
             m[0] = m[1] = m[2] = m[3] = FP4 ? 1.f : 512.f;
             z[0] = z[1] = z[2] = z[3] = FP4 ? 0.f : -8.f;
-        } else if constexpr (FP4) {
+        } else if constexpr (FP4 || KC) {
             m[0] = s0; m[1] = s1; m[2] = s2; m[3] = s3;
             z[0] = z[1] = z[2] = z[3] = 0.f;
         } else {
@@ -674,6 +707,20 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
                 // first x fragments of the MFMA phase, read under the rest of the decode
 #pragma unroll
                 for (int f = 0; f < R; ++f) afr[f & 3] = la[a_lds_unit<BK>(16 * f + i, 4 * h + q)];
+            }
+            if constexpr (KC) {
+                // dword r[t] = 8 consecutive k of MFMA t's weight row: byte p = the k pair p
+#pragma unroll
+                for (int t = p0; t < p0 + 2; ++t) {
+                    const f32x2_t f0 = e2m1_pair_to_f32<0>(r[t]), f1 = e2m1_pair_to_f32<1>(r[t]);
+                    const f32x2_t f2 = e2m1_pair_to_f32<2>(r[t]), f3 = e2m1_pair_to_f32<3>(r[t]);
+                    bf[t][0] = pack_bf16_rne(f0[0] * m[t], f0[1] * m[t]);
+                    bf[t][1] = pack_bf16_rne(f1[0] * m[t], f1[1] * m[t]);
+                    bf[t][2] = pack_bf16_rne(f2[0] * m[t], f2[1] * m[t]);
+                    bf[t][3] = pack_bf16_rne(f3[0] * m[t], f3[1] * m[t]);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+                continue;
             }
             if constexpr (F8) {
                 // byte t of the dwords of k rows 2p, 2p+1, decoded as a pair through fp16 (see
@@ -878,6 +925,18 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
                 __builtin_amdgcn_raw_buffer_store_b32(
                     pack_bf16_rne(swiglu(acc[mt][0][r], acc[mt][2][r]), swiglu(acc[mt][1][r], acc[mt][3][r])), ro, vo,
                     (16 * mt + r) * NO * 2, 0);
+    } else if (h == 0 && KC) {
+        // K-contiguous containers: MFMA t holds column 64 cw + 16 t + i, one 2-byte store each
+        const rsrc_t ry = make_rsrc(P.y + row0 * (int64_t)P.N, (int64_t)rows * P.N * 2);
+        const int vy = (4 * q * P.N + n0 + 64 * cw + i) * 2;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+#pragma unroll
+                for (int t = 0; t < 4; ++t)
+                    __builtin_amdgcn_raw_buffer_store_b16((uint16_t)(pack_bf16_rne(acc[mt][t][r], 0.f) & 0xffffu), ry,
+                                                          vy + 32 * t, (16 * mt + r) * P.N * 2, 0);
     } else if (h == 0) {
         // epilogue through a buffer resource that ends after the tile's last valid row: stores to
         // padded rows fall outside it and are dropped
@@ -923,8 +982,7 @@ template <int FMT, int KIND>
 struct KernelCfg {
     static constexpr bool PAIR = KIND == GK_PAIR || KIND == GK_PAIR_EXACT;
     static constexpr bool SKINNY = KIND == GK_SKINNY;
-    static_assert(!PAIR || FMT == MOE_FMT_INT4 || FMT == MOE_FMT_FP4_REF || FMT == MOE_FMT_INT8 || FMT == MOE_FMT_FP8_REF,
-                  "the k-split tile routine decodes int4, int8 and the reference fp4 / fp8 containers");
+    static_assert(!PAIR || FMT != MOE_FMT_BF16, "the k-split tile routine decodes quantized containers");
     static constexpr int WAVES = PAIR ? 8 : 4;
     static constexpr int BN = GM_BN;                                             // columns per tile
     static constexpr int WG_PER_CU = SKINNY ? GM_SKINNY_WAVES : 1;
@@ -1116,7 +1174,7 @@ static int launch_gemm_fmt(const moe_grouped_args* a, hipStream_t stream) {
     // The N-contiguous containers run on the k-split kernel at every batch size: measured faster than the
     // small-tile kernel down to decode batches of 1-2 rows per expert (256 experts of 7168 x 2048: int4
     // 243 vs 344 us at 128 rows, fp4 476 vs 519 us and fp8 610 vs 784 us at 512 rows).
-    if constexpr (FMT == MOE_FMT_INT4 || FMT == MOE_FMT_FP4_REF || FMT == MOE_FMT_FP8_REF || FMT == MOE_FMT_INT8) {
+    if constexpr (FMT != MOE_FMT_BF16) {
         return launch_gemm_kind<FMT, GK_PAIR>(P, a, stream);
     } else {
         // Decode-like batches (on average at most 24 rows per expert; group_list itself stays on the
