@@ -452,15 +452,17 @@ template <int FMT>
 constexpr int pair_stages() { return (FMT == MOE_FMT_INT8 || FMT == MOE_FMT_FP8_REF) ? 4 : 5; }
 // 16-byte units of scales per k step: rows of 256 bf16, int4 one per 32-k sub-step (groups are multiples
 // of 32), the reference fp4 container one per 16 k; fp8 one unit per wavefront holding the fp32 scale of
-// its 128 x 128 block; int8 none (per-channel scales stay in registers); the K-contiguous fp4 containers 4
-// (per-32 scales) or 8 bytes (per-16) for each of the tile's 256 weight rows
+// its 128 x 128 block; int8 none (per-channel scales stay in registers)
 template <int FMT>
-constexpr int pair_sc_units() {
-    return (FMT == MOE_FMT_FP4_REF || FMT == MOE_FMT_FP4_B16) ? 128 : (FMT == MOE_FMT_INT4 || FMT == MOE_FMT_FP4_B32) ? 64
-           : FMT == MOE_FMT_FP8_REF ? 8 : 0;
+constexpr int pair_sc_units() { return FMT == MOE_FMT_FP4_REF ? 128 : FMT == MOE_FMT_INT4 ? 64 : FMT == MOE_FMT_FP8_REF ? 8 : 0; }
+// The K-contiguous fp4 containers keep their scales [N, K/block] outside the stages: 16 bytes (2 or 4 steps'
+// worth) per weight row at a time, three buffers of 256 rows
+template <int FMT>
+constexpr int pair_kc_scale_units() { return (FMT == MOE_FMT_FP4_B32 || FMT == MOE_FMT_FP4_B16) ? 3 * 256 : 0; }
+template <int FMT>
+constexpr int pair_lds_units() {
+    return pair_stages<FMT>() * (PAIR_A_UNITS + pair_b_units<FMT>() + pair_sc_units<FMT>()) + pair_kc_scale_units<FMT>();
 }
-template <int FMT>
-constexpr int pair_lds_units() { return pair_stages<FMT>() * (PAIR_A_UNITS + pair_b_units<FMT>() + pair_sc_units<FMT>()); }
 
 // EXACT selects the arithmetic of the GEMV op (grouped_soft_gemv/op_kernel/gemv_impl.h:147-199: the
 // dequantized weights stay fp32): the B fragments then hold the codes themselves, which are exact in
@@ -528,7 +530,7 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
                         : (lane >> 3) * (P.N >> 1) + (((lane & 7) ^ (4 * (wv & 1))) * 16);
     constexpr int NA = (2 * MT + 7) / 8;   // x load instructions per wavefront per step
     constexpr int NB = B8 ? 2 : 1;         // packed-tile instructions
-    constexpr int NI = NA + NB + (PAIR_SC_UNITS ? 1 : 0);   // + an eighth of the step's scales
+    constexpr int NI = NA + NB + ((PAIR_SC_UNITS || KC) ? 1 : 0);   // + an eighth of the step's scales
     int ja[NA], ca[NA];
 #pragma unroll
     for (int m = 0; m < NA; ++m) {
@@ -539,10 +541,20 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
     }
     const int cb = KC ? n0 * (P.K >> 1) : B8 ? 8 * wv * P.N + n0 : 8 * wv * (P.N >> 1) + (n0 >> 1);
     const int kb_step = KC ? BK / 2 : B8 ? BK * P.N : BK * (P.N >> 1);
-    // K-contiguous fp4 scales: 4 bytes per lane.  Per-16: dword 64 wv + lane = half (lane & 1) of row
-    // 32 wv + (lane >> 1); per-32: lanes < 32, dword 32 wv + lane = row 32 wv + lane
-    const int kc_vs = KBLK == 16 ? (kc_n * (P.K / 16) + 2 * (lane & 1)) * 2 : (32 * wv + lane) * (P.K / 32) * 2;
-    const int kc_cs = n0 * (P.K / KBLK) * 2;
+    // K-contiguous fp4 scales.  Fetching the 4 or 8 bytes a weight row needs per step costs a request per
+    // row and step (measured: 20 % of the kernel); instead 16 bytes of a row -- the scales of SUP steps --
+    // are fetched at a time: the load slot of step kt brings, for step index kp = kt + KC_D, the rows
+    // [RPS (kp % SUP), + RPS) of super-block kp / SUP (one lane per row, RPW rows per wavefront) into buffer
+    // (kp / SUP) % 3 of 256 rows x 16 bytes behind the stages.  KC_D = SUP + 3: a load issued in step t is
+    // visible after barrier t + 2, and the scales of step s are read during step s - 1.  Three buffers: the
+    // first load into a buffer comes after the last read of its previous occupant.
+    constexpr int SUP = KBLK == 32 ? 4 : 2, KC_D = SUP + 3, RPS = 256 / SUP, RPW = RPS / 8;
+    const int kc_vs = lane * (P.K / KBLK) * 2;
+    auto kc_issue_scale = [&](int kp) {
+        const int sb = kp / SUP, j = kp % SUP, row = RPS * j + RPW * wv;
+        if (lane < RPW)
+            lds_load16(rs, lds_s + (sb % 3) * 256 + row, kc_vs, (n0 + row) * (P.K / KBLK) * 2 + sb * 16);
+    };
     // scales of a step: int4 2 rows of 512 bytes, 128 bytes (8 lanes) per wavefront: bytes [128 (wv & 3), +128) of
     // row wv >> 2; fp4 4 rows (one per 16 k), 256 bytes (16 lanes) per wavefront: bytes [256 (wv & 1), +256) of row wv >> 1
     const int cs = FP4 ? n0 * 2 + (wv & 1) * 256 : n0 * 2 + (wv & 3) * 128;
@@ -557,9 +569,7 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
             lds_load16(rw, lds_b + ST * PAIR_B_UNITS + wv * (PAIR_B_UNITS / 8) + e * 64, vb,
                        cb + (B8 ? 4 * e * P.N : 0) + (kt + AHEAD) * kb_step);
         } else if constexpr (KC) {
-            if (KBLK == 16 || lane < 32)
-                __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, MOE_LDS_PTR(lds_s + ST * PAIR_SC_UNITS + wv * (PAIR_SC_UNITS / 8)), 4,
-                                                         kc_vs, kc_cs + (kt + AHEAD) * (BK / KBLK) * 2, 0, 0);
+            kc_issue_scale(kt + KC_D);
         } else if constexpr (F8) {
             // the block scale of the stage's 128-k block, 4 bytes by lane 0 (past K: reads as 0, unused)
             if (lane == 0)
@@ -612,6 +622,11 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
     // groups -AHEAD .. -1: stages 0 .. AHEAD-1; stages 0 and 1 must have landed before the first barrier
     // (WAITN: the loads of the S - 3 youngest groups may still be in flight at a barrier)
     constexpr int WAITN = (S - 3) * NI;
+    if constexpr (KC) {
+        // the scale loads the groups below do not cover (older than all of them: landed by the first barrier)
+#pragma unroll
+        for (int kp = 0; kp < KC_D - AHEAD; ++kp) kc_issue_scale(kp);
+    }
 #pragma unroll
     for (int st0 = 0; st0 < AHEAD; ++st0) issue_group(st0 - AHEAD, st0);
     asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(WAITN) : "memory");
@@ -623,7 +638,8 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
     // this lane's packed dwords and scales of its sub-step of LDS stage st
     uint32_t r[8];
     u32x2_t sc = {0u, 0u}, sc2 = {0u, 0u};   // sc2: with EXACT, the fp4 scales of the second 16 k of the sub-step
-    auto read_raw = [&](int st) {
+    // (s: the step the stage belongs to)
+    auto read_raw = [&](int st, int s) {
         const uint16_t* sc16 = reinterpret_cast<const uint16_t*>(lds_s + st * PAIR_SC_UNITS);
         if constexpr (FP4) {
             // Reference pre-shuffle (grouped_gemm/test/python/test_group_gemm_fp4.py:129-142): the tile row
@@ -646,12 +662,15 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
             // MFMA t takes weight row n = 64 cw + 16 t + i: its 8 codes k = 32 h + 8 q + [0, 8) are dword q of
             // the row's half h; the scale of that block
             const uint32_t* t32 = reinterpret_cast<const uint32_t*>(lds_b + st * PAIR_B_UNITS);
+            // the row's 8 scales of super-block s / SUP; this lane's block among them
+            const uint16_t* sup = reinterpret_cast<const uint16_t*>(lds_s + ((s / SUP) % 3) * 256) +
+                                  (KBLK == 16 ? 4 * (s % SUP) + 2 * h + (q >> 1) : 2 * (s % SUP) + h);
             uint32_t s4[4];
 #pragma unroll
             for (int t = 0; t < 4; ++t) {
                 const int n = 64 * cw + 16 * t + i;
                 r[t] = t32[(2 * n + (h ^ ((i >> 3) & 1))) * 4 + q];
-                s4[t] = KBLK == 16 ? sc16[4 * n + 2 * h + (q >> 1)] : sc16[2 * n + h];
+                s4[t] = sup[8 * n];
             }
             sc[0] = s4[0] | (s4[1] << 16);
             sc[1] = s4[2] | (s4[3] << 16);
@@ -669,7 +688,7 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
             sc = *reinterpret_cast<const u32x2_t*>(sc16 + 256 * h + col0);
         }
     };
-    read_raw(0);
+    read_raw(0, 0);
 
     // One data step; st = step mod S is its LDS stage, sn the next one, sl the stage this step's loads
     // go to (wave-uniform).
@@ -871,7 +890,7 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
             }
 #pragma unroll
             for (int m = (mt * NI + MT - 1) / MT; m < ((mt + 1) * NI + MT - 1) / MT; ++m) issue(m, kt, sl);
-            if (mt == 0) read_raw(sn);
+            if (mt == 0) read_raw(sn, kt + 1);
             __builtin_amdgcn_sched_barrier(0);
         }
         __builtin_amdgcn_s_setprio(0);

@@ -43,7 +43,7 @@ extern "C" {
 typedef void *moe_stream_t;
 
 /* moe_grouped_gemm keeps a table of G + 1 tile counts in LDS next to its tile buffers. */
-#define MOE_GEMM_MAX_EXPERTS 2047
+#define MOE_GEMM_MAX_EXPERTS 1024
 
 typedef enum moe_status {
     MOE_OK = 0,

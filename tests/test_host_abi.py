@@ -68,8 +68,8 @@ def test_grouped_validate_accepts_good_and_rejects_bad(op):
     assert val(ctypes.byref(gargs(0, G=0))) == mg.ERR_BAD_SHAPE
     assert val(ctypes.byref(gargs(0, K=1 << 31, scale_rows=(1 << 31) // 16))) == mg.ERR_TOO_LARGE  # reference limit
     # the grouped GEMM keeps a tile table of G + 1 entries in LDS; the GEMV op falls back to a kernel without one
-    assert val(ctypes.byref(gargs(0, G=2047))) == mg.MOE_OK
-    assert val(ctypes.byref(gargs(0, G=2048))) == (mg.ERR_TOO_LARGE if op == "gemm" else mg.MOE_OK)
+    assert val(ctypes.byref(gargs(0, G=1024))) == mg.MOE_OK
+    assert val(ctypes.byref(gargs(0, G=1025))) == (mg.ERR_TOO_LARGE if op == "gemm" else mg.MOE_OK)
     assert val(ctypes.byref(gargs(0, weight=None))) == mg.ERR_NULL_POINTER
     assert val(ctypes.byref(gargs(0, group_list=None))) == mg.ERR_NULL_POINTER
     assert val(ctypes.byref(gargs(0, scale=None))) == mg.ERR_NULL_POINTER
