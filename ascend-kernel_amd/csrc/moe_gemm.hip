@@ -14,7 +14,7 @@
 // L2.  A workgroup has 4 wavefronts; every wavefront owns 64 of the 256 columns for
 // ALL rows of the tile, so each weight element is dequantized exactly once per tile.
 // x tiles go through a double-buffered, XOR-swizzled LDS tile shared by the 4 waves.
-// (That is gemm_tile, used by the K-contiguous containers.  The N-contiguous ones -- int4, int8 and
+// (That is gemm_tile, used by the bf16 container.  The quantized ones -- int4, int8, the K-contiguous fp4 containers and
 // the reference's fp4 and fp8 containers -- use a tile routine with 8 wavefronts and LDS-direct loads
 // instead, see gemm_tile_pair.)
 //
@@ -104,7 +104,7 @@ struct BCtx {
 };
 
 // Each weight container provides
-//   Raw        packed registers of one k step (or one sub-step ring, see load_sub)
+//   Raw        packed registers of one k step
 //   load_sub   global loads of 32-k sub-step s of the step starting at k0
 //   Dq         the decode, cut into units so that it can be interleaved with MFMAs:
 //              prep(raw, c, s) once per sub-step, then unit(raw, c, s, p, t, out) for
@@ -114,66 +114,12 @@ struct BCtx {
 template <int FMT>
 struct BTraits;
 
-// ------------------------------------------- fp4 block-32 / block-16, [N, K/2]
-// K-contiguous: MFMA t, lane (i, q) owns column 64w + 16t + i and loads the 16 bytes
-// holding k = k0 + 32q + [0,32) (one scale block of 32, or two of 16); sub-step s uses
-// k = k0 + 32q + 8s + [0,8), so the matching x chunk is 4q + s.
-template <int BLK>
-struct BTraitsFp4K {
-    static constexpr int BK = 128, NS = 4;
-    // One 16-byte load per t serves all 4 sub-steps, so the registers cannot be reloaded
-    // sub-step by sub-step: a whole step is loaded into a second register set (load_sub
-    // ignores its sub-step argument and is called once per step).
-    static constexpr bool DOUBLE_RAW = true;
-    static constexpr int MT_MAX = 10;  // larger tiles spill: BK = 128 doubles the x staging registers
-    static constexpr int SPB = 32 / BLK;   // scales per 16-byte load
-    struct Raw {
-        u32x4_t r[4];
-        uint32_t sc[4];   // block 32: the scale as fp32 bits; block 16: the two bf16 scales, unpacked where used
-    };
-    __device__ static __forceinline__ int a_chunk(int s, int q) { return 4 * q + s; }
-    __device__ static __forceinline__ int col(const BCtx& c, int t) { return 64 * c.w + 16 * t + c.i; }
-    __device__ static __forceinline__ void init(BCtx& c) {
-        c.vw = (64 * c.w + c.i) * (c.K >> 1) + 16 * c.q;
-        c.vs = ((64 * c.w + c.i) * (c.K / BLK) + SPB * c.q) * 2;
-    }
-    __device__ static __forceinline__ void load_sub(Raw& raw, const BCtx& c, int k0, int) {
-#pragma unroll
-        for (int t = 0; t < 4; ++t) {
-            raw.r[t] = ldg_b128(c.rw, c.vw, (c.n0 + 16 * t) * (c.K >> 1) + (k0 >> 1));
-            const int so = ((c.n0 + 16 * t) * (c.K / BLK) + k0 / BLK) * 2;
-            if constexpr (BLK == 32)
-                raw.sc[t] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b16(c.rs, c.vs, so, 0) << 16;
-            else
-                raw.sc[t] = ldg_b32(c.rs, c.vs, so);
-        }
-    }
-    struct Dq {
-        __device__ __forceinline__ void init_tile(const BCtx&) {}
-        __device__ __forceinline__ void prep(const Raw&, const BCtx&, int) {}
-        __device__ __forceinline__ void unit(const Raw& raw, const BCtx&, int s, int p, int t, u32x4_t out[4]) {
-            const uint32_t wd = pinned(raw.r[t][s]);
-            // sub-steps 0, 1 / 2, 3 are the two blocks of 16
-            const float sc = BLK == 32 ? __uint_as_float(raw.sc[t]) : (s >> 1) ? bf16_hi(raw.sc[t]) : bf16_lo(raw.sc[t]);
-            out[t][p] = pinned(p == 0   ? e2m1_pair_scaled_bf16<0>(wd, sc)
-                               : p == 1 ? e2m1_pair_scaled_bf16<1>(wd, sc)
-                               : p == 2 ? e2m1_pair_scaled_bf16<2>(wd, sc)
-                                        : e2m1_pair_scaled_bf16<3>(wd, sc));
-        }
-    };
-};
-template <>
-struct BTraits<MOE_FMT_FP4_B32> : BTraitsFp4K<32> {};
-template <>
-struct BTraits<MOE_FMT_FP4_B16> : BTraitsFp4K<16> {};
-
 // ------------------------------------------------------------------ bf16, [N, K]
 // K-contiguous: lane (i, q) loads 32 contiguous bytes, k = k0 + 16q + [0,16); sub-step
 // s uses the half k0 + 16q + 8s + [0,8), so the matching x chunk is 2q + s.
 template <>
 struct BTraits<MOE_FMT_BF16> {
     static constexpr int BK = 64, NS = 2;
-    static constexpr bool DOUBLE_RAW = false;
     static constexpr int MT_MAX = 11;
     struct Raw {
         u32x4_t r[4][2];
@@ -215,20 +161,9 @@ __device__ __forceinline__ void make_ctx(BCtx& c, const GemmParams& P, int g, in
     c.K = P.K; c.N = P.N; c.n0 = n0;
     c.i = lane & 15; c.q = lane >> 4; c.w = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int64_t KN = (int64_t)P.K * P.N;
-    switch (FMT) {
-        case MOE_FMT_FP4_B32:
-            c.rw = make_rsrc(P.w + g * (KN >> 1), KN >> 1);
-            c.rs = make_rsrc(static_cast<const uint16_t*>(P.scale) + g * (KN >> 5), KN >> 4);
-            break;
-        case MOE_FMT_FP4_B16:
-            c.rw = make_rsrc(P.w + g * (KN >> 1), KN >> 1);
-            c.rs = make_rsrc(static_cast<const uint16_t*>(P.scale) + g * (KN >> 4), KN >> 3);
-            break;
-        default:
-            c.rw = make_rsrc(P.w + g * KN * 2, KN * 2);
-            c.rs = c.rw;
-            break;
-    }
+    static_assert(FMT == MOE_FMT_BF16, "the 4-wavefront tile routine serves the bf16 container");
+    c.rw = make_rsrc(P.w + g * KN * 2, KN * 2);
+    c.rs = c.rw;
 }
 
 // Epilogue: fp32 -> bf16 (RNE), rows beyond the chunk are dropped.
@@ -282,7 +217,7 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& P, u32x4_t* lds_a, i
         for (int t = 0; t < 4; ++t) acc[mt][t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
     u32x4_t areg[PASSES];
-    typename T::Raw raw, raw_next;
+    typename T::Raw raw;
     const int nk = P.K / BK;
 
     // Every pass is done by all threads: rows past the tile read as zeros (they lie beyond the
@@ -303,8 +238,7 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& P, u32x4_t* lds_a, i
     //  * weights: while the MFMAs of sub-step f run, the fragments of sub-step f+1 are
     //    decoded, one unit (two elements of one column) at a time between MFMAs; as soon as
     //    a sub-step's packed registers have been decoded they are refilled with the same
-    //    sub-step of the next k step, straight from global memory a full step ahead
-    //    (formats whose loads span a whole step keep a second register set);
+    //    sub-step of the next k step, straight from global memory a full step ahead;
     //  * x: fragments come from LDS through a ring of 4 register sets, read RING
     //    fragments ahead of their MFMAs; the x tile of step kt+1 travels through registers
     //    into the other LDS buffer.
@@ -318,7 +252,7 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& P, u32x4_t* lds_a, i
     load_a(0);
     store_a(0);
 #pragma unroll
-    for (int s = 0; s < (T::DOUBLE_RAW ? 1 : NS); ++s) T::load_sub(raw, c, 0, s);
+    for (int s = 0; s < NS; ++s) T::load_sub(raw, c, 0, s);
     u32x4_t bf[2][4];
     dq.prep(raw, c, 0);
 #pragma unroll
@@ -327,10 +261,7 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& P, u32x4_t* lds_a, i
         for (int t = 0; t < 4; ++t) dq.unit(raw, c, 0, p, t, bf[0]);
     __syncthreads();
     // raw[0] <- sub-step 0 of step 1, a full step ahead
-    if (T::DOUBLE_RAW)
-        T::load_sub(raw_next, c, BK, 0);
-    else
-        T::load_sub(raw, c, BK, 0);
+    T::load_sub(raw, c, BK, 0);
 
     // One k step.  The global loads of the next x tile are issued one per MFMA slot at the start
     // of the first sub-step, the LDS writes one per slot at the end of the last one, so that
@@ -351,7 +282,6 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& P, u32x4_t* lds_a, i
             const int sn = (s + 1) % NS;                 // sub-step being decoded
             u32x4_t* bcur = bf[s & 1];
             u32x4_t* bnxt = bf[(s + 1) & 1];
-            if (T::DOUBLE_RAW && sn == 0) raw = raw_next;  // the next step's registers become current
 #pragma unroll
             for (int slot = 0; slot < SLOTS; ++slot) {
                 const int mt = slot >> 2, t = slot & 3, f = s * MT + mt;
@@ -369,11 +299,7 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& P, u32x4_t* lds_a, i
                 }
                 if (slot == ((UNITS - 1) * SLOTS) / UNITS) {
                     // everything of sub-step sn has been decoded: refill its registers
-                    if (T::DOUBLE_RAW) {
-                        if (sn == 0) T::load_sub(raw_next, c, (kt + 2) * BK, 0);
-                    } else {
-                        T::load_sub(raw, c, (kt + (sn == 0 ? 2 : 1)) * BK, sn);
-                    }
+                    T::load_sub(raw, c, (kt + (sn == 0 ? 2 : 1)) * BK, sn);
                 }
                 if (s == NS - 1 && slot >= SLOTS - NW) {
                     const int wi = slot - (SLOTS - NW);
