@@ -428,7 +428,7 @@ constexpr int GF_ROWS = 16;               // activation rows per pass
 constexpr int GF_LDS_UNITS = 4096;        // 64 KiB of x per staged chunk
 constexpr int GF_U = 4;                   // 128-k groups (one 16-byte load per lane each) per loop iteration
 constexpr int GF_KSTEP = 128 * GF_U;      // k per loop iteration; K must be a multiple
-constexpr int GF_GEMM_ROWS_PER_EXPERT = 20;// grouped GEMM calls with at most this many rows per expert on average come here
+constexpr int GF_GEMM_ROWS_PER_EXPERT = 12;// grouped GEMM calls with at most this many rows per expert on average come here
 
 __device__ __forceinline__ uint32_t e2m1_pair_bf16(uint32_t word, int sel) {
     switch (sel) {
@@ -702,7 +702,8 @@ bool gemv_preferred(const moe_grouped_args* a) {
     // read every weight row as contiguous runs.  The bf16 vector kernel takes 4 rows of an expert per
     // pass over its weights (same arithmetic as the GEMM: the weights are bf16 already).  The
     // matrix-core fp4_b32 kernel takes 16 and has a variant with the GEMM's weight rounding; the
-    // bound is where the small-tile GEMM kernel overtakes it (measured at DeepSeek-V3 shapes).
+    // bound is where the k-split GEMM kernel overtakes it (measured at DeepSeek-V3 shapes, 256 experts of
+    // 7168 x 2048: 8 rows per expert 496 vs 631 us, 16 rows 754 vs 651 us).
     if (a->format == MOE_FMT_FP4_B32 || a->format == MOE_FMT_FP4_B16)
         return a->K % GF_KSTEP == 0 && a->M <= GF_GEMM_ROWS_PER_EXPERT * a->G;
     if (a->format == MOE_FMT_BF16) return a->M <= 4 * a->G;

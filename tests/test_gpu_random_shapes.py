@@ -23,9 +23,9 @@ def _say(msg):
 def _random_counts(rng, G, regime):
     if regime == "decode":        # M <= 4 G
         c = rng.integers(0, 5, G)
-    elif regime == "mid":         # around the 16-row block size, M <= 20 G mostly
+    elif regime == "mid":         # around the 16-row block size: both sides of the GEMV / GEMM kernel dispatch bound (12 G)
         c = rng.choice([0, 1, 5, 8, 15, 16, 17, 19], G)
-    elif regime == "small_tile":  # 20 G < M <= 24 G
+    elif regime == "small_tile":  # 20 G < M <= 24 G (bf16: the small-tile kernel)
         c = np.full(G, 22) + rng.integers(-1, 2, G)
     else:                         # prefill: ragged, up to a few row blocks, some empty experts
         c = rng.choice([0, 3, 31, 33, 64, 100, 161, 200], G)
