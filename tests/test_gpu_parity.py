@@ -118,6 +118,24 @@ def test_gemm_parity_deep_k_and_wide_n(fmt, K, N):
     H.assert_close(got, H.oracle_out(case), what=f"{fmt} K={K} N={N}")
 
 
+@pytest.mark.parametrize("op", ["gemm", "gemv"])
+@pytest.mark.parametrize("fmt", ["fp4", "fp8", "int8", "int4", "fp4_b32", "fp4_b16"])
+def test_several_tiles_per_workgroup(fmt, op):
+    """More tiles than the persistent grid has workgroups (256): every workgroup runs several tiles in a
+    row, of different experts, row counts and column blocks, re-using its LDS ring."""
+    if op == "gemv" and fmt not in H.GEMV_FORMATS:
+        pytest.skip("the GEMV op has no such container")
+    _say(f"several tiles per workgroup fmt={fmt} op={op}")
+    rng = np.random.default_rng(zlib.crc32(f"tiles/{fmt}/{op}".encode()))
+    G, K, N = 96, 256, 2048
+    counts = rng.choice([0, 1, 3, 16, 17, 33, 40], G)
+    gl = list(np.cumsum(counts))
+    case = H.make_case(fmt, G, K, N, gl, seed=3, extra_rows=1, group=64)
+    got = H.run_cabi(case, H.upload(case), op)
+    H.assert_close(got, H.oracle_out(case, gemv=op == "gemv"), rows=slice(0, gl[-1]), what=f"tiles {fmt}/{op}")
+    assert (got[gl[-1]:] == 0x7FC0).all()
+
+
 def test_gemm_int4_group_size_32_and_64():
     for group in (32, 64, 256):
         _say(f"gemm int4 group={group}")
