@@ -329,8 +329,8 @@ __device__ __forceinline__ void lds_load16(rsrc_t r, const u32x4_t* dst, int vof
 }
 
 // ---------------------------------------------------------------------------------
-// Tile routine for the N-contiguous containers (int4, int8, reference fp4 / fp8) with two wavefronts per
-// SIMD that split the k range.
+// Tile routine for the quantized containers (int4, int8, reference fp4 / fp8, K-contiguous fp4) with two
+// wavefronts per SIMD that split the k range.  Described for int4; what differs for the others follows.
 //
 // A single wavefront issues at most one instruction every ~5 cycles whatever its kind, and an
 // MFMA holds the SIMD's vector issue port for about 8 of its 16 cycles: with one wavefront
@@ -349,12 +349,12 @@ __device__ __forceinline__ void lds_load16(rsrc_t r, const u32x4_t* dst, int vof
 // barrier one wavefront of the SIMD starts decoding while the other starts multiplying.
 //
 // Everything the k loop consumes -- x tile, packed weight tile, scales -- is brought in by
-// LDS-direct loads into a ring of 5 stages.  The loads of stage kt+4 (it replaces stage kt-1,
+// LDS-direct loads into a ring of S = 5 stages.  The loads of stage kt+4 (it replaces stage kt-1,
 // last read before barrier kt-1) and the LDS reads of the packed dwords of stage kt+1 are
 // spread between the MFMAs of step kt; before barrier kt each wavefront waits until its own
 // loads of stage kt+2 have landed.  vmcnt counts a wavefront's loads in order and every
 // wavefront issues the same number NI of them per step (waves without a row block of their
-// own repeat one), so "at most 2 NI outstanding" means exactly that.
+// own repeat one), so "at most (S - 3) NI outstanding" means exactly that.
 //
 // Decode of a k-row pair (a, b) of one dword column: v_perm gathers the two bytes of each row
 // this lane owns, the low nibbles (& 0x0f0f0f0f) and high nibbles (>> 4 & 0x0f0f0f0f) are bytes
@@ -366,6 +366,16 @@ __device__ __forceinline__ void lds_load16(rsrc_t r, const u32x4_t* dst, int vof
 // brought in by the same loads, a lane's 8 k rows of its 2 bytes are two 16-byte LDS reads, each
 // byte pair decodes to 4 floats with v_cvt_scalef32_pk_f32_fp4 and takes one multiply by the
 // column's scale of that 16-k block (4 scale rows per step instead of 2).
+//
+// int8 and the reference fp8 container: a step's tile is 64 rows of 256 bytes (two load instructions
+// per wavefront), which leaves room for S = 4 stages; a lane's 4 columns are one dword of each of its 8 k
+// rows.  int8 keeps its per-channel scale and offset in registers; fp8 decodes two codes at a time through
+// fp16 (see e4m3_ref_pair_over_256_fp16) and gets the fp32 scale of its 128 x 128 block through the ring,
+// 4 bytes per wavefront and step.
+//
+// K-contiguous fp4 (weight [N, K/2]): a step's tile is 256 weight rows x 32 bytes; MFMA t of a lane takes
+// weight row 64 cw + 16 t + i, whose 8 codes of the sub-step are one dword; the scales [N, K/block] are
+// fetched 16 bytes per row at a time into buffers of their own (see kc_issue_scale).
 // ---------------------------------------------------------------------------------
 constexpr int PAIR_CAPB = 10;                         // x stages hold 160 rows
 constexpr int PAIR_MT_MAX = 10;
