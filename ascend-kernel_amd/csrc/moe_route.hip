@@ -133,10 +133,13 @@ __global__ __launch_bounds__(RT_BLOCK) void route_rank_kernel(const int32_t* __r
 }
 
 __global__ __launch_bounds__(256) void route_gather_kernel(const u32x4_t* __restrict__ x, const int32_t* __restrict__ row_token,
+                                                           const int64_t* __restrict__ group_list, int E,
                                                            u32x4_t* __restrict__ x_sorted, int64_t n, int units) {
     // 4 rows per workgroup, one wavefront each
     const int64_t r = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (r >= n) return;
+    // Only rows below group_list[E - 1] (written by the scan kernel earlier on this stream) have a token:
+    // dropped choices leave the tail of row_token unwritten, and the tail of x_sorted stays untouched.
+    if (r >= n || r >= group_list[E - 1]) return;
     const u32x4_t* src = x + (int64_t)row_token[r] * units;
     u32x4_t* dst = x_sorted + r * units;
     // 8 independent 16-byte loads in flight per lane
@@ -181,7 +184,8 @@ int launch_route(const moe_route_args* a, hipStream_t stream) {
     if (a->x && n > 0) {
         hipLaunchKernelGGL(route_gather_kernel, dim3((unsigned)((n + 3) / 4)), dim3(256), 0, stream,
                            static_cast<const u32x4_t*>(a->x), static_cast<const int32_t*>(a->row_token),
-                           static_cast<u32x4_t*>(a->x_sorted), n, (int)(a->K / 8));
+                           static_cast<const int64_t*>(a->group_list), (int)a->E, static_cast<u32x4_t*>(a->x_sorted), n,
+                           (int)(a->K / 8));
         if (hipGetLastError() != hipSuccess) return MOE_ERR_LAUNCH;
     }
     return MOE_OK;

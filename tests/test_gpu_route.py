@@ -77,6 +77,39 @@ def test_route_ties_and_given_ids_with_dropped_choices():
     assert np.array_equal(rt[: ref_rt.size], ref_rt)
 
 
+def test_route_dropped_choices_with_rows_gathered():
+    """Dropped choices (ids outside [0, E)) together with the row gather: only rows below
+    group_list[E - 1] have a token; the gather must leave the rest of x_sorted untouched and must not
+    read the unwritten tail of row_token."""
+    _say("route dropped ids + gather")
+    rng = np.random.default_rng(11)
+    T, E, K, topk = 700, 9, 128, 5
+    given = rng.integers(-2, E + 2, (T, topk)).astype(np.int32)
+    x = oracle.f32_to_bf16_bits(rng.standard_normal((T, K)).astype(np.float32))
+    ids, _, gl, rt, roc, xs = _route(None, given, x, T, E, K, topk)
+    ref_gl, ref_rt, ref_roc = R.route_sort(given, E)
+    total = int(ref_gl[-1])
+    assert 0 < total < T * topk
+    assert np.array_equal(gl, ref_gl) and np.array_equal(roc, ref_roc)
+    assert np.array_equal(rt[:total], ref_rt) and (rt[total:] == -5).all()
+    assert np.array_equal(xs[:total], x[ref_rt])
+    assert (xs[total:] == 0x7FC0).all()          # sentinel rows untouched
+    # a row of NaN logits selects no expert (every comparison fails): its choices are dropped too
+    T, E, K, topk = 6, 8, 64, 2
+    logits = rng.standard_normal((T, E)).astype(np.float32)
+    logits[2, :] = np.nan
+    x = oracle.f32_to_bf16_bits(rng.standard_normal((T, K)).astype(np.float32))
+    ids, _, gl, rt, roc, xs = _route(logits, None, x, T, E, K, topk)
+    assert int(gl[-1]) == (T - 1) * topk and (roc.reshape(T, topk)[2] == -1).all()
+    valid = [t for t in range(T) if t != 2]
+    ref_ids, _ = R.route_topk(logits[valid], topk)
+    full = np.full((T, topk), -1, dtype=np.int32)
+    full[valid] = ref_ids
+    ref_gl, ref_rt, _ = R.route_sort(full, E)
+    assert np.array_equal(gl, ref_gl) and np.array_equal(rt[: ref_rt.size], ref_rt)
+    assert np.array_equal(xs[: ref_rt.size], x[ref_rt]) and (xs[ref_rt.size:] == 0x7FC0).all()
+
+
 def test_routed_rows_feed_the_grouped_gemm():
     """End to end on the device: logits -> routing -> grouped GEMM on the sorted rows with the
     group_list the routing wrote; expected value from the oracle on the oracle's own sort."""
