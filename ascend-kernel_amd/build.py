@@ -118,6 +118,10 @@ def _check_accumulator_moves(src: str) -> None:
             if any(s1 >= s0 and e1 <= e0 and (s1, e1) != (s0, e0) for s1, e1 in loops):
                 continue  # not innermost
             body = [l.split(";")[0].strip() for l in lines[s0:e0 + 1]]
+            # a k loop stores nothing to global memory; a backward branch around a whole tile (a steps' MFMAs
+            # placed after their loop, then the epilogue) is not one
+            if any(l.startswith(("buffer_store", "global_store")) for l in body):
+                continue
             accs = set()
             for l in body:
                 if l.startswith("v_mfma"):
@@ -143,6 +147,28 @@ def _check_accumulator_moves(src: str) -> None:
                     continue
                 if any(r in accs for r in regs(parts[1].split(",")[0])):
                     raise RuntimeError(f"{src}: {m.group(1)} writes an accumulator right before its MFMA: {prev}")
+            # ... and nothing but another MFMA may touch the result right behind it (the epilogues wait out the
+            # latency with s_nop first); covers the k steps that sit outside the loops
+            for nxt in code[i + 1:i + 1 + ACC_WRITE_GAP]:
+                if nxt.startswith("s_nop 15"):
+                    break
+                parts = nxt.split(None, 1)
+                if nxt.startswith("v_mfma") or nxt.startswith("s_") or len(parts) < 2:
+                    continue
+                if any(r in accs for r in regs(parts[1])):
+                    raise RuntimeError(f"{src}: {m.group(1)} touches an accumulator right behind its MFMA: {nxt}")
+        # LDS reads issued from inline asm (the transposing reads): the compiler believes their result is
+        # there at once, so nothing may name the destination registers before the asm wait that follows
+        for i, l in enumerate(code):
+            if not l.startswith("ds_read_b64_tr_b4"):
+                continue
+            dst = set(regs(l.split(None, 1)[1].split(",")[0]))
+            for nxt in code[i + 1:]:
+                if nxt.startswith("s_waitcnt") and "lgkmcnt(0)" in nxt:
+                    break
+                parts = nxt.split(None, 1)
+                if len(parts) == 2 and any(r in dst for r in regs(parts[1])):
+                    raise RuntimeError(f"{src}: {m.group(1)} names the result of an asm LDS read in flight: {nxt}")
 
 
 def _wait(procs):
