@@ -182,6 +182,17 @@ int moe_route(const moe_route_args* a, moe_stream_t stream) {
     return moe::launch_route(a, static_cast<hipStream_t>(stream));
 }
 
+int moe_route_static(const moe_route_args* a, moe_stream_t stream) {
+    if (!a) return MOE_ERR_NULL_POINTER;
+    // args->workspace is not used: validate with a stand-in so that NULL is accepted there
+    moe_route_args b = *a;
+    b.workspace = reinterpret_cast<void*>(uintptr_t{256});
+    int rc = moe_route_validate(&b);
+    if (rc != MOE_OK) return rc;
+    if (b.T == 0) return moe::launch_route(&b, static_cast<hipStream_t>(stream));   // one kernel that zeroes group_list
+    return moe::launch_route_static(a, static_cast<hipStream_t>(stream));
+}
+
 int moe_grouped_gemm(const moe_grouped_args* a, moe_stream_t stream) {
     int rc = moe_grouped_gemm_validate(a);
     if (rc != MOE_OK) return rc;

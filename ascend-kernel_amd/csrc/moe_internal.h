@@ -16,5 +16,7 @@ int launch_gemm_exact(const moe_grouped_args* a, hipStream_t stream);
 int launch_grouped_gemm(const moe_grouped_args* a, hipStream_t stream);
 int launch_prepack_fp4_ref(const moe_prepack_fp4_args* a, hipStream_t stream);
 int launch_route(const moe_route_args* a, hipStream_t stream);
+// the same with the workspace in the library's own static device array (a->workspace is ignored)
+int launch_route_static(const moe_route_args* a, hipStream_t stream);
 size_t route_workspace_bytes(const moe_route_args* a);
 }  // namespace moe

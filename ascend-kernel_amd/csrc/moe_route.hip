@@ -12,6 +12,8 @@
 //   route_scan_kernel    one workgroup: per expert, prefix over the blocks; then over experts
 //   route_rank_kernel    per block, every choice's rank among the earlier choices of its expert
 //   route_gather_kernel  x rows copied into sorted order, 16 bytes per lane
+#include <atomic>
+
 #include "moe_device.h"
 #include "moe_internal.h"
 
@@ -158,6 +160,31 @@ size_t route_workspace_bytes(const moe_route_args* a) {
     const int64_t n = a->T * a->topk;
     const int64_t nblocks = (n + RT_BLOCK - 1) / RT_BLOCK;
     return (size_t)(2 * nblocks * a->E) * sizeof(int32_t);   // per-block counts and per-block first rows
+}
+
+// Scratch of moe_route_static: the per-block counts and first rows live in this array instead of a
+// caller-provided workspace.  One copy per GPU, held until the process ends; every call on a GPU uses
+// that GPU's copy (the count kernel rewrites all of the part a call reads, so nothing needs clearing,
+// but two calls that overlap in time on one GPU race on it).
+static __device__ __align__(256) unsigned char scratch[MOE_ROUTE_STATIC_SCRATCH_BYTES];
+
+// Device address of `scratch` on each GPU (the array's name is only a host-side handle).  Filled on the
+// first call on a device, with that device current.
+constexpr int RT_MAX_DEVICES = 64;
+static std::atomic<void*> scratch_addr[RT_MAX_DEVICES];
+
+int launch_route_static(const moe_route_args* a, hipStream_t stream) {
+    if (route_workspace_bytes(a) > (size_t)MOE_ROUTE_STATIC_SCRATCH_BYTES) return MOE_ERR_TOO_LARGE;
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= RT_MAX_DEVICES) return MOE_ERR_NO_DEVICE;
+    void* ptr = scratch_addr[dev].load(std::memory_order_acquire);
+    if (!ptr) {
+        if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess || !ptr) return MOE_ERR_NO_DEVICE;
+        scratch_addr[dev].store(ptr, std::memory_order_release);   // a race stores the same address twice
+    }
+    moe_route_args b = *a;
+    b.workspace = ptr;
+    return launch_route(&b, stream);
 }
 
 int launch_route(const moe_route_args* a, hipStream_t stream) {

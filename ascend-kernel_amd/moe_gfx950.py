@@ -26,7 +26,7 @@ SYMBOLS = (
     "moe_dequant_fp4_bf16_workspace_bytes", "moe_grouped_gemm_workspace_bytes", "moe_grouped_gemv_workspace_bytes",
     "moe_dequant_fp4_bf16", "moe_grouped_gemm", "moe_grouped_gemv",
     "moe_prepack_fp4_ref_validate", "moe_prepack_fp4_ref_workspace_bytes", "moe_prepack_fp4_ref",
-    "moe_route_validate", "moe_route_workspace_bytes", "moe_route",
+    "moe_route_validate", "moe_route_workspace_bytes", "moe_route", "moe_route_static",
 )
 
 
@@ -76,6 +76,11 @@ for _n, _t in (("dequant_fp4_bf16", DequantArgs), ("grouped_gemm", GroupedArgs),
     getattr(lib, f"moe_{_n}_workspace_bytes").argtypes = [ctypes.POINTER(_t)]
     getattr(lib, f"moe_{_n}").restype = ctypes.c_int
     getattr(lib, f"moe_{_n}").argtypes = [ctypes.POINTER(_t), ctypes.c_void_p]
+
+
+lib.moe_route_static.restype = ctypes.c_int
+lib.moe_route_static.argtypes = [ctypes.POINTER(RouteArgs), ctypes.c_void_p]
+ROUTE_STATIC_SCRATCH_BYTES = 2 << 20
 
 
 class MoeError(RuntimeError):
@@ -138,3 +143,8 @@ def route_workspace_bytes(args: RouteArgs) -> int:
 
 def route(args: RouteArgs, stream: int = 0) -> None:
     _check(lib.moe_route(ctypes.byref(args), ctypes.c_void_p(stream)), "moe_route")
+
+
+def route_static(args: RouteArgs, stream: int = 0) -> None:
+    """moe_route with the library's own static scratch: args.workspace is ignored, nothing is allocated."""
+    _check(lib.moe_route_static(ctypes.byref(args), ctypes.c_void_p(stream)), "moe_route_static")

@@ -4,8 +4,10 @@
  *
  * Plain C: raw device pointers, sizes, an opaque stream handle.  No torch types.
  * Every launch is asynchronous on the given stream, never synchronizes the
- * device, never copies group_list to the host, allocates nothing and keeps no
- * state between calls (re-entrant).  All functions return MOE_OK (0) or a
+ * device, never copies group_list to the host and allocates nothing.  The only
+ * state between calls is set-up done once per process or GPU (a kernel attribute,
+ * the address of moe_route_static's scratch array); calls are re-entrant except
+ * where moe_route_static says otherwise.  All functions return MOE_OK (0) or a
  * negative moe_status; nothing throws across this boundary.
  *
  * What each entry point replaces in the reference (paths relative to its tree):
@@ -221,6 +223,18 @@ int moe_grouped_gemm(const moe_grouped_args *args, moe_stream_t stream);
 int moe_grouped_gemv(const moe_grouped_args *args, moe_stream_t stream);
 int moe_prepack_fp4_ref(const moe_prepack_fp4_args *args, moe_stream_t stream);
 int moe_route(const moe_route_args *args, moe_stream_t stream);
+
+/* moe_route for callers that cannot allocate device memory or carry a workspace around (code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the
+ * reference.  Same arguments and results as moe_route; args->workspace is ignored (may be NULL): the
+ * scratch is a static device array inside the library, MOE_ROUTE_STATIC_SCRATCH_BYTES per GPU, held
+ * until the process ends.  Calls whose moe_route_workspace_bytes() exceeds it return MOE_ERR_TOO_LARGE
+ * (with 256 experts that is more than 1048576 routed choices T * topk).  Allocates nothing; the first
+ * call on a GPU looks the array's address up (hipGetSymbolAddress), so make that call with the GPU
+ * current and outside a stream capture.  All calls on one GPU share the array: calls that overlap in
+ * time on the same GPU race on it -- keep them on one stream or otherwise ordered. */
+#define MOE_ROUTE_STATIC_SCRATCH_BYTES (2u << 20)
+int moe_route_static(const moe_route_args *args, moe_stream_t stream);
 
 #ifdef __cplusplus
 }
