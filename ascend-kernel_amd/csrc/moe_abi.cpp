@@ -53,6 +53,23 @@ int validate_grouped(const moe_grouped_args* a, int64_t k_mult, int64_t n_mult, 
     if (!aligned16(a->x) || !aligned16(a->weight) || !aligned16(a->y) || !aligned16(a->scale) ||
         !aligned16(a->offset) || (reinterpret_cast<uintptr_t>(a->group_list) & 7u))
         return MOE_ERR_BAD_ALIGNMENT;
+    // The kernels address one expert's weight and scale slab, and one tile's rows of x and y, with 32-bit
+    // byte offsets through buffer resources: each must stay below 2 GiB.
+    const int64_t lim = int64_t{1} << 31;
+    const int64_t kn = a->K * a->N;   // both fit int32
+    int64_t wbytes = kn, sbytes = 0;
+    switch (a->format) {
+        case MOE_FMT_FP4_REF: wbytes = kn / 2; sbytes = a->scale_rows * a->N * 2; break;
+        case MOE_FMT_FP8_REF: sbytes = (a->K / 128) * (a->N / 128) * 4; break;
+        case MOE_FMT_INT8: sbytes = a->N * 2; break;
+        case MOE_FMT_INT4: wbytes = kn / 2; sbytes = a->scale_rows * a->N * 2; break;
+        case MOE_FMT_FP4_B32: wbytes = kn / 2; sbytes = kn / 32 * 2; break;
+        case MOE_FMT_FP4_B16: wbytes = kn / 2; sbytes = kn / 16 * 2; break;
+        case MOE_FMT_BF16: wbytes = kn * 2; break;
+        default: break;
+    }
+    const int64_t tile_rows = 256;   // upper bound on the rows of one tile
+    if (wbytes >= lim || sbytes >= lim || tile_rows * a->K * 2 >= lim || tile_rows * a->N * 2 >= lim) return MOE_ERR_TOO_LARGE;
     return MOE_OK;
 }
 
@@ -69,7 +86,7 @@ const char* moe_strerror(int status) {
         case MOE_ERR_BAD_FORMAT: return "unknown weight format / computeType";
         case MOE_ERR_BAD_SHAPE: return "shape not valid for this weight format";
         case MOE_ERR_BAD_ALIGNMENT: return "size or pointer alignment not supported by the kernels";
-        case MOE_ERR_TOO_LARGE: return "M, K, N or G out of int32 range, or more experts than the grouped GEMM supports";
+        case MOE_ERR_TOO_LARGE: return "M, K, N or G out of int32 range, an expert's weight or scale slab of 2 GiB or more, or more experts than the op supports";
         case MOE_ERR_LAUNCH: return "kernel launch failed";
         case MOE_ERR_NO_DEVICE: return "no gfx950 device";
         default: return "unknown moe_status";
@@ -104,7 +121,9 @@ int moe_dequant_fp4_bf16_validate(const moe_dequant_args* a) {
 int moe_grouped_gemm_validate(const moe_grouped_args* a) {
     // the fp4_b32 tile routine steps through K 128 at a time
     const bool fp4_k = a && (a->format == MOE_FMT_FP4_B32 || a->format == MOE_FMT_FP4_B16);
-    const int rc = validate_grouped(a, fp4_k ? 128 : 64, 256, true);
+    // columns: tiles of 256; the reference's fp8 container comes in multiples of 128
+    // (grouped_gemm/op_host/grouped_matmul_antiquant_tiling.cpp:616-621), its last tile may be half empty
+    const int rc = validate_grouped(a, fp4_k ? 128 : 64, a && a->format == MOE_FMT_FP8_REF ? 128 : 256, true);
     if (rc != MOE_OK) return rc;
     // the GEMM kernels keep G + 1 tile counts in LDS next to their tile buffers
     return a->G > MOE_GEMM_MAX_EXPERTS ? MOE_ERR_TOO_LARGE : MOE_OK;
@@ -115,7 +134,13 @@ int moe_grouped_gemm_validate(const moe_grouped_args* a) {
 int moe_grouped_gemv_validate(const moe_grouped_args* a) {
     if (a && a->format == MOE_FMT_INT8) return MOE_ERR_BAD_FORMAT;  // the GEMV op has no offset operand
     const bool k_major = a && (a->format == MOE_FMT_BF16 || a->format == MOE_FMT_FP4_B32 || a->format == MOE_FMT_FP4_B16);
-    return validate_grouped(a, k_major ? 32 : 64, k_major ? 1 : 256, false);
+    const int rc = validate_grouped(a, k_major ? 32 : 64, k_major ? 1 : a && a->format == MOE_FMT_FP8_REF ? 128 : 256, false);
+    if (rc != MOE_OK) return rc;
+    // experts are the y dimension of the GEMV grids; an fp8 N that is not a multiple of 256 needs the matrix-core
+    // kernel, which keeps G + 1 tile counts in LDS
+    if (a->G > 65535) return MOE_ERR_TOO_LARGE;
+    if (a->format == MOE_FMT_FP8_REF && a->N % 256 && a->G > MOE_GEMM_MAX_EXPERTS) return MOE_ERR_TOO_LARGE;
+    return MOE_OK;
 }
 
 int moe_prepack_fp4_ref_validate(const moe_prepack_fp4_args* a) {

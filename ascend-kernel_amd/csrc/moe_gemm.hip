@@ -442,7 +442,11 @@ __device__ __forceinline__ void pair_finish(const GemmParams& P, u32x4_t* smem, 
         if (rd < ROUNDS) __syncthreads();
     }
 
-    if (h == 0 && P.epilogue == MOE_EPILOGUE_SWIGLU) {
+    // the last tile of an N that is not a multiple of 256 (the reference's fp8 container: multiples of 128)
+    // computes columns past N from whatever follows in the slab: they are not stored
+    const bool live = KC || n0 + col0 < P.N;
+    if (!live) {
+    } else if (h == 0 && P.epilogue == MOE_EPILOGUE_SWIGLU) {
         // this lane's 4 columns are (gate, gate, up, up) of 2 output columns; y has N / 2 columns
         const int NO = P.N >> 1;
         const rsrc_t ro = make_rsrc(P.y + row0 * (int64_t)NO, (int64_t)rows * NO * 2);
@@ -1274,7 +1278,7 @@ __global__ __launch_bounds__((64 * KernelCfg<FMT, KIND>::WAVES), (KernelCfg<FMT,
     constexpr int MTM = C::MTM;
     int* prefix = reinterpret_cast<int*>(smem + C::lds_units());      // [G + 1]
     const int tid = threadIdx.x;
-    const int ntile_n = P.N / C::BN;
+    const int ntile_n = (P.N + C::BN - 1) / C::BN;
 
     // exclusive scan of tiles per expert: each thread takes a contiguous run of experts
     {
@@ -1389,20 +1393,16 @@ static int launch_gemm_kind(const GemmParams& P, const moe_grouped_args* a, hipS
     const size_t lds = (size_t)C::lds_units() * 16 + ((size_t)a->G + 1) * sizeof(int);
     const size_t lds_max = (160 * 1024 - 2048) / C::WG_PER_CU;
     if (lds > lds_max) return MOE_ERR_TOO_LARGE;
-    static bool attr_set = false;  // idempotent; a race only repeats the same call
-    if (!attr_set) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void*>(&grouped_gemm_kernel<FMT, KIND>),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_max) != hipSuccess)
-            return MOE_ERR_LAUNCH;
-        attr_set = true;
-    }
+    static std::atomic<uint64_t> lds_set{0};
+    if (const int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(&grouped_gemm_kernel<FMT, KIND>), (int)lds_max, lds_set))
+        return rc;
     int dev = 0, cus = 256;
     if (hipGetDevice(&dev) != hipSuccess) return MOE_ERR_NO_DEVICE;
     if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return MOE_ERR_NO_DEVICE;
     // persistent grid: as many workgroups as the CUs hold, but no more than an upper bound on the
     // tile count that needs no look at group_list (every expert adds at most one partly filled chunk)
     const int64_t max_chunks = a->M / (16 * C::MTM) + a->G;
-    const int64_t max_tiles = max_chunks * (a->N / C::BN);
+    const int64_t max_tiles = max_chunks * ((a->N + C::BN - 1) / C::BN);
     const int64_t want = max_tiles < (int64_t)cus * C::WG_PER_CU ? max_tiles : (int64_t)cus * C::WG_PER_CU;
     // a multiple of 8 so that the XCD-aware order covers every tile index
     const int64_t grid = want > 0 ? (want + 7) / 8 * 8 : 8;

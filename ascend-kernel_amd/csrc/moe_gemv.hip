@@ -682,13 +682,8 @@ template <int FMT>
 static int launch_nmajor(const moe_grouped_args* a, hipStream_t stream) {
     const size_t lds = (size_t)4 * GV_ROWS * 256 * 4 + (size_t)GV_ROWS * a->K * 2;
     if (lds > 160 * 1024) return MOE_ERR_TOO_LARGE;
-    static bool attr_set = false;  // idempotent; a race only repeats the same call
-    if (!attr_set) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void*>(&gemv_nmajor_kernel<FMT>),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) != hipSuccess)
-            return MOE_ERR_LAUNCH;
-        attr_set = true;
-    }
+    static std::atomic<uint64_t> lds_set{0};
+    if (const int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(&gemv_nmajor_kernel<FMT>), 160 * 1024, lds_set)) return rc;
     dim3 grid((unsigned)(a->N / 256), (unsigned)a->G);
     hipLaunchKernelGGL((gemv_nmajor_kernel<FMT>), grid, dim3(256), lds, stream,
                        static_cast<const uint16_t*>(a->x), static_cast<const uint8_t*>(a->weight), a->scale,

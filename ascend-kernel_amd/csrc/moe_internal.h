@@ -2,9 +2,25 @@
 #pragma once
 #include <hip/hip_runtime.h>
 
+#include <atomic>
+#include <cstdint>
+
 #include "moe_gfx950.h"
 
 namespace moe {
+// Raises a kernel's dynamic LDS limit once per GPU (the attribute belongs to the kernel's image on the
+// current device).  `done` is that kernel's bit mask of devices already set up: the only state the
+// launchers keep.  A race repeats the same call.
+inline int ensure_dynamic_lds(const void* kernel, int bytes, std::atomic<uint64_t>& done) {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return MOE_ERR_NO_DEVICE;
+    if (!((done.load(std::memory_order_acquire) >> dev) & 1u)) {
+        if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes) != hipSuccess) return MOE_ERR_LAUNCH;
+        done.fetch_or(uint64_t{1} << dev, std::memory_order_release);
+    }
+    return MOE_OK;
+}
+
 int launch_dequant_fp4_bf16(const moe_dequant_args* a, hipStream_t stream);
 // gemm_rounding: use the grouped GEMM's arithmetic (weights rounded to bf16) where the two ops differ.
 int launch_grouped_gemv(const moe_grouped_args* a, hipStream_t stream, bool gemm_rounding = false);

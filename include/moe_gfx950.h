@@ -55,8 +55,11 @@ typedef enum moe_status {
     MOE_ERR_BAD_ALIGNMENT = -4,  /* K/N/cols not a multiple the kernels need, or a
                                     pointer not aligned to 16 bytes                   */
     MOE_ERR_TOO_LARGE = -5,      /* M, K, N or G beyond int32 (reference limit,
-                                    grouped_matmul_antiquant_tiling.cpp:260-264), or
-                                    more experts than MOE_GEMM_MAX_EXPERTS            */
+                                    grouped_matmul_antiquant_tiling.cpp:260-264); one
+                                    expert's weight or scale slab of 2 GiB or more, or
+                                    K or N of 4194304 or more (32-bit byte offsets);
+                                    more experts than MOE_GEMM_MAX_EXPERTS (grouped
+                                    GEMM) or 65535 (grouped GEMV)                     */
     MOE_ERR_LAUNCH = -6,         /* hipLaunchKernel reported an error                 */
     MOE_ERR_NO_DEVICE = -7       /* no gfx950 device / wrong architecture             */
 } moe_status;
@@ -73,7 +76,8 @@ typedef enum moe_status {
  *                  K % 64 == 0, N % 256 == 0.
  * MOE_FMT_FP8_REF  reference computeType "fp8": uint8 [G, K, N] e4m3 bits decoded with
  *                  the reference's bit trick (0x7F/0xFF give +-480, no NaN);
- *                  scale fp32 [G, K/128, N/128]; offset ignored.
+ *                  scale fp32 [G, K/128, N/128]; offset ignored.  K % 128 == 0, N % 128 == 0
+ *                  (every other N-contiguous container: N % 256 == 0).
  * MOE_FMT_INT8     int8 [G, K, N]; scale bf16 [G, N]; offset bf16 [G, N];
  *                  W = bf16((float(q) + float(offset)) * float(scale)).
  * MOE_FMT_INT4     uint8 [G, K, N/2], low nibble = even n, codes 0..15, zero point 8;

@@ -119,6 +119,20 @@ def test_gemm_parity_deep_k_and_wide_n(fmt, K, N):
 
 
 @pytest.mark.parametrize("op", ["gemm", "gemv"])
+@pytest.mark.parametrize("N", [128, 384, 1408])
+def test_fp8_n_multiple_of_128(N, op):
+    """The reference tiles uint8 weights 128 columns wide (grouped_gemm/op_host/grouped_matmul_antiquant_tiling.cpp:616-621,
+    grouped_soft_gemv/op_host/grouped_soft_gemv_tiling.cpp:105-128): N need not be a multiple of the 256-column
+    tile here.  The half-empty last tile must write nothing past column N (the row's successor starts there)."""
+    _say(f"fp8 N={N} op={op}")
+    gl = [3, 3, 40, 41] if op == "gemv" else [5, 140, 140, 301]
+    case = H.make_case("fp8", len(gl), 512, N, gl, seed=N, extra_rows=2)
+    got = H.run_cabi(case, H.upload(case), op)
+    H.assert_close(got, H.oracle_out(case, gemv=op == "gemv"), rows=slice(0, gl[-1]), what=f"fp8 N={N} {op}")
+    assert (got[gl[-1]:] == 0x7FC0).all()
+
+
+@pytest.mark.parametrize("op", ["gemm", "gemv"])
 @pytest.mark.parametrize("fmt", ["fp4", "fp8", "int8", "int4", "fp4_b32", "fp4_b16"])
 def test_several_tiles_per_workgroup(fmt, op):
     """More tiles than the persistent grid has workgroups (256): every workgroup runs several tiles in a

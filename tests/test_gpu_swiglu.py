@@ -54,6 +54,15 @@ def test_swiglu_epilogue(fmt, gl):
     assert (got[gl[-1]:] == 0x7FC0).all(), "rows beyond group_list[-1] were written"
 
 
+def test_swiglu_fp8_half_empty_last_tile():
+    _say("swiglu fp8 N=384")
+    gl = [5, 140, 140, 301]
+    case = H.make_case("fp8", len(gl), 256, 384, gl, seed=5, extra_rows=2)
+    got = _run(case)
+    H.assert_close(got, _expected(case), rows=slice(0, gl[-1]), what="swiglu fp8 N=384")
+    assert (got[gl[-1]:] == 0x7FC0).all(), "rows beyond group_list[-1] were written"
+
+
 def test_swiglu_int4_prefill_tile_sizes():
     """Every row-block count of the int4 prefill kernel (1..10 blocks of 16 rows) and ragged last blocks."""
     _say("swiglu int4 tile sizes")

@@ -85,6 +85,48 @@ def test_grouped_validate_accepts_good_and_rejects_bad(op):
     assert val(ctypes.byref(gargs(0, group_list=P + 4))) == mg.ERR_BAD_ALIGNMENT
 
 
+@pytest.mark.parametrize("op", ["gemm", "gemv"])
+def test_slab_and_grid_limits(op):
+    """One expert's weight / scale slab is addressed with 32-bit byte offsets, and the GEMV grids carry the
+    expert index in their y dimension: sizes beyond either are refused, not wrapped."""
+    val = getattr(mg.lib, f"moe_grouped_{op}_validate")
+    # bf16 [N, K]: 32768 x 32768 x 2 bytes = 2 GiB per expert; one row of tiles less fits
+    assert val(ctypes.byref(gargs(5, K=32768, N=32768))) == mg.ERR_TOO_LARGE
+    assert val(ctypes.byref(gargs(5, K=32768, N=32768 - 256))) == mg.MOE_OK
+    # fp8: one byte per weight, 46336 x 46336 < 2 GiB <= 46464 x 46464
+    assert val(ctypes.byref(gargs(1, K=46336, N=46336))) == mg.MOE_OK
+    assert val(ctypes.byref(gargs(1, K=46464, N=46464))) == mg.ERR_TOO_LARGE
+    # 4-bit codes: the fp4_b16 scales (K N / 8 bytes) stay below the codes (K N / 2 bytes)
+    assert val(ctypes.byref(gargs(6, K=65536, N=65536))) == mg.ERR_TOO_LARGE
+    assert val(ctypes.byref(gargs(6, K=65536, N=32768))) == mg.MOE_OK
+    # a 256-row tile of x or y must stay below 2 GiB as well
+    assert val(ctypes.byref(gargs(5, K=1 << 22, N=256))) == mg.ERR_TOO_LARGE
+    if op == "gemv":
+        assert val(ctypes.byref(gargs(5, G=65535))) == mg.MOE_OK
+        assert val(ctypes.byref(gargs(5, G=65536))) == mg.ERR_TOO_LARGE
+
+
+@pytest.mark.parametrize("op", ["gemm", "gemv"])
+def test_fp8_accepts_n_multiple_of_128(op):
+    # the reference tiles uint8 weights 128 columns wide (grouped_gemm/op_host/grouped_matmul_antiquant_tiling.cpp:616-621)
+    val = getattr(mg.lib, f"moe_grouped_{op}_validate")
+    assert val(ctypes.byref(gargs(1, N=384))) == mg.MOE_OK
+    assert val(ctypes.byref(gargs(1, N=1408))) == mg.MOE_OK
+    assert val(ctypes.byref(gargs(1, N=320))) == mg.ERR_BAD_ALIGNMENT
+    assert val(ctypes.byref(gargs(3, N=384))) == mg.ERR_BAD_ALIGNMENT      # the other N-contiguous containers: 256
+    if op == "gemv":   # beyond the tile table of the matrix-core kernel only whole 256-column tiles
+        assert val(ctypes.byref(gargs(1, N=384, G=1025))) == mg.ERR_TOO_LARGE
+        assert val(ctypes.byref(gargs(1, N=512, G=1025))) == mg.MOE_OK
+
+
+def test_route_static_limit_is_checked_on_the_host():
+    # 2 * ceil(T * topk / 1024) * E * 4 bytes of scratch: 1024 experts, 2^20 choices -> 8 MiB > 2 MiB
+    a = mg.route_args(P, 0, P, P, P, P, P, 0, 0, 1 << 17, 1024, 0, 8)
+    assert mg.route_workspace_bytes(a) > mg.ROUTE_STATIC_SCRATCH_BYTES
+    assert mg.lib.moe_route_static(ctypes.byref(a), None) == mg.ERR_TOO_LARGE
+    assert mg.lib.moe_route_static(None, None) == mg.ERR_NULL_POINTER
+
+
 def test_gemm_needs_offset_only_for_int8_and_gemv_rejects_int8():
     assert mg.lib.moe_grouped_gemm_validate(ctypes.byref(gargs(2, offset=None))) == mg.ERR_NULL_POINTER
     assert mg.lib.moe_grouped_gemm_validate(ctypes.byref(gargs(3, offset=None))) == mg.MOE_OK
