@@ -2,14 +2,15 @@
 """Benchmark of the MoE antiquant ops on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload dsv3_int4_prefill] [--no-extra] [--no-cpu]
+                    [--only headline|dequant|route|gemv_bf16|gemm_int8|fused_fp4|reference_containers|prepack]
 
 A step is one pass of the hot path over one batch of synthetic input that is already
 resident in HBM.  The headline workload is the DeepSeek-V3-shaped int4-antiquant MoE
 prefill: 256 experts, 4096 tokens x top-8 = 32768 sorted rows, gate_up (K=7168, N=4096)
 followed by down (K=2048, N=7168), int4 weights with zero point 8 and bf16 per-group-128
 scales.  One JSON line is printed: whole-step TFLOP/s, the roofline of the dominant kernel
-(measured with events on the launch stream), the CPU oracle timed on a bounded sample of
-the same workload, and -- unless --no-extra -- the other benchmark configurations
+(measured with events on the launch stream), the CPU baselines (a torch restatement of the
+reference's host-side check and the C oracle, timed on bounded samples), and -- unless --no-extra -- the other benchmark configurations
 (FP4 dequant, grouped GEMV, int8 GEMM, fused FP4 GEMM at decode shape vs dequant + bf16
 GEMM) as GB/s or TFLOP/s with their own roofline fractions.
 
@@ -30,11 +31,21 @@ sys.path.insert(0, ROOT)
 
 PEAK_HBM_GBS = 8000.0        # MI355X HBM3E, 8 TB/s
 PEAK_BF16_TFLOPS = 2500.0    # MI355X dense bf16 MFMA, 2.5 PFLOP/s
-# HBM bytes per launch of the int4 grouped GEMM on this workload (mean of the gate_up and down
-# launches), from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs of this script scaled by the
-# --copy-calibration copy (summary under profiles/): 3.27 GB read + 0.369 GB written.
-# Algorithmic bytes: 3.21 GB + 0.369 GB.
-INT4_GEMM_HBM_BYTES_PER_LAUNCH = 3.65e9
+# HBM bytes per launch of the int4 grouped GEMM on this workload (mean of the gate_up and down launches) are
+# not something a timing run can see: they come from two rocprofv3 --pmc runs of this script (FETCH_SIZE,
+# WRITE_SIZE), scaled by the --copy-calibration copy.  The figure, the kernel it was taken on and the summary
+# it comes from are kept in this file next to the profile summaries.
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "grouped_gemm_int4_dsv3_prefill_hbm_traffic.json")
+
+
+def measured_traffic():
+    """(bytes per launch, provenance) from the committed counter summary, or (None, None)."""
+    try:
+        with open(TRAFFIC_FILE) as f:
+            t = json.load(f)
+        return float(t["hbm_bytes_per_launch"]), {k: t[k] for k in ("source", "measured_on", "kernel") if k in t}
+    except (OSError, ValueError, KeyError):
+        return None, None
 
 
 def routed_counts(torch, tokens, experts, topk, gen, max_rows=None):
@@ -140,7 +151,7 @@ def build_dsv3_int4_prefill(torch, mg, gen):
     counts = routed_counts(torch, tokens, G, topk, gen)
     gl = counts.cumsum(0).to(torch.int64).cuda()
     M = tokens * topk
-    ops, flops = [], []
+    ops, flops, nbytes = [], [], []
     for name, K, N in (("gate_up", H, 2 * I), ("down", I, H)):
         x = bf16_normal(torch, (M, K))
         w = torch.randint(0, 256, (G, K, N // 2), dtype=torch.uint8, device="cuda")   # two uniform nibbles per byte
@@ -148,12 +159,36 @@ def build_dsv3_int4_prefill(torch, mg, gen):
         y = torch.empty(M, N, dtype=torch.bfloat16, device="cuda")
         ops.append(Op(mg, torch, "gemm", "int4", x, w, s, None, gl, y, scale_rows=K // 128))
         flops.append(2.0 * M * K * N)
-    return dict(ops=ops, flops=flops, names=["gate_up", "down"], M=M, G=G,
+        nbytes.append(x.numel() * 2 + w.numel() + s.numel() * 2 + y.numel() * 2)
+    return dict(ops=ops, flops=flops, names=["gate_up", "down"], M=M, G=G, bytes_per_launch=sum(nbytes) / len(nbytes),
                 desc="DeepSeek-V3 MoE prefill, int4 antiquant: 256 experts, 4096 tokens x top-8 = 32768 rows, "
                      "gate_up K=7168 N=4096 + down K=2048 N=7168, zero point 8, bf16 scales per 128 k")
 
 
-def run_extra(torch, mg, gen, iters, warmup):
+EXTRA = ("dequant", "prepack", "route", "gemv_bf16", "gemm_int8", "fused_fp4", "reference_containers")
+
+
+def run_extra(torch, mg, gen, iters, warmup, only=None):
+    """The other benchmark configurations; `only` names one of EXTRA to run just that one (for profiles that
+    must hold a single workload's kernels)."""
+    out = {}
+    want = lambda name: only is None or only == name
+    if want("dequant"):
+        out.update(extra_dequant(torch, mg, warmup))
+    if want("prepack"):
+        out.update(extra_prepack(torch, mg, warmup))
+    if want("route"):
+        out.update(extra_route(torch, mg, warmup))
+    if want("gemv_bf16"):
+        out.update(extra_gemv_bf16(torch, mg, gen, iters, warmup))
+    if want("gemm_int8"):
+        out.update(extra_gemm_int8(torch, mg, iters, warmup))
+    if want("fused_fp4") or want("reference_containers"):
+        out.update(extra_decode_256e(torch, mg, gen, iters, warmup, fused=want("fused_fp4"), ref=want("reference_containers")))
+    return out
+
+
+def extra_dequant(torch, mg, warmup):
     out = {}
     # c1: FP4 e2m1 -> BF16 dequant of a 7168 x 2048 weight, per-32 bf16 scales
     R, C = 7168, 2048
@@ -184,7 +219,12 @@ def run_extra(torch, mg, gen, iters, warmup):
                                              "sets (cold) / on the same buffers (Infinity Cache warm); graph_replay: the same 320 "
                                              "rotating launches captured in one HIP graph (no host launch cost)")
     del codes, scales, outs
+    return out
 
+
+def extra_prepack(torch, mg, warmup):
+    out = {}
+    stream = lambda: torch.cuda.current_stream().cuda_stream
     # weight preparation for the reference's "fp4" container: checkpoint codes [G, N, K/2] + scales [G, N, K/16]
     # -> [G, K, N/2] + [G, K/16, N] (nibble transpose + tile permutation, scale merge + transpose)
     G, K, N = 32, 7168, 2048
@@ -201,7 +241,12 @@ def run_extra(torch, mg, gen, iters, warmup):
     nbytes = 2 * (ck.numel() + sck.numel() * 2)
     out["prepack_fp4_ref_32e"] = dict(bytes=nbytes, us=t * 1e6, GBps=nbytes / t / 1e9, frac_hbm=nbytes / t / 1e9 / PEAK_HBM_GBS)
     del ck, sck, wo, so
+    return out
 
+
+def extra_route(torch, mg, warmup):
+    out = {}
+    stream = lambda: torch.cuda.current_stream().cuda_stream
     # routing for configuration 4: 4096 tokens, 256 experts, top-8, K = 7168: logits -> top-k -> group_list
     # and the token rows gathered into expert order
     T, E, K, topk = 4096, 256, 7168, 8
@@ -221,7 +266,11 @@ def run_extra(torch, mg, gen, iters, warmup):
     out["routing_4096x256_top8"] = dict(bytes=nbytes, us=t * 1e6, GBps=nbytes / t / 1e9, frac_hbm=nbytes / t / 1e9 / PEAK_HBM_GBS,
                                         note="5 kernels: top-k, histogram, scan, rank, row gather")
     del lg, xr, xs
+    return out
 
+
+def extra_gemv_bf16(torch, mg, gen, iters, warmup):
+    out = {}
     # c2: grouped GEMV decode, 64 experts, 32 rows (4 tokens x top-8), K=7168, N=2048, bf16 weights [G,N,K]
     G, K, N = 64, 7168, 2048
     counts = routed_counts(torch, 4, G, 8, gen, max_rows=4)
@@ -237,7 +286,11 @@ def run_extra(torch, mg, gen, iters, warmup):
     out["grouped_gemv_bf16_64e"] = dict(active_experts=A, rows=M, bytes=nbytes, us=t * 1e6, GBps=nbytes / t / 1e9,
                                         frac_hbm=nbytes / t / 1e9 / PEAK_HBM_GBS)
     del x, w, y, op
+    return out
 
+
+def extra_gemm_int8(torch, mg, iters, warmup):
+    out = {}
     # c3: int8 antiquant grouped GEMM, 8 experts, multinomial 4096 rows, K=4096, N=14336
     G, M, K, N = 8, 4096, 4096, 14336
     counts = torch.distributions.Multinomial(M, torch.full((G,), 1.0 / G)).sample().to(torch.int64)
@@ -253,7 +306,13 @@ def run_extra(torch, mg, gen, iters, warmup):
     out["grouped_gemm_int8_8e"] = dict(flops=fl, us=t * 1e6, TFLOPs=fl / t / 1e12,
                                        frac_mfma=fl / t / 1e12 / PEAK_BF16_TFLOPS)
     del x, w, s, o, y, op
+    return out
 
+
+def extra_decode_256e(torch, mg, gen, iters, warmup, fused=True, ref=True):
+    out = {}
+    stream = lambda: torch.cuda.current_stream().cuda_stream
+    run_fused, run_ref = fused, ref
     # c5: fused FP4 (e2m1, per-32 bf16 scales) grouped GEMM at decode shape vs dequant + bf16 grouped GEMM
     G, K, N = 256, 7168, 2048
     counts = routed_counts(torch, 64, G, 8, gen)
@@ -261,9 +320,19 @@ def run_extra(torch, mg, gen, iters, warmup):
     M = int(counts.sum())
     A = int((counts > 0).sum())
     x = bf16_normal(torch, (M, K))
+    y = torch.empty(M, N, dtype=torch.bfloat16, device="cuda")
+    if run_fused:
+        out.update(decode_fused_fp4(torch, mg, iters, warmup, G, K, N, M, A, x, gl, y))
+    if run_ref:
+        out.update(decode_reference_containers(torch, mg, iters, warmup, G, K, N, M, A, x, gl, y))
+    return out
+
+
+def decode_fused_fp4(torch, mg, iters, warmup, G, K, N, M, A, x, gl, y):
+    out = {}
+    stream = lambda: torch.cuda.current_stream().cuda_stream
     w = torch.randint(0, 256, (G, N, K // 2), dtype=torch.uint8, device="cuda")
     s = bf16_uniform(torch, (G, N, K // 32), 2.0 ** -8, 2.0 ** -2)
-    y = torch.empty(M, N, dtype=torch.bfloat16, device="cuda")
     fused = Op(mg, torch, "gemm", "fp4_b32", x, w, s, None, gl, y)
     wd = torch.empty(G, N, K, dtype=torch.bfloat16, device="cuda")
     y2 = torch.empty(M, N, dtype=torch.bfloat16, device="cuda")
@@ -284,7 +353,11 @@ def run_extra(torch, mg, gen, iters, warmup):
                                              gemv_op_us=t_v * 1e6, gemv_op_frac_hbm=nbytes / t_v / 1e9 / PEAK_HBM_GBS,
                                              max_abs_diff_fused_vs_separate=diff)
     del w, s, wd, y2, y3, fused, sep, gemv
+    return out
 
+
+def decode_reference_containers(torch, mg, iters, warmup, G, K, N, M, A, x, gl, y):
+    out = {}
     # the same decode batch on the reference's own containers (N-contiguous: pre-shuffled fp4 with per-16
     # scales, fp8 with 128 x 128 block scales) and on int4 group-128, through both ops
     ref = {}
@@ -308,33 +381,153 @@ def run_extra(torch, mg, gen, iters, warmup):
     return out
 
 
-def cpu_baseline(torch, seed):
-    """The CPU oracle on a bounded sample of the headline workload: the gate_up GEMM
-    (K=7168, N=4096, int4, group 128) of 64 of the 256 experts (a quarter of the rows)."""
+# --------------------------------------------------------------------------- CPU baselines
+# The reference checks its NPU ops against torch code on the host: unpack the codes with int16 shifts, decode them
+# with a bit trick into bf16, apply the scales block by block in a Python loop, then one matmul per expert
+# (grouped_gemm/test/python/test_group_gemm_fp4.py:86-102 and :196-217, test_group_gemm_fp8.py:16-47).  The
+# functions below restate those loops in torch for each benchmark configuration and are timed on the host's
+# cores on a bounded sample; the C/OpenMP oracle is timed beside them on the headline workload.
+def _timed(fn, budget_s):
+    reps, t0 = 0, time.perf_counter()
+    while reps == 0 or time.perf_counter() - t0 < budget_s:
+        fn()
+        reps += 1
+    return reps, time.perf_counter() - t0
+
+
+def _unpack_nibbles(torch, packed):
+    """uint8 [..., n/2] (even element in the low nibble) -> uint8 [..., n], one code per byte (unpack_weight)."""
+    t = packed.to(torch.int16)
+    t = ((t & 0x00F0) << 4) | (t & 0x000F)
+    return t.view(torch.uint8)
+
+
+def _e2m1_to_bf16(torch, codes):
+    """e2m1 codes (one per byte) -> bf16 by the reference's bit trick (fp4_dequant): sign to bit 15, the three
+    magnitude bits to the top of a bf16 subnormal-range pattern, times 2^126."""
+    w = codes.to(torch.int16)
+    w = ((w & 0x0008) << 12) | ((w & 0x0007) << 6)
+    return w.view(torch.bfloat16) * torch.tensor(0x7E80, dtype=torch.int16).view(torch.bfloat16)
+
+
+def torch_cpu_fp4_dequant(torch, codes, scale, block):
+    w = _e2m1_to_bf16(torch, _unpack_nibbles(torch, codes))
+    for i in range(scale.shape[-1]):
+        w[..., i * block:(i + 1) * block] *= scale[..., i].unsqueeze(-1)
+    return w
+
+
+def torch_cpu_int4_weights(torch, packed, scale, group):
+    """int4 [G, K, N/2], zero point 8, scale bf16 [G, K/group, N] -> bf16 [G, K, N]."""
+    w = _unpack_nibbles(torch, packed).to(torch.bfloat16) - 8
+    for i in range(scale.shape[-2]):
+        w[:, i * group:(i + 1) * group, :] *= scale[:, i, :].unsqueeze(-2)
+    return w
+
+
+def torch_cpu_grouped_matmul(torch, x, w_kn, counts):
+    """One fp32 matmul per expert over its rows (what npu_grouped_matmul is checked against); w_kn[g] is [K, N]."""
+    y = torch.empty(x.shape[0], w_kn.shape[-1], dtype=torch.bfloat16)
+    r0 = 0
+    for g, m in enumerate(counts):
+        if m:
+            y[r0:r0 + m] = (x[r0:r0 + m].float() @ w_kn[g].float()).to(torch.bfloat16)
+        r0 += m
+    return y
+
+
+def cpu_baseline(torch, seed, extra=True):
     import numpy as np
 
     import oracle
 
+    torch.manual_seed(seed)
+    cores = torch.get_num_threads()
+    bf = torch.bfloat16
+    uni = lambda shape, lo, hi: (torch.rand(shape) * (hi - lo) + lo).to(bf)
+
+    # headline: the gate_up GEMM (K=7168, N=4096, int4 group 128) of 4 of the 256 experts, 128 rows each
+    G, K, N = 4, 7168, 4096
+    counts = [128] * G
+    M = sum(counts)
+    x = torch.randn(M, K).to(bf)
+    w = torch.randint(0, 256, (G, K, N // 2), dtype=torch.uint8)
+    sc = uni((G, K // 128, N), 1e-3, 1e-2)
+    reps, dt = _timed(lambda: torch_cpu_grouped_matmul(torch, x, torch_cpu_int4_weights(torch, w, sc, 128), counts), 5.0)
+    fl = 2.0 * M * K * N
+    res = dict(value=fl * reps / dt / 1e12, unit="TFLOP/s", cores=cores, kind="port",
+               sample=f"torch restatement of the reference's host check (int16 unpack, bf16 decode, per-group scale loop, "
+                      f"one fp32 matmul per expert): {reps} x gate_up GEMM of {G} experts ({M} rows, K={K}, N={N}, int4 "
+                      f"group 128) in {dt:.2f} s on {cores} torch threads, dequant included")
+    # the C / OpenMP oracle on the same shape, 16 experts
     rng = np.random.default_rng(seed)
-    G, K, N = 64, 7168, 4096
-    counts = rng.multinomial(128 * G, np.full(G, 1.0 / G))
-    gl = np.cumsum(counts).astype(np.int64)
-    M = int(gl[-1])
-    x = torch.from_numpy(rng.standard_normal((M, K)).astype(np.float32)).to(torch.bfloat16)
-    xb = x.view(torch.int16).numpy().view(np.uint16)
-    w = rng.integers(0, 256, (G, K, N // 2), dtype=np.uint8)
-    s = torch.from_numpy(rng.uniform(1e-3, 1e-2, (G, K // 128, N)).astype(np.float32)).to(torch.bfloat16)
-    sb = s.view(torch.int16).numpy().view(np.uint16)
+    Gc = 16
+    cnt = rng.multinomial(128 * Gc, np.full(Gc, 1.0 / Gc))
+    glc = np.cumsum(cnt).astype(np.int64)
+    Mc = int(glc[-1])
+    xb = torch.randn(Mc, K).to(bf).view(torch.int16).numpy().view(np.uint16)
+    wc = rng.integers(0, 256, (Gc, K, N // 2), dtype=np.uint8)
+    sb = uni((Gc, K // 128, N), 1e-3, 1e-2).view(torch.int16).numpy().view(np.uint16)
     oracle.lib()
-    reps, t0 = 0, time.perf_counter()
-    while reps == 0 or time.perf_counter() - t0 < 10.0:      # about 10 s of wall time on all host threads
-        oracle.grouped_gemm(oracle.FMT_INT4, xb, w, sb, None, gl)
-        reps += 1
-    dt = time.perf_counter() - t0
-    fl = 2.0 * M * K * N * reps
-    return dict(value=fl / dt / 1e12, unit="TFLOP/s", cores=oracle.num_threads(), kind="port",
-                sample=f"{reps} x gate_up GEMM of {G} experts ({M} rows, K={K}, N={N}, int4 group 128): "
-                       f"{fl / 1e9:.1f} GFLOP in {dt:.2f} s on the oracle's OpenMP loops (dequant included)")
+    reps, dt = _timed(lambda: oracle.grouped_gemm(oracle.FMT_INT4, xb, wc, sb, None, glc), 5.0)
+    res["c_port"] = dict(value=2.0 * Mc * K * N * reps / dt / 1e12, unit="TFLOP/s", cores=oracle.num_threads(),
+                         sample=f"{reps} x gate_up GEMM of {Gc} experts ({Mc} rows) in {dt:.2f} s on the oracle's OpenMP loops")
+    del x, w, sc, xb, wc, sb
+    if not extra:
+        return res
+    wl = {}
+    # c1: FP4 dequant of 7168 x 2048, per-32 scales
+    R, C = 7168, 2048
+    codes = torch.randint(0, 256, (R, C // 2), dtype=torch.uint8)
+    s1 = uni((R, C // 32), 2.0 ** -8, 2.0 ** -2)
+    reps, dt = _timed(lambda: torch_cpu_fp4_dequant(torch, codes, s1, 32), 2.5)
+    nb = R * C // 2 + R * (C // 32) * 2 + R * C * 2
+    wl["fp4_dequant_7168x2048"] = dict(value=nb * reps / dt / 1e9, unit="GB/s", sample=f"{reps} x the full weight in {dt:.2f} s")
+    # c2: bf16 grouped GEMV, 64 experts, 32 rows
+    G, K, N = 64, 7168, 2048
+    counts = [1] * 16 + [2] * 8          # the active experts; the other 40 have no rows and are never touched
+    x = torch.randn(sum(counts), K).to(bf)
+    w = (torch.randn(len(counts), N, K) * 0.02).to(bf)
+    A = len(counts)
+
+    def gemv():
+        r0 = 0
+        for g, m in enumerate(counts):
+            if m:
+                (x[r0:r0 + m].float() @ w[g].float().t()).to(bf)
+            r0 += m
+
+    reps, dt = _timed(gemv, 2.5)
+    nb = A * N * K * 2 + sum(counts) * (K + N) * 2
+    wl["grouped_gemv_bf16_64e"] = dict(value=nb * reps / dt / 1e9, unit="GB/s",
+                                       sample=f"{reps} x {A} active experts, {sum(counts)} rows in {dt:.2f} s")
+    del x, w
+    # c3: int8 antiquant GEMM, 1 of the 8 experts (512 rows)
+    K, N, m = 4096, 14336, 512
+    x = torch.randn(m, K).to(bf)
+    q = torch.randint(-127, 128, (K, N), dtype=torch.int8)
+    s3, o3 = uni((N,), 1e-3, 1e-2), uni((N,), -2.0, 2.0)
+    reps, dt = _timed(lambda: (x.float() @ ((q.float() + o3.float()) * s3.float()).to(bf).float()).to(bf), 2.5)
+    wl["grouped_gemm_int8_8e"] = dict(value=2.0 * m * K * N * reps / dt / 1e12, unit="TFLOP/s",
+                                      sample=f"{reps} x one expert of 512 rows (K={K}, N={N}) in {dt:.2f} s, dequant included")
+    del x, q
+    # c5: FP4 weights at decode shape: dequant + matmul of 8 active experts, 2 rows each
+    G, K, N = 8, 7168, 2048
+    codes = torch.randint(0, 256, (G, N, K // 2), dtype=torch.uint8)
+    s5 = uni((G, N, K // 32), 2.0 ** -8, 2.0 ** -2)
+    x = torch.randn(2 * G, K).to(bf)
+
+    def fused():
+        wd = torch_cpu_fp4_dequant(torch, codes, s5, 32)
+        for g in range(G):
+            (x[2 * g:2 * g + 2].float() @ wd[g].float().t()).to(bf)
+
+    reps, dt = _timed(fused, 2.5)
+    nb = G * (N * K // 2 + N * (K // 32) * 2) + 2 * G * (K + N) * 2
+    wl["fused_fp4_gemm_decode_256e"] = dict(value=nb * reps / dt / 1e9, unit="GB/s",
+                                            sample=f"{reps} x 8 active experts, 16 rows in {dt:.2f} s (packed bytes / time)")
+    res["workloads"] = wl
+    return res
 
 
 def main():
@@ -344,6 +537,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="dsv3_int4_prefill")
     ap.add_argument("--no-extra", action="store_true", help="skip the other benchmark configurations")
+    ap.add_argument("--only", choices=("headline",) + EXTRA, default=None,
+                    help="run just this workload's GPU launches and print its figures (for profiles of one kernel)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU oracle baseline")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one plain 1 GiB device copy (known traffic) to scale FETCH_SIZE / WRITE_SIZE")
@@ -363,6 +558,13 @@ def main():
     torch.cuda.set_device(0)
     gen = torch.Generator().manual_seed(0)
     torch.manual_seed(0)
+
+    if args.only in EXTRA:
+        print(json.dumps({"only": args.only, "workloads": run_extra(torch, mg, gen, max(args.steps, 20), args.warmup, only=args.only)}),
+              flush=True)
+        return
+    if args.only == "headline":
+        args.no_extra = args.no_cpu = True
 
     if args.copy_calibration:
         src = torch.empty(1 << 30, dtype=torch.uint8, device="cuda").fill_(1)
@@ -390,8 +592,10 @@ def main():
     t_each = time_launches(torch, ops, args.steps, 1)
     avg_launch = sum(t_each) / len(t_each)
     achieved = (step_flops / len(ops)) / avg_launch / 1e12
+    traffic, traffic_from = measured_traffic()
     roofline = dict(bound="mfma", achieved=achieved, peak=PEAK_BF16_TFLOPS, unit="TFLOP/s",
-                    frac=achieved / PEAK_BF16_TFLOPS, traffic=INT4_GEMM_HBM_BYTES_PER_LAUNCH,
+                    frac=achieved / PEAK_BF16_TFLOPS, traffic=traffic, traffic_from=traffic_from,
+                    algorithmic_bytes_per_launch=wl["bytes_per_launch"],
                     kernel="moe::grouped_gemm_kernel<int4>",
                     per_launch={n: dict(us=t * 1e6, TFLOPs=f / t / 1e12, frac=f / t / 1e12 / PEAK_BF16_TFLOPS)
                                 for n, t, f in zip(wl["names"], t_each, wl["flops"])})
@@ -428,7 +632,7 @@ def main():
         result["workloads"]["gate_up_swiglu_fused"] = fused
         torch.cuda.empty_cache()
     if not args.no_cpu:
-        result["cpu_baseline"] = cpu_baseline(torch, 0)
+        result["cpu_baseline"] = cpu_baseline(torch, 0, extra=not args.no_extra)
     print(json.dumps(result), flush=True)
 
 
