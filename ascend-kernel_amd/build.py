@@ -157,18 +157,6 @@ def _check_accumulator_moves(src: str) -> None:
                     continue
                 if any(r in accs for r in regs(parts[1])):
                     raise RuntimeError(f"{src}: {m.group(1)} touches an accumulator right behind its MFMA: {nxt}")
-        # LDS reads issued from inline asm (the transposing reads): the compiler believes their result is
-        # there at once, so nothing may name the destination registers before the asm wait that follows
-        for i, l in enumerate(code):
-            if not l.startswith("ds_read_b64_tr_b4"):
-                continue
-            dst = set(regs(l.split(None, 1)[1].split(",")[0]))
-            for nxt in code[i + 1:]:
-                if nxt.startswith("s_waitcnt") and "lgkmcnt(0)" in nxt:
-                    break
-                parts = nxt.split(None, 1)
-                if len(parts) == 2 and any(r in dst for r in regs(parts[1])):
-                    raise RuntimeError(f"{src}: {m.group(1)} names the result of an asm LDS read in flight: {nxt}")
 
 
 def _wait(procs):

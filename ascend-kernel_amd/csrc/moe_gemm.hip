@@ -97,16 +97,6 @@ __device__ __forceinline__ V pinned(V v) {
     return v;
 }
 
-// Compile-time loop: f(std::integral_constant<int, B>{}) ... f(std::integral_constant<int, E - 1>{}).  Used where
-// every index must be a constant at instantiation time (register arrays, instruction placement).
-template <int B, int E, typename F>
-__device__ __forceinline__ void static_for(F&& f) {
-    if constexpr (B < E) {
-        f(std::integral_constant<int, B>{});
-        static_for<B + 1, E>(f);
-    }
-}
-
 // Per-lane view of one tile for the weight loaders.
 struct BCtx {
     rsrc_t rw, rs;       // weight / scale slab of the expert
@@ -412,71 +402,45 @@ constexpr int pair_lds_units() {
     return pair_stages<FMT>() * (PAIR_A_UNITS + pair_b_units<FMT>() + pair_sc_units<FMT>()) + pair_kc_scale_units<FMT>();
 }
 
-// End of a k-split tile: the partial sums of wavefront wv + 4 (h == 1) are added to those of wv through LDS
-// and the h == 0 wavefronts store the tile (plain, K-contiguous column order, or with the fused activation).
+// End of a k-split tile.  The two wavefronts of a pair (same columns, the two k halves) hold partial sums of the
+// whole tile; each hands the row blocks the other will finish to it through LDS, adds what it receives to the
+// row blocks it keeps and stores those: the first half of the tile's 16-row blocks is finished by the h == 0
+// wavefront, the second by h == 1, so both reduce and store at the same time.  Rounds of at most 4 row
+// blocks (8 wavefronts x 4 blocks x 4 KB fit the x stage area, free now).
 template <int MT, bool KC>
 __device__ __forceinline__ void pair_finish(const GemmParams& P, u32x4_t* smem, f32x4_t (&acc)[MT][4], int h, int cw, int lane,
                                             int col0, int64_t row0, int rows, int n0) {
     const int i = lane & 15, q = lane >> 4;
-    // two row blocks per round, through two alternating LDS buffers (in the x stage area, free now)
-    constexpr int RB = 2, ROUNDS = (MT + RB - 1) / RB;
-    u32x4_t* red = smem;   // [2 buffers][4 column groups][RB * 4 fragments][64 lanes]
-    auto red_unit = [&](int buf, int k) { return ((buf * 4 + cw) * (RB * 4) + k) * 64 + lane; };
-#pragma unroll
-    for (int rd = 0; rd <= ROUNDS; ++rd) {
-        if (h == 1 && rd < ROUNDS) {
-#pragma unroll
-            for (int b = 0; b < RB; ++b)
-#pragma unroll
-                for (int t = 0; t < 4; ++t)
-                    if (rd * RB + b < MT) red[red_unit(rd & 1, b * 4 + t)] = __builtin_bit_cast(u32x4_t, acc[rd * RB + b][t]);
-        }
-        if (h == 0 && rd > 0) {
-#pragma unroll
-            for (int b = 0; b < RB; ++b)
-#pragma unroll
-                for (int t = 0; t < 4; ++t)
-                    if ((rd - 1) * RB + b < MT)
-                        acc[(rd - 1) * RB + b][t] += __builtin_bit_cast(f32x4_t, red[red_unit((rd - 1) & 1, b * 4 + t)]);
-        }
-        if (rd < ROUNDS) __syncthreads();
-    }
-
+    constexpr int RR = 4, MH = (MT + 1) / 2, ROUNDS = (MH + RR - 1) / RR;
     // the last tile of an N that is not a multiple of 256 (the reference's fp8 container: multiples of 128)
     // computes columns past N from whatever follows in the slab: they are not stored
     const bool live = KC || n0 + col0 < P.N;
-    if (!live) {
-    } else if (h == 0 && P.epilogue == MOE_EPILOGUE_SWIGLU) {
-        // this lane's 4 columns are (gate, gate, up, up) of 2 output columns; y has N / 2 columns
-        const int NO = P.N >> 1;
-        const rsrc_t ro = make_rsrc(P.y + row0 * (int64_t)NO, (int64_t)rows * NO * 2);
-        const int vo = (4 * q * NO + ((n0 + col0) >> 1)) * 2;
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt)
+    const bool swi = P.epilogue == MOE_EPILOGUE_SWIGLU;
+    // stores go through a buffer resource that ends after the tile's last valid row: those to padded rows
+    // fall outside it and are dropped
+    const int NO = swi ? P.N >> 1 : P.N;
+    const rsrc_t ry = make_rsrc(P.y + row0 * (int64_t)NO, (int64_t)rows * NO * 2);
+    auto store_block = [&](int mt) {
+        if (!live) return;
+        if (swi) {
+            // this lane's 4 columns are (gate, gate, up, up) of 2 output columns; y has N / 2 columns
+            const int vo = (4 * q * NO + ((n0 + col0) >> 1)) * 2;
 #pragma unroll
             for (int r = 0; r < 4; ++r)
                 __builtin_amdgcn_raw_buffer_store_b32(
-                    pack_bf16_rne(swiglu(acc[mt][0][r], acc[mt][2][r]), swiglu(acc[mt][1][r], acc[mt][3][r])), ro, vo,
+                    pack_bf16_rne(swiglu(acc[mt][0][r], acc[mt][2][r]), swiglu(acc[mt][1][r], acc[mt][3][r])), ry, vo,
                     (16 * mt + r) * NO * 2, 0);
-    } else if (h == 0 && KC) {
-        // K-contiguous containers: MFMA t holds column 64 cw + 16 t + i, one 2-byte store each
-        const rsrc_t ry = make_rsrc(P.y + row0 * (int64_t)P.N, (int64_t)rows * P.N * 2);
-        const int vy = (4 * q * P.N + n0 + 64 * cw + i) * 2;
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt)
+        } else if (KC) {
+            // K-contiguous containers: MFMA t holds column 64 cw + 16 t + i, one 2-byte store each
+            const int vy = (4 * q * P.N + n0 + 64 * cw + i) * 2;
 #pragma unroll
             for (int r = 0; r < 4; ++r)
 #pragma unroll
                 for (int t = 0; t < 4; ++t)
                     __builtin_amdgcn_raw_buffer_store_b16((uint16_t)(pack_bf16_rne(acc[mt][t][r], 0.f) & 0xffffu), ry,
                                                           vy + 32 * t, (16 * mt + r) * P.N * 2, 0);
-    } else if (h == 0) {
-        // epilogue through a buffer resource that ends after the tile's last valid row: stores to
-        // padded rows fall outside it and are dropped
-        const rsrc_t ry = make_rsrc(P.y + row0 * (int64_t)P.N, (int64_t)rows * P.N * 2);
-        const int vy = (4 * q * P.N + n0 + col0) * 2;
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt)
+        } else {
+            const int vy = (4 * q * P.N + n0 + col0) * 2;
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 u32x2_t v;
@@ -484,8 +448,37 @@ __device__ __forceinline__ void pair_finish(const GemmParams& P, u32x4_t* smem, 
                 v[1] = pack_bf16_rne(acc[mt][2][r], acc[mt][3][r]);
                 __builtin_amdgcn_raw_buffer_store_b64(v, ry, vy, (16 * mt + r) * P.N * 2, 0);
             }
-    }
-    __syncthreads();   // the reduction buffers are read: the next tile may load into the ring
+        }
+    };
+    // H: which half this wavefront finishes (a compile-time constant in each branch, so that every register
+    // index is one); both kinds of wavefront take the same barriers
+    auto finish = [&](auto HC) __attribute__((always_inline)) {
+        constexpr int H = decltype(HC)::value;
+        constexpr int KEEP0 = H == 0 ? 0 : MH, KEEPN = H == 0 ? MH : MT - MH;
+        constexpr int SEND0 = H == 0 ? MH : 0, SENDN = MT - KEEPN;
+        u32x4_t* out_slot = smem + (cw * 2 + (1 - H)) * (RR * 4 * 64) + lane;
+        const u32x4_t* in_slot = smem + (cw * 2 + H) * (RR * 4 * 64) + lane;
+#pragma unroll
+        for (int rd = 0; rd < ROUNDS; ++rd) {
+            if (rd > 0) __syncthreads();   // the previous round's slots are read
+#pragma unroll
+            for (int b = rd * RR; b < (rd + 1) * RR && b < SENDN; ++b)
+#pragma unroll
+                for (int t = 0; t < 4; ++t) out_slot[((b - rd * RR) * 4 + t) * 64] = __builtin_bit_cast(u32x4_t, acc[SEND0 + b][t]);
+            __syncthreads();
+#pragma unroll
+            for (int b = rd * RR; b < (rd + 1) * RR && b < KEEPN; ++b) {
+#pragma unroll
+                for (int t = 0; t < 4; ++t) acc[KEEP0 + b][t] += __builtin_bit_cast(f32x4_t, in_slot[((b - rd * RR) * 4 + t) * 64]);
+                store_block(KEEP0 + b);
+            }
+        }
+    };
+    if (h == 0)
+        finish(std::integral_constant<int, 0>{});
+    else
+        finish(std::integral_constant<int, 1>{});
+    __syncthreads();   // the slots are read: the next tile may load into the ring
 }
 
 // EXACT selects the arithmetic of the GEMV op (grouped_soft_gemv/op_kernel/gemv_impl.h:147-199: the
@@ -935,276 +928,6 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
 }
 
 // ---------------------------------------------------------------------------------
-// int4 prefill tile routine on v_mfma_f32_32x32x16_bf16: the k-split pair of gemm_tile_pair with half as many
-// matrix instructions per flop.  A SIMD issues MFMAs and ordinary vector instructions through one port
-// (measured: about 8 cycles per MFMA of either shape, 4-5 per vector instruction), and the int4 decode alone
-// needs 2.5 vector instructions per weight; the 16x16x32 routine therefore spends as much issue time as
-// matrix-pipe time.  The 32x32x16 shape does the same flops with half the MFMA issue slots.
-//
-//  * A wavefront (cw, h) still owns 64 columns and one 32-k half of every 64-k step.  Its 64 columns are two
-//    32-column blocks cb, its 32 k two MFMA steps kb of 16.  Lane l = 32 hi + c supplies, for (cb, kb),
-//    column 64 cw + 32 cb + c and k = 32 h + 16 hi + 8 kb + [0, 8).
-//  * Those 16 codes of one column are 16 different rows of the packed tile (a row holds one k, 2 columns per
-//    byte).  ds_read_b64_tr_b4 does the transposition: the 16 lanes of a group each address 8 bytes of one
-//    row (16 adjacent columns), and lane r of the group receives nibble r of all 16 rows -- two reads per
-//    lane and step, each dword 8 consecutive k of one column.
-//  * The operands are swapped (weights as the MFMA's first matrix, x as its second), so that a lane's 16
-//    accumulators of a block are 4 runs of 4 consecutive output columns of ONE row (row 32 rb + c, columns
-//    64 cw + 32 cb + 8 j + 4 hi + [0, 4)): the epilogue packs each run into one 8-byte store, and a run is
-//    exactly one (gate, gate, up, up) group of the fused activation.
-//  * Row blocks are 32 rows: a tile of mt 16-row blocks runs RB = ceil(mt / 2) of them.
-//  * End of tile: wavefront (cw, h) hands the partial sums of column block 1 - h to its partner through
-//    LDS, adds what it receives to column block h and stores that block: both wavefronts of a pair reduce
-//    and store half of the tile each.
-// Stages, loads and the phase scheme (decode phase, MFMA phase, barrier placement) are those of gemm_tile_pair.
-// ---------------------------------------------------------------------------------
-typedef float f32x16_t __attribute__((ext_vector_type(16)));
-
-__device__ __forceinline__ void mfma_32x32x16_v(f32x16_t& acc, const u32x4_t& a, const u32x4_t& b) {
-    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(acc) : "v"(a), "v"(b));
-}
-
-constexpr int PAIR32_RB_MAX = PAIR_CAPB / 2;   // 32-row blocks per tile
-
-template <int RB>
-__device__ __forceinline__ void gemm_tile_pair32(const GemmParams& P, u32x4_t* smem, int g, int64_t row0, int rows, int n0) {
-    constexpr int FMT = MOE_FMT_INT4;
-    constexpr int BK = 64, S = pair_stages<FMT>(), PAIR_SC_UNITS = pair_sc_units<FMT>(), PAIR_B_UNITS = pair_b_units<FMT>();
-    constexpr int AHEAD = S - 1;
-    constexpr int MT = 2 * RB;   // 16-row blocks the x loads cover
-    static_assert(RB >= 1 && RB <= PAIR32_RB_MAX, "row blocks beyond the x stage");
-    u32x4_t* lds_a = smem;
-    u32x4_t* lds_b = lds_a + S * PAIR_A_UNITS;
-    u32x4_t* lds_s = lds_b + S * PAIR_B_UNITS;
-
-    const int tid = threadIdx.x, lane = tid & 63;
-    const int c = lane & 31, hi = lane >> 5;
-    const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int cw = wv & 3;
-    const int h = 1 - (wv >> 2);   // see gemm_tile_pair
-    const int nk = P.K / BK;
-
-    const int64_t KN = (int64_t)P.K * P.N;
-    const rsrc_t rw = make_rsrc(P.w + g * (KN >> 1), KN >> 1);
-    const rsrc_t rs = make_rsrc(static_cast<const uint16_t*>(P.scale) + (int64_t)g * P.scale_rows * P.N,
-                                (int64_t)P.scale_rows * P.N * 2);
-    const uint32_t per = (uint32_t)((P.K / P.scale_rows) >> 5);
-    const uint32_t gmul = per == 1 ? 0u : 0xffffffffu / per + 1u;
-    auto scale_row = [&](uint32_t sub) { return gmul ? (int)__umulhi(sub, gmul) : (int)sub; };
-    const rsrc_t rx = make_rsrc(P.x + row0 * (int64_t)P.K, (int64_t)rows * P.K * 2);
-    const int va = ((lane >> 3) * P.K + (((lane & 7) ^ (lane >> 3)) * 8)) * 2;
-    // packed tile: instruction wv brings rows 8 wv + (lane >> 3); position lane & 7 of a row holds its
-    // 16-byte chunk (lane & 7) ^ (row & 7), which spreads the 16 rows a transposing read touches over the banks
-    const int vb = (lane >> 3) * (P.N >> 1) + (((lane & 7) ^ (lane >> 3)) * 16);
-    constexpr int NA = (2 * MT + 7) / 8, NI = NA + 2;
-    int ja[NA], ca[NA];
-#pragma unroll
-    for (int m = 0; m < NA; ++m) {
-        int j = wv + 8 * m;
-        if (8 * NA > 2 * MT) j = j % (2 * MT);
-        ja[m] = j * 64;
-        ca[m] = 8 * j * P.K * 2;
-    }
-    const int cb0 = 8 * wv * (P.N >> 1) + (n0 >> 1);
-    const int kb_step = BK * (P.N >> 1);
-    const int cs = n0 * 2 + (wv & 3) * 128;
-    const int lane16 = lane * 16;
-    const bool s_lane = lane < 8;
-    auto issue = [&](int m, int kt, int ST) {
-        if (m < NA) {
-            lds_load16(rx, lds_a + ST * PAIR_A_UNITS + ja[m], va, ca[m] + (kt + AHEAD) * (BK * 2));
-        } else if (m == NA) {
-            lds_load16(rw, lds_b + ST * PAIR_B_UNITS + wv * (PAIR_B_UNITS / 8), vb, cb0 + (kt + AHEAD) * kb_step);
-        } else {
-            const int grow = scale_row((uint32_t)((kt + AHEAD) * 2 + (wv >> 2)));
-            if (s_lane) lds_load16(rs, lds_s + ST * PAIR_SC_UNITS + wv * (PAIR_SC_UNITS / 8), lane16, grow * (P.N * 2) + cs);
-        }
-    };
-
-    uint32_t mask = 0x0f0f0f0fu;
-    asm volatile("" : "+s"(mask));   // kept opaque so that it stays one SGPR operand
-    // byte offsets inside a stage.  Transposing read of column block cb: row 32 h + 16 hi + r (r = lane & 15),
-    // chunk 2 cw + cb at position chunk ^ (row & 7), half (lane >> 4) & 1 of the chunk
-    const int r16 = lane & 15;
-    const int tr_off = (32 * h + 16 * hi + r16) * 128 + (((2 * cw) ^ (r16 & 7)) * 16) + 8 * ((lane >> 4) & 1);
-    const int tr_d1 = (r16 & 1) ? -16 : 16;   // column block 1: chunk 2 cw + 1, the neighbouring position
-    // scales of the wavefront's sub-step: row h of the stage's two, columns 64 cw + 32 cb + c
-    const int sc_off = (256 * h + 64 * cw + c) * 2;
-    // x fragment of (rb, kb): row 32 rb + c, chunk 4 h + 2 hi + kb
-    const int a_unit = c * 8 + ((4 * h + 2 * hi) ^ (c & 7));
-
-    f32x16_t acc[RB][2];
-#pragma unroll
-    for (int rb = 0; rb < RB; ++rb)
-#pragma unroll
-        for (int cb = 0; cb < 2; ++cb)
-#pragma unroll
-            for (int e = 0; e < 16; e += 4)
-                asm volatile("v_mov_b32 %0, 0\n\tv_mov_b32 %1, 0\n\tv_mov_b32 %2, 0\n\tv_mov_b32 %3, 0"
-                             : "=v"(acc[rb][cb][e]), "=v"(acc[rb][cb][e + 1]), "=v"(acc[rb][cb][e + 2]), "=v"(acc[rb][cb][e + 3]));
-    u32x4_t bf[2][2], afr[4];
-    constexpr int F = 2 * RB;                 // x fragments per step: (rb, kb)
-    constexpr int R = 3 < F ? 3 : F;          // read ahead of their MFMAs
-
-    constexpr int WAITN = (S - 3) * NI;
-#pragma unroll
-    for (int st0 = 0; st0 < AHEAD; ++st0)
-#pragma unroll
-        for (int m = 0; m < NI; ++m) issue(m, st0 - AHEAD, st0);
-    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(WAITN) : "memory");
-
-    // this lane's packed codes (d[cb][kb]: 8 consecutive k of one column) and scales of LDS stage st
-    // (the transposing reads are written as asm: given the builtin, the compiler cannot tell them from the
-    // LDS-direct loads in flight and waits for all of those first; the decode phase waits for the reads itself)
-    u32x2_t d[2];
-    uint32_t sraw[2];
-    auto read_raw = [&](int st) {
-        const char* tb = reinterpret_cast<const char*>(lds_b + st * PAIR_B_UNITS) + tr_off;
-        asm volatile("ds_read_b64_tr_b4 %0, %1" : "=v"(d[0]) : "v"((uint32_t)(size_t)MOE_LDS_PTR(tb)));
-        asm volatile("ds_read_b64_tr_b4 %0, %1" : "=v"(d[1]) : "v"((uint32_t)(size_t)MOE_LDS_PTR(tb + tr_d1)));
-        const uint16_t* sp = reinterpret_cast<const uint16_t*>(reinterpret_cast<const char*>(lds_s + st * PAIR_SC_UNITS) + sc_off);
-        sraw[0] = sp[0];
-        sraw[1] = sp[32];
-    };
-    // the asm reads have landed (placed where every LDS read of the phase has been waited for anyway, and
-    // before the loop's back edge: no copy of d may be made while a read is in flight)
-    auto raw_landed = [&]() { asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(d[0]), "+v"(d[1])); };
-    read_raw(0);
-    raw_landed();
-
-    auto a_read = [&](const u32x4_t* la, int f) { afr[f & 3] = la[(a_unit ^ (f & 1)) + (f >> 1) * 256]; };
-
-    auto step = [&](int kt, int st, int sn, int sl) {
-        const u32x4_t* la = lds_a + st * PAIR_A_UNITS;
-        // ---- decode phase: d[cb][kb] -> bf[cb][kb]; W = RNE_bf16((q - 8) s) as q' (512 s) - 8 s with q' = q / 512
-        // from the e4m3 reading of the nibble (see gemm_tile_pair)
-#pragma unroll
-        for (int cb = 0; cb < 2; ++cb) {
-            if (cb == 1) {
-                if (h == 1) {
-                    if (kt > 0) asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(WAITN) : "memory");
-                }
-#pragma unroll
-                for (int f = 0; f < R; ++f) a_read(la, f);
-            }
-            const float s = __uint_as_float(sraw[cb] << 16);
-            const float m = s * 512.f, z = -8.f * s;
-            uint32_t lo[2], hn[2];
-            f32x2_t e0[2], e1[2], o0[2], o1[2];
-#pragma unroll
-            for (int kb = 0; kb < 2; ++kb) { lo[kb] = d[cb][kb] & mask; hn[kb] = d[cb][kb] >> 4; }
-            __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for (int kb = 0; kb < 2; ++kb) {
-                hn[kb] &= mask;
-                e0[kb] = __builtin_amdgcn_cvt_pk_f32_fp8(lo[kb], false);   // k0 k2
-                e1[kb] = __builtin_amdgcn_cvt_pk_f32_fp8(lo[kb], true);    // k4 k6
-            }
-            __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for (int kb = 0; kb < 2; ++kb) {
-                o0[kb] = __builtin_amdgcn_cvt_pk_f32_fp8(hn[kb], false);   // k1 k3
-                o1[kb] = __builtin_amdgcn_cvt_pk_f32_fp8(hn[kb], true);    // k5 k7
-            }
-            float w[2][8];
-#pragma unroll
-            for (int kb = 0; kb < 2; ++kb) {
-                w[kb][0] = fmaf(e0[kb][0], m, z); w[kb][2] = fmaf(e0[kb][1], m, z);
-                w[kb][4] = fmaf(e1[kb][0], m, z); w[kb][6] = fmaf(e1[kb][1], m, z);
-            }
-            __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for (int kb = 0; kb < 2; ++kb) {
-                w[kb][1] = fmaf(o0[kb][0], m, z); w[kb][3] = fmaf(o0[kb][1], m, z);
-                w[kb][5] = fmaf(o1[kb][0], m, z); w[kb][7] = fmaf(o1[kb][1], m, z);
-            }
-            __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-                for (int p = 0; p < 4; ++p) bf[cb][kb][p] = pack_bf16_rne(w[kb][2 * p], w[kb][2 * p + 1]);
-            __builtin_amdgcn_sched_barrier(0);
-        }
-        // ---- MFMA phase (raised priority, see gemm_tile_pair): this step's loads and the packed codes of the
-        // next step are fetched between the MFMAs
-        __builtin_amdgcn_s_setprio(3);
-#pragma unroll
-        for (int f = 0; f < F; ++f) {
-            const int rb = f >> 1, kb = f & 1;
-            if (f + R < F) a_read(la, f + R);
-            mfma_32x32x16_v(acc[rb][0], bf[0][kb], afr[f & 3]);
-            mfma_32x32x16_v(acc[rb][1], bf[1][kb], afr[f & 3]);
-#pragma unroll
-            for (int m = (f * NI + F - 1) / F; m < ((f + 1) * NI + F - 1) / F; ++m) issue(m, kt, sl);
-            if (f == 0) read_raw(sn);
-            __builtin_amdgcn_sched_barrier(0);
-        }
-        __builtin_amdgcn_s_setprio(0);
-        raw_landed();
-        if (h == 0) asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(WAITN) : "memory");   // barrier kt
-    };
-    for (int kt = 0, st = 0, sl = S - 1; kt < nk; ++kt) {
-        const int sn = st == S - 1 ? 0 : st + 1;
-        step(kt, st, sn, sl);
-        st = sn;
-        sl = sl == S - 1 ? 0 : sl + 1;
-    }
-    if (h == 1) asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(WAITN) : "memory");       // barrier nk-1
-    // drain this wavefront's loads (they target stages past K and are never read); the accumulators were
-    // last written by MFMAs the compiler cannot see: wait out their latency
-    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_nop 15\n\ts_nop 15\n\ts_nop 15\n\ts_nop 15\n\ts_barrier" ::: "memory");
-
-    // ---- exchange and store.  Rounds of at most 4 row blocks (8 wavefronts x 4 blocks x 4 KB fill the stage
-    // area); slot (cw, h) of a round receives what wavefront (cw, h) adds to its column block h.
-    constexpr int RR = 4, ROUNDS = (RB + RR - 1) / RR;
-    auto finish = [&](auto HC) __attribute__((always_inline)) {
-        constexpr int H = decltype(HC)::value;
-        u32x4_t* out_slot = smem + (cw * 2 + (1 - H)) * (RR * 4 * 64) + lane;
-        const u32x4_t* in_slot = smem + (cw * 2 + H) * (RR * 4 * 64) + lane;
-        const int ncol = n0 + 64 * cw + 32 * H + 4 * hi;    // first of this lane's 4-column runs (8 columns apart)
-        const bool swi = P.epilogue == MOE_EPILOGUE_SWIGLU;
-        const int NO = swi ? P.N >> 1 : P.N;
-        const rsrc_t ry = make_rsrc(P.y + row0 * (int64_t)NO, (int64_t)rows * NO * 2);
-        const int vy = (c * NO + (swi ? ncol >> 1 : ncol)) * 2;
-#pragma unroll
-        for (int rd = 0; rd < ROUNDS; ++rd) {
-            if (rd > 0) __syncthreads();   // the previous round's slots are read
-#pragma unroll
-            for (int rb = rd * RR; rb < (rd + 1) * RR && rb < RB; ++rb)
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const f32x4_t v = {acc[rb][1 - H][4 * j], acc[rb][1 - H][4 * j + 1], acc[rb][1 - H][4 * j + 2], acc[rb][1 - H][4 * j + 3]};
-                    out_slot[((rb - rd * RR) * 4 + j) * 64] = __builtin_bit_cast(u32x4_t, v);
-                }
-            __syncthreads();
-#pragma unroll
-            for (int rb = rd * RR; rb < (rd + 1) * RR && rb < RB; ++rb)
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const f32x4_t o = __builtin_bit_cast(f32x4_t, in_slot[((rb - rd * RR) * 4 + j) * 64]);
-                    const float y0 = acc[rb][H][4 * j] + o[0], y1 = acc[rb][H][4 * j + 1] + o[1];
-                    const float y2 = acc[rb][H][4 * j + 2] + o[2], y3 = acc[rb][H][4 * j + 3] + o[3];
-                    if (swi) {
-                        // (gate, gate, up, up) -> 2 output columns
-                        __builtin_amdgcn_raw_buffer_store_b32(pack_bf16_rne(swiglu(y0, y2), swiglu(y1, y3)), ry, vy + 8 * j,
-                                                              32 * rb * NO * 2, 0);
-                    } else {
-                        u32x2_t v;
-                        v[0] = pack_bf16_rne(y0, y1);
-                        v[1] = pack_bf16_rne(y2, y3);
-                        __builtin_amdgcn_raw_buffer_store_b64(v, ry, vy + 16 * j, 32 * rb * NO * 2, 0);
-                    }
-                }
-        }
-    };
-    if (h == 0)
-        finish(std::integral_constant<int, 0>{});
-    else
-        finish(std::integral_constant<int, 1>{});
-    __syncthreads();   // the slots are read: the next tile may load into the ring
-}
-
-// ---------------------------------------------------------------------------------
 // Tile scheduler (role of GMMAntiquantProcess::Process,
 // grouped_gemm/op_kernel/grouped_matmul_antiquant.h:241-288).  Expert g with m_g rows
 // has ceil(m_g/16) row blocks, cut into the fewest chunks of <= MT_MAX blocks, as
@@ -1226,11 +949,6 @@ __device__ __forceinline__ void expert_chunks(int m, int& chunks, int& bpc) {
 //   GK_PAIR_EXACT  GK_PAIR with the GEMV op's arithmetic (weights not rounded to bf16), tiles of at most 32 rows
 enum { GK_GENERAL = 0, GK_SKINNY = 1, GK_PAIR = 2, GK_PAIR_EXACT = 3 };
 constexpr int PAIR_EXACT_MT_MAX = 2;
-// int4 tiles of at least this many 16-row blocks run on the 32x32x16 routine (smaller ones would pad a lone
-// 16-row block to 32 rows for nothing: they are HBM bound)
-#ifndef MOE_PAIR32_MT_MIN
-#define MOE_PAIR32_MT_MIN 3
-#endif
 
 template <int FMT, int KIND>
 struct KernelCfg {
@@ -1260,10 +978,7 @@ struct KernelCfg {
 template <int FMT, int MT, int KIND>
 __device__ __forceinline__ void run_tile(const GemmParams& P, u32x4_t* smem, int g, int64_t row0, int rows, int n0) {
     using C = KernelCfg<FMT, KIND>;
-    if constexpr (KIND == GK_PAIR && FMT == MOE_FMT_INT4 && MT >= MOE_PAIR32_MT_MIN) {
-        // the scheduler rounds these tiles up to whole 32-row blocks: odd counts are never dispatched
-        if constexpr ((MT & 1) == 0) gemm_tile_pair32<MT / 2>(P, smem, g, row0, rows, n0);
-    } else if constexpr (C::PAIR)
+    if constexpr (C::PAIR)
         gemm_tile_pair<FMT, MT, KIND == GK_PAIR_EXACT>(P, smem, g, row0, rows, n0);
     else
         gemm_tile<FMT, MT, C::CAPB>(P, smem, g, row0, rows, n0);
@@ -1338,9 +1053,7 @@ __global__ __launch_bounds__((64 * KernelCfg<FMT, KIND>::WAVES), (KernelCfg<FMT,
         const int chunk = local / ntile_n, nt = local % ntile_n;
         const int rbeg = chunk * bpc * 16;
         const int rows = min(m - rbeg, bpc * 16);
-        int mt = (rows + 15) >> 4;
-        if constexpr (KIND == GK_PAIR && FMT == MOE_FMT_INT4)
-            if (mt >= MOE_PAIR32_MT_MIN) mt = (mt + 1) & ~1;   // 32-row blocks (gemm_tile_pair32)
+        const int mt = (rows + 15) >> 4;
         const int rlo = __builtin_amdgcn_readfirstlane((int)(uint32_t)(gbeg & 0xffffffffLL));
         const int rhi = __builtin_amdgcn_readfirstlane((int)(gbeg >> 32));
         const int64_t row0 = (((int64_t)rhi << 32) | (uint32_t)rlo) + rbeg;
