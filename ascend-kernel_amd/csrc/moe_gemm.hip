@@ -580,7 +580,10 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
     // m-th load of group kt (stage kt+AHEAD of x, packed tile and scales), into LDS stage ST
     auto issue = [&](int m, int kt, int ST) {
         if (m < NA) {
-            lds_load16(rx, lds_a + ST * PAIR_A_UNITS + ja[m], va, ca[m] + (kt + AHEAD) * (BK * 2));
+            // past K a row's next bytes are the following row's (valid memory, real traffic): the loads of the last
+            // AHEAD steps are sent beyond the end of the resource instead, where they cost nothing and return 0
+            const int koff = kt + AHEAD < nk ? (kt + AHEAD) * (BK * 2) : 0x7ff00000;
+            lds_load16(rx, lds_a + ST * PAIR_A_UNITS + ja[m], va, ca[m] + koff);
         } else if (m < NA + NB) {
             const int e = m - NA;
             lds_load16(rw, lds_b + ST * PAIR_B_UNITS + wv * (PAIR_B_UNITS / 8) + e * 64, vb,
@@ -1050,7 +1053,9 @@ __global__ __launch_bounds__((64 * KernelCfg<FMT, KIND>::WAVES), (KernelCfg<FMT,
         int chunks, bpc;
         expert_chunks<MTM>(m, chunks, bpc);
         const int local = __builtin_amdgcn_readfirstlane(T - prefix[g]);
-        const int chunk = local / ntile_n, nt = local % ntile_n;
+        // row chunks innermost: the tiles that share a weight column tile are neighbours in the order, run at
+        // the same time on one XCD and pull that slice of the expert's weights into its L2 once
+        const int nt = local / chunks, chunk = local % chunks;
         const int rbeg = chunk * bpc * 16;
         const int rows = min(m - rbeg, bpc * 16);
         const int mt = (rows + 15) >> 4;
