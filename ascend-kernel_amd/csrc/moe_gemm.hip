@@ -607,7 +607,10 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
 
     // perm selector: bytes 2hh, 2hh+1 of row a, then of row b (hh = half of the dword this lane owns)
     const uint32_t h2 = 2u * (uint32_t)(cw & 1);
-    uint32_t sel = h2 | ((h2 + 1u) << 8) | ((4u + h2) << 16) | ((5u + h2) << 24);
+    // (int4 with the GEMV op's arithmetic: row a and row b interleaved, so that a 16-bit word holds a k pair)
+    constexpr bool I4X = EXACT && FMT == MOE_FMT_INT4;
+    uint32_t sel = I4X ? h2 | ((4u + h2) << 8) | ((h2 + 1u) << 16) | ((5u + h2) << 24)
+                       : h2 | ((h2 + 1u) << 8) | ((4u + h2) << 16) | ((5u + h2) << 24);
     uint32_t mask = 0x0f0f0f0fu;
     asm volatile("" : "+s"(mask), "+s"(sel));   // kept opaque so that each stays one SGPR operand
     const int d = 16 * (cw >> 1) + i;            // dword column of this lane
@@ -832,6 +835,21 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
             }
 #pragma unroll
             for (int p = 0; p < 2; ++p) { lo[p] = pr[p] & mask; hi[p] = pr[p] >> 4; }
+            if constexpr (I4X) {
+                // The codes themselves as bf16, two at a time: a nibble read as e4m3 is q / 512, and the scaled
+                // convert (scale 2^9: only the exponent of that operand counts) yields the bf16 pair (q_a, q_b) of
+                // one column.  The zero point is taken off in the MFMA phase.
+#pragma unroll
+                for (int p = 0; p < 2; ++p) {
+                    hi[p] &= mask;
+                    bf[0][p0 + p] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(lo[p], 512.f, false));
+                    bf[2][p0 + p] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(lo[p], 512.f, true));
+                    bf[1][p0 + p] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(hi[p], 512.f, false));
+                    bf[3][p0 + p] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(hi[p], 512.f, true));
+                }
+                __builtin_amdgcn_sched_barrier(0);
+                continue;
+            }
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int p = 0; p < 2; ++p) {
@@ -896,10 +914,18 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
                         for (int e = 0; e < 4; ++e) acc[mt][t][e] = fmaf(dhi[e], sb[t], fmaf(dlo[e], sa[t], acc[mt][t][e]));
                     }
                 } else {
+                    // int4: the fragments hold q, not q - 8: each product starts from -8 sum_k x[m][k] (one more
+                    // MFMA per x fragment, against a constant fragment of -8.0), so dd = sum_k x (q - 8)
+                    f32x4_t start = zero;
+                    if constexpr (I4X) {
+                        const u32x4_t m8 = {0xc100c100u, 0xc100c100u, 0xc100c100u, 0xc100c100u};
+                        start = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                            __builtin_bit_cast(bf16x8_t, afr[mt & 3]), __builtin_bit_cast(bf16x8_t, m8), zero, 0, 0, 0);
+                    }
 #pragma unroll
                     for (int t = 0; t < 4; ++t) {
                         const f32x4_t dd = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-                            __builtin_bit_cast(bf16x8_t, afr[mt & 3]), __builtin_bit_cast(bf16x8_t, bf[t]), zero, 0, 0, 0);
+                            __builtin_bit_cast(bf16x8_t, afr[mt & 3]), __builtin_bit_cast(bf16x8_t, bf[t]), start, 0, 0, 0);
 #pragma unroll
                         for (int e = 0; e < 4; ++e) acc[mt][t][e] = fmaf(dd[e], sa[t], acc[mt][t][e]);
                     }
