@@ -7,11 +7,11 @@
 // Order of the sorted rows: by expert id, then by flat choice index t * topk + j (a stable sort), so
 // the result is deterministic and independent of the launch geometry.
 //
-//   route_topk_kernel    one wavefront per token: softmax statistics and top-k by repeated arg-max
-//   route_count_kernel   per 1024-choice block, a histogram over experts (LDS atomics)
-//   route_scan_kernel    one workgroup: per expert, prefix over the blocks; then over experts
-//   route_rank_kernel    per block, every choice's rank among the earlier choices of its expert
-//   route_gather_kernel  x rows copied into sorted order, 16 bytes per lane
+//   route_topk_kernel     one wavefront per token: softmax statistics and top-k by repeated arg-max
+//   route_count_kernel    per 1024-choice block, a histogram over experts (LDS atomics)
+//   route_rank_kernel     per block: prefix of the counts over experts and earlier blocks (group_list), then every
+//                         choice's rank among the earlier choices of its expert -> its sorted row
+//   route_scatter_kernel  a token's x row read once and written to the sorted row of each of its choices
 #include <atomic>
 
 #include "moe_device.h"
@@ -84,82 +84,111 @@ __global__ __launch_bounds__(RT_BLOCK) void route_count_kernel(const int32_t* __
     for (int e = threadIdx.x; e < E; e += RT_BLOCK) block_counts[(int64_t)blockIdx.x * E + e] = hist[e];
 }
 
-// block_counts[b][e] -> block_base[b][e] = first sorted row of block b's choices of expert e;
-// group_list[e] = rows of experts <= e.  Input and output are separate arrays so that the loads of
-// a thread's column do not have to wait for its stores.
-__global__ __launch_bounds__(RT_MAX_E) void route_scan_kernel(const int32_t* __restrict__ block_counts,
-                                                              int32_t* __restrict__ block_base,
-                                                              int64_t* __restrict__ group_list, int nblocks, int E) {
-    __shared__ int scan[RT_MAX_E];
-    const int e = threadIdx.x;
-    int total = 0;
-    if (e < E)
-        for (int b = 0; b < nblocks; ++b) total += block_counts[(int64_t)b * E + e];
-    scan[e] = e < E ? total : 0;
+// Rank of every choice of block b among the choices of its expert, and with it the sorted row:
+//   row = (choices of lower experts) + (choices of this expert in earlier blocks) + (in earlier wavefronts of
+//         this block) + (in lower lanes of this wavefront)
+// Every block derives the first two terms from the per-block counts itself (nblocks x E integers: cheaper than
+// a kernel of its own for the scan); block 0 also writes group_list.  The third comes from per-wavefront
+// histograms in LDS, the fourth from comparing with the lanes below.  Dynamic LDS: (16 + 2) * E integers.
+__global__ __launch_bounds__(RT_BLOCK) void route_rank_kernel(const int32_t* __restrict__ ids, const int32_t* __restrict__ block_counts,
+                                                              int64_t* __restrict__ group_list,
+                                                              int32_t* __restrict__ row_token, int32_t* __restrict__ row_of_choice,
+                                                              int64_t n, int E, int topk, int nblocks) {
+    extern __shared__ int rank_lds[];
+    int* scan = rank_lds;            // [E] inclusive scan of the experts' totals
+    int* base = scan + E;            // [E] first sorted row of this block's choices of expert e
+    int* wh = base + E;              // [16][E] choices of expert e in wavefront w -> in the wavefronts before w
+    const int e = threadIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int blk = blockIdx.x;
+    int total = 0, before = 0;
+    if (e < E) {
+        // independent loads, 4 blocks at a time
+        int b = 0;
+        for (; b + 4 <= nblocks; b += 4) {
+            const int c0 = block_counts[(int64_t)b * E + e], c1 = block_counts[(int64_t)(b + 1) * E + e];
+            const int c2 = block_counts[(int64_t)(b + 2) * E + e], c3 = block_counts[(int64_t)(b + 3) * E + e];
+            total += c0 + c1 + c2 + c3;
+            before += (b < blk ? c0 : 0) + (b + 1 < blk ? c1 : 0) + (b + 2 < blk ? c2 : 0) + (b + 3 < blk ? c3 : 0);
+        }
+        for (; b < nblocks; ++b) {
+            const int c = block_counts[(int64_t)b * E + e];
+            total += c;
+            before += b < blk ? c : 0;
+        }
+        scan[e] = total;
+    }
+    for (int j = threadIdx.x; j < 16 * E; j += RT_BLOCK) wh[j] = 0;
     __syncthreads();
-    // inclusive scan over experts (Hillis-Steele, 10 steps for 1024)
-    for (int off = 1; off < RT_MAX_E; off <<= 1) {
-        const int add = e >= off ? scan[e - off] : 0;
+    // inclusive scan over experts (Hillis-Steele)
+    for (int off = 1; off < E; off <<= 1) {
+        const int add = (e < E && e >= off) ? scan[e - off] : 0;
         __syncthreads();
-        scan[e] += add;
+        if (e < E) scan[e] += add;
         __syncthreads();
     }
     if (e < E) {
-        group_list[e] = scan[e];
-        int run = scan[e] - total;
-        for (int b = 0; b < nblocks; ++b) {
-            block_base[(int64_t)b * E + e] = run;
-            run += block_counts[(int64_t)b * E + e];
+        base[e] = scan[e] - total + before;
+        if (blk == 0) group_list[e] = scan[e];
+    }
+    const int64_t i = (int64_t)blk * RT_BLOCK + threadIdx.x;
+    const int my = i < n ? ids[i] : -1;
+    const bool valid = (unsigned)my < (unsigned)E;   // ids outside [0, E) are dropped
+    if (valid) atomicAdd(&wh[wave * E + my], 1);
+    __syncthreads();
+    if (e < E) {
+        int run = 0;
+#pragma unroll
+        for (int w = 0; w < 16; ++w) {
+            const int t = wh[w * E + e];
+            wh[w * E + e] = run;
+            run += t;
         }
     }
-}
-
-__global__ __launch_bounds__(RT_BLOCK) void route_rank_kernel(const int32_t* __restrict__ ids, const int32_t* __restrict__ block_base,
-                                                              int32_t* __restrict__ row_token, int32_t* __restrict__ row_of_choice,
-                                                              int64_t n, int E, int topk) {
-    __shared__ int sid[RT_BLOCK];
-    const int64_t i = (int64_t)blockIdx.x * RT_BLOCK + threadIdx.x;
-    const int my = i < n ? ids[i] : -1;
-    sid[threadIdx.x] = my;
+    // equal ids in the lanes below this one
+    int lower = 0;
+    for (int k = 0; k < 63; ++k) {
+        const int ek = __builtin_amdgcn_readlane(my, k);
+        lower += (ek == my && k < lane) ? 1 : 0;
+    }
     __syncthreads();
     if (i >= n) return;
-    if ((unsigned)my >= (unsigned)E) {
+    if (!valid) {
         row_of_choice[i] = -1;
         return;
     }
-    int rank = 0;
-    for (int j = 0; j < (int)threadIdx.x; ++j) rank += sid[j] == my;
-    const int dst = block_base[(int64_t)blockIdx.x * E + my] + rank;
+    const int dst = base[my] + wh[wave * E + my] + lower;
     row_token[dst] = (int32_t)(i / topk);
     row_of_choice[i] = dst;
 }
 
-__global__ __launch_bounds__(256) void route_gather_kernel(const u32x4_t* __restrict__ x, const int32_t* __restrict__ row_token,
-                                                           const int64_t* __restrict__ group_list, int E,
-                                                           u32x4_t* __restrict__ x_sorted, int64_t n, int units) {
-    // 4 rows per workgroup, one wavefront each
-    const int64_t r = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-    // Only rows below group_list[E - 1] (written by the scan kernel earlier on this stream) have a token:
-    // dropped choices leave the tail of row_token unwritten, and the tail of x_sorted stays untouched.
-    if (r >= n || r >= group_list[E - 1]) return;
-    const u32x4_t* src = x + (int64_t)row_token[r] * units;
-    u32x4_t* dst = x_sorted + r * units;
-    // 8 independent 16-byte loads in flight per lane
-    for (int u0 = threadIdx.x & 63; u0 < units; u0 += 8 * 64) {
-        u32x4_t v[8];
+// x rows copied into sorted order, token by token: a workgroup reads one token's row once (16 bytes per
+// thread and load, 4 loads in flight) and writes it to the sorted row of each of its choices.  Dropped
+// choices (row_of_choice < 0) write nothing, so the rows past group_list[E - 1] stay untouched.
+__global__ __launch_bounds__(256) void route_scatter_kernel(const u32x4_t* __restrict__ x, const int32_t* __restrict__ row_of_choice,
+                                                            u32x4_t* __restrict__ x_sorted, int topk, int units) {
+    const int t = blockIdx.x;
+    const u32x4_t* src = x + (int64_t)t * units;
+    const int32_t* roc = row_of_choice + (int64_t)t * topk;
+    for (int u0 = threadIdx.x; u0 < units; u0 += 4 * 256) {
+        u32x4_t v[4];
 #pragma unroll
-        for (int j = 0; j < 8; ++j)
-            if (u0 + 64 * j < units) v[j] = src[u0 + 64 * j];
+        for (int j = 0; j < 4; ++j)
+            if (u0 + 256 * j < units) v[j] = src[u0 + 256 * j];
+        for (int c = 0; c < topk; ++c) {
+            const int r = __builtin_amdgcn_readfirstlane(roc[c]);
+            if (r < 0) continue;
+            u32x4_t* dst = x_sorted + (int64_t)r * units;
 #pragma unroll
-        for (int j = 0; j < 8; ++j)
-            if (u0 + 64 * j < units) __builtin_nontemporal_store(v[j], dst + u0 + 64 * j);
+            for (int j = 0; j < 4; ++j)
+                if (u0 + 256 * j < units) __builtin_nontemporal_store(v[j], dst + u0 + 256 * j);
+        }
     }
 }
 
 size_t route_workspace_bytes(const moe_route_args* a) {
     const int64_t n = a->T * a->topk;
     const int64_t nblocks = (n + RT_BLOCK - 1) / RT_BLOCK;
-    return (size_t)(2 * nblocks * a->E) * sizeof(int32_t);   // per-block counts and per-block first rows
+    return (size_t)(nblocks * a->E) * sizeof(int32_t);   // per-block counts
 }
 
 // Scratch of moe_route_static: the per-block counts and first rows live in this array instead of a
@@ -192,7 +221,6 @@ int launch_route(const moe_route_args* a, hipStream_t stream) {
     const int nblocks = (int)((n + RT_BLOCK - 1) / RT_BLOCK);
     int32_t* ids = static_cast<int32_t*>(a->topk_ids);
     int32_t* counts = static_cast<int32_t*>(a->workspace);
-    int32_t* base = counts + (int64_t)nblocks * a->E;
     if (a->logits && a->T > 0) {
         hipLaunchKernelGGL(route_topk_kernel, dim3((unsigned)((a->T + 3) / 4)), dim3(256), 0, stream,
                            static_cast<const float*>(a->logits), static_cast<float*>(a->topk_weight), ids, (int)a->T,
@@ -201,18 +229,19 @@ int launch_route(const moe_route_args* a, hipStream_t stream) {
     }
     if (nblocks > 0)
         hipLaunchKernelGGL(route_count_kernel, dim3((unsigned)nblocks), dim3(RT_BLOCK), 0, stream, ids, counts, n, (int)a->E);
-    hipLaunchKernelGGL(route_scan_kernel, dim3(1), dim3(RT_MAX_E), 0, stream, counts, base,
-                       static_cast<int64_t*>(a->group_list), nblocks, (int)a->E);
-    if (nblocks > 0)
-        hipLaunchKernelGGL(route_rank_kernel, dim3((unsigned)nblocks), dim3(RT_BLOCK), 0, stream, ids, base,
-                           static_cast<int32_t*>(a->row_token), static_cast<int32_t*>(a->row_of_choice), n, (int)a->E,
-                           (int)a->topk);
+    // one block even without choices: it writes group_list (all zeros then)
+    const size_t lds = (size_t)18 * a->E * sizeof(int);
+    static std::atomic<uint64_t> lds_set{0};
+    if (const int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(&route_rank_kernel), 18 * RT_MAX_E * (int)sizeof(int), lds_set))
+        return rc;
+    hipLaunchKernelGGL(route_rank_kernel, dim3((unsigned)(nblocks > 0 ? nblocks : 1)), dim3(RT_BLOCK), lds, stream, ids, counts,
+                       static_cast<int64_t*>(a->group_list), static_cast<int32_t*>(a->row_token),
+                       static_cast<int32_t*>(a->row_of_choice), n, (int)a->E, (int)a->topk, nblocks);
     if (hipGetLastError() != hipSuccess) return MOE_ERR_LAUNCH;
     if (a->x && n > 0) {
-        hipLaunchKernelGGL(route_gather_kernel, dim3((unsigned)((n + 3) / 4)), dim3(256), 0, stream,
-                           static_cast<const u32x4_t*>(a->x), static_cast<const int32_t*>(a->row_token),
-                           static_cast<const int64_t*>(a->group_list), (int)a->E, static_cast<u32x4_t*>(a->x_sorted), n,
-                           (int)(a->K / 8));
+        hipLaunchKernelGGL(route_scatter_kernel, dim3((unsigned)a->T), dim3(256), 0, stream,
+                           static_cast<const u32x4_t*>(a->x), static_cast<const int32_t*>(a->row_of_choice),
+                           static_cast<u32x4_t*>(a->x_sorted), (int)a->topk, (int)(a->K / 8));
         if (hipGetLastError() != hipSuccess) return MOE_ERR_LAUNCH;
     }
     return MOE_OK;

@@ -271,7 +271,7 @@ def extra_route(torch, mg, warmup):
     t = time_batch(torch, lambda: mg.route(ra, stream()), 20, warmup)
     nbytes = T * E * 4 + T * K * 2 + n * K * 2      # logits + x read (x rows are re-read from cache) + sorted rows written
     out["routing_4096x256_top8"] = dict(bytes=nbytes, us=t * 1e6, GBps=nbytes / t / 1e9, frac_hbm=nbytes / t / 1e9 / PEAK_HBM_GBS,
-                                        note="5 kernels: top-k, histogram, scan, rank, row gather")
+                                        note="4 kernels: top-k, histogram, scan + rank, row scatter")
     del lg, xr, xs
     return out
 

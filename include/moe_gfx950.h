@@ -233,7 +233,7 @@ int moe_route(const moe_route_args *args, moe_stream_t stream);
  * reference.  Same arguments and results as moe_route; args->workspace is ignored (may be NULL): the
  * scratch is a static device array inside the library, MOE_ROUTE_STATIC_SCRATCH_BYTES per GPU, held
  * until the process ends.  Calls whose moe_route_workspace_bytes() exceeds it return MOE_ERR_TOO_LARGE
- * (with 256 experts that is more than 1048576 routed choices T * topk).  Allocates nothing; the first
+ * (with 256 experts that is more than 2097152 routed choices T * topk).  Allocates nothing; the first
  * call on a GPU looks the array's address up (hipGetSymbolAddress), so make that call with the GPU
  * current and outside a stream capture.  All calls on one GPU share the array: calls that overlap in
  * time on the same GPU race on it -- keep them on one stream or otherwise ordered. */

@@ -57,7 +57,7 @@ def test_route_static_matches_route_twice_second_smaller():
 def test_route_static_rejects_sizes_beyond_its_scratch():
     import moe_gfx950 as mg
 
-    # 2 * ceil(T * topk / 1024) * E * 4 bytes of scratch: 1024 experts, 2^20 choices -> 8 MiB > 2 MiB
+    # ceil(T * topk / 1024) * E * 4 bytes of scratch: 1024 experts, 2^20 choices -> 4 MiB > 2 MiB
     args = mg.route_args(16, 0, 16, 16, 16, 16, 16, 0, 0, 1 << 17, 1024, 0, 8)
     assert mg.route_workspace_bytes(args) > mg.ROUTE_STATIC_SCRATCH_BYTES
     with pytest.raises(mg.MoeError) as e:
