@@ -354,9 +354,9 @@ __device__ __forceinline__ void lds_load16(rsrc_t r, const u32x4_t* dst, int vof
 // LDS-direct loads into a ring of S = 5 stages.  The loads of stage kt+4 (it replaces stage kt-1,
 // last read before barrier kt-1) and the LDS reads of the packed dwords of stage kt+1 are
 // spread between the MFMAs of step kt; before barrier kt each wavefront waits until its own
-// loads of stage kt+2 have landed.  vmcnt counts a wavefront's loads in order and every
-// wavefront issues the same number NI of them per step (waves without a row block of their
-// own repeat one), so "at most (S - 3) NI outstanding" means exactly that.
+// loads of stage kt+2 have landed.  vmcnt counts a wavefront's loads in order and a
+// wavefront issues the same number of them in every step (NI, or NI - 1 for those without a row block of
+// their own in the last round of x loads), so "at most S - 3 groups outstanding" is a fixed count.
 //
 // Decode of a k-row pair (a, b) of one dword column: v_perm gathers the two bytes of each row
 // this lane owns, the low nibbles (& 0x0f0f0f0f) and high nibbles (>> 4 & 0x0f0f0f0f) are bytes
@@ -381,7 +381,10 @@ __device__ __forceinline__ void lds_load16(rsrc_t r, const u32x4_t* dst, int vof
 // ---------------------------------------------------------------------------------
 constexpr int PAIR_CAPB = 10;                         // x stages hold 160 rows
 constexpr int PAIR_MT_MAX = 10;
-constexpr int PAIR_A_UNITS = 16 * PAIR_CAPB * 8;      // 16-byte units of one x stage
+constexpr int PAIR_EXACT_MT_MAX = 2;                  // row blocks per tile with the GEMV op's arithmetic
+// 16-byte units of one x stage: 160 rows, or the 32 rows of the GEMV op's tiles (whose small stages let two
+// workgroups share a CU: one computes while the other waits at its barrier)
+constexpr int pair_a_units(bool exact) { return 16 * (exact ? PAIR_EXACT_MT_MAX : PAIR_CAPB) * 8; }
 // packed tile of one k step: 64 rows of 128 bytes (4-bit codes) or of 256 bytes (int8, fp8)
 template <int FMT>
 constexpr int pair_b_units() { return (FMT == MOE_FMT_INT8 || FMT == MOE_FMT_FP8_REF) ? 64 * 16 : 64 * 8; }
@@ -398,8 +401,8 @@ constexpr int pair_sc_units() { return FMT == MOE_FMT_FP4_REF ? 128 : FMT == MOE
 template <int FMT>
 constexpr int pair_kc_scale_units() { return (FMT == MOE_FMT_FP4_B32 || FMT == MOE_FMT_FP4_B16) ? 3 * 256 : 0; }
 template <int FMT>
-constexpr int pair_lds_units() {
-    return pair_stages<FMT>() * (PAIR_A_UNITS + pair_b_units<FMT>() + pair_sc_units<FMT>()) + pair_kc_scale_units<FMT>();
+constexpr int pair_lds_units(bool exact) {
+    return pair_stages<FMT>() * (pair_a_units(exact) + pair_b_units<FMT>() + pair_sc_units<FMT>()) + pair_kc_scale_units<FMT>();
 }
 
 // End of a k-split tile.  The two wavefronts of a pair (same columns, the two k halves) hold partial sums of the
@@ -411,7 +414,7 @@ template <int MT, bool KC>
 __device__ __forceinline__ void pair_finish(const GemmParams& P, u32x4_t* smem, f32x4_t (&acc)[MT][4], int h, int cw, int lane,
                                             int col0, int64_t row0, int rows, int n0) {
     const int i = lane & 15, q = lane >> 4;
-    constexpr int RR = 4, MH = (MT + 1) / 2, ROUNDS = (MH + RR - 1) / RR;
+    constexpr int MH = (MT + 1) / 2, RR = MH < 4 ? MH : 4, ROUNDS = (MH + RR - 1) / RR;
     // the last tile of an N that is not a multiple of 256 (the reference's fp8 container: multiples of 128)
     // computes columns past N from whatever follows in the slab: they are not stored
     const bool live = KC || n0 + col0 < P.N;
@@ -500,6 +503,8 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
     constexpr int BK = 64, S = pair_stages<FMT>(), PAIR_SC_UNITS = pair_sc_units<FMT>();
     constexpr int PAIR_B_UNITS = pair_b_units<FMT>();
     constexpr int AHEAD = S - 1;   // a step's loads fill the stage of step kt + AHEAD
+    constexpr int PAIR_A_UNITS = pair_a_units(EXACT);
+    static_assert(16 * MT * 8 <= PAIR_A_UNITS, "tile rows beyond the x stage");
     u32x4_t* lds_a = smem;
     u32x4_t* lds_b = lds_a + S * PAIR_A_UNITS;
     u32x4_t* lds_s = lds_b + S * PAIR_B_UNITS;
@@ -551,11 +556,13 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
     int ja[NA], ca[NA];
 #pragma unroll
     for (int m = 0; m < NA; ++m) {
-        int j = wv + 8 * m;
-        if (8 * NA > 2 * MT) j = j % (2 * MT);   // repeat a block rather than issue fewer loads
+        const int j = wv + 8 * m;
         ja[m] = j * 64;
         ca[m] = 8 * j * P.K * 2;
     }
+    // the tile has 2 MT blocks of 8 rows: the wavefronts whose last block lies beyond them issue one load less
+    // per step, and count one less per group in their waits
+    const bool skip_last = wv + 8 * (NA - 1) >= 2 * MT;
     const int cb = KC ? n0 * (P.K >> 1) : B8 ? 8 * wv * P.N + n0 : 8 * wv * (P.N >> 1) + (n0 >> 1);
     const int kb_step = KC ? BK / 2 : B8 ? BK * P.N : BK * (P.N >> 1);
     // K-contiguous fp4 scales.  Fetching the 4 or 8 bytes a weight row needs per step costs a request per
@@ -580,6 +587,7 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
     // m-th load of group kt (stage kt+AHEAD of x, packed tile and scales), into LDS stage ST
     auto issue = [&](int m, int kt, int ST) {
         if (m < NA) {
+            if (m == NA - 1 && skip_last) return;
             // past K a row's next bytes are the following row's (valid memory, real traffic): the loads of the last
             // AHEAD steps are sent beyond the end of the resource instead, where they cost nothing and return 0
             const int koff = kt + AHEAD < nk ? (kt + AHEAD) * (BK * 2) : 0x7ff00000;
@@ -645,6 +653,13 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
     // groups -AHEAD .. -1: stages 0 .. AHEAD-1; stages 0 and 1 must have landed before the first barrier
     // (WAITN: the loads of the S - 3 youngest groups may still be in flight at a barrier)
     constexpr int WAITN = (S - 3) * NI;
+    // wait until this wavefront's loads of all but the S - 3 youngest groups have landed, then the step's barrier
+    auto ring_barrier = [&]() {
+        if (skip_last)
+            asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(WAITN - (S - 3)) : "memory");
+        else
+            asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(WAITN) : "memory");
+    };
     if constexpr (KC) {
         // the scale loads the groups below do not cover (older than all of them: landed by the first barrier)
 #pragma unroll
@@ -652,7 +667,7 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
     }
 #pragma unroll
     for (int st0 = 0; st0 < AHEAD; ++st0) issue_group(st0 - AHEAD, st0);
-    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(WAITN) : "memory");
+    ring_barrier();
     if constexpr (I8) {
         ch_s[0] = bf16_lo(ch_sb[0]); ch_s[1] = bf16_hi(ch_sb[0]); ch_s[2] = bf16_lo(ch_sb[1]); ch_s[3] = bf16_hi(ch_sb[1]);
         ch_o[0] = bf16_lo(ch_ob[0]); ch_o[1] = bf16_hi(ch_ob[0]); ch_o[2] = bf16_lo(ch_ob[1]); ch_o[3] = bf16_hi(ch_ob[1]);
@@ -744,7 +759,7 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
                     // barrier kt-1 for the wavefronts that own sub-step 1, half way through their decode
                     // (not in the tile's first step: the barrier of the prologue stands for it); x stage
                     // kt is visible behind it
-                    if (kt > 0) asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(WAITN) : "memory");
+                    if (kt > 0) ring_barrier();
                 }
                 // first x fragments of the MFMA phase, read under the rest of the decode
 #pragma unroll
@@ -940,7 +955,7 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
             __builtin_amdgcn_sched_barrier(0);
         }
         __builtin_amdgcn_s_setprio(0);
-        if (h == 0) asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(WAITN) : "memory");   // barrier kt
+        if (h == 0) ring_barrier();   // barrier kt
     };
     for (int kt = 0, st = 0, sl = S - 1; kt < nk; ++kt) {
         const int sn = st == S - 1 ? 0 : st + 1;
@@ -948,7 +963,7 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
         st = sn;
         sl = sl == S - 1 ? 0 : sl + 1;
     }
-    if (h == 1) asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(WAITN) : "memory");       // barrier nk-1
+    if (h == 1) ring_barrier();       // barrier nk-1
     // drain this wavefront's loads (they target stages past K and are never read); the
     // accumulators were last written by MFMAs the compiler cannot see: wait out their latency
     asm volatile("s_waitcnt vmcnt(0)\n\ts_nop 15\n\ts_nop 15\n\ts_barrier" ::: "memory");
@@ -977,8 +992,6 @@ __device__ __forceinline__ void expert_chunks(int m, int& chunks, int& bpc) {
 //   GK_PAIR     N-contiguous containers: 8 wavefronts, k range split between the two wavefronts of a SIMD
 //   GK_PAIR_EXACT  GK_PAIR with the GEMV op's arithmetic (weights not rounded to bf16), tiles of at most 32 rows
 enum { GK_GENERAL = 0, GK_SKINNY = 1, GK_PAIR = 2, GK_PAIR_EXACT = 3 };
-constexpr int PAIR_EXACT_MT_MAX = 2;
-
 template <int FMT, int KIND>
 struct KernelCfg {
     static constexpr bool PAIR = KIND == GK_PAIR || KIND == GK_PAIR_EXACT;
@@ -986,7 +999,10 @@ struct KernelCfg {
     static_assert(!PAIR || FMT != MOE_FMT_BF16, "the k-split tile routine decodes quantized containers");
     static constexpr int WAVES = PAIR ? 8 : 4;
     static constexpr int BN = GM_BN;                                             // columns per tile
-    static constexpr int WG_PER_CU = SKINNY ? GM_SKINNY_WAVES : 1;
+    // the 4-bit containers with the GEMV op's arithmetic: two workgroups per CU (their stages hold 32 rows of x)
+    static constexpr bool TWO_PER_CU = KIND == GK_PAIR_EXACT && FMT == MOE_FMT_INT4;
+    static constexpr int WG_PER_CU = SKINNY ? GM_SKINNY_WAVES : TWO_PER_CU ? 2 : 1;
+    static constexpr int WAVES_PER_SIMD = WG_PER_CU * (PAIR ? 2 : 1);
     static constexpr int CAPB = SKINNY ? GM_SKINNY_BLOCKS : PAIR ? PAIR_CAPB : GM_MT_MAX;
     static constexpr int fmt_mt_max() {
         if constexpr (PAIR)
@@ -998,7 +1014,7 @@ struct KernelCfg {
     // 16-byte LDS units of the tile routine (the tile prefix array follows them)
     static constexpr int lds_units() {
         if constexpr (PAIR)
-            return pair_lds_units<FMT>();
+            return pair_lds_units<FMT>(KIND == GK_PAIR_EXACT);
         else
             return 2 * 16 * CAPB * (BTraits<FMT>::BK / 8);
     }
@@ -1014,7 +1030,7 @@ __device__ __forceinline__ void run_tile(const GemmParams& P, u32x4_t* smem, int
 }
 
 template <int FMT, int KIND>
-__global__ __launch_bounds__((64 * KernelCfg<FMT, KIND>::WAVES), (KernelCfg<FMT, KIND>::WG_PER_CU)) void grouped_gemm_kernel(GemmParams P) {
+__global__ __launch_bounds__((64 * KernelCfg<FMT, KIND>::WAVES), (KernelCfg<FMT, KIND>::WAVES_PER_SIMD)) void grouped_gemm_kernel(GemmParams P) {
     using C = KernelCfg<FMT, KIND>;
     constexpr int WAVES = C::WAVES;
     extern __shared__ u32x4_t smem[];
