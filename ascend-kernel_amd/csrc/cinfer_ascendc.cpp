@@ -146,7 +146,8 @@ void GroupedGemm(at::Tensor x, at::Tensor weight, at::Tensor antiquantScaleOptio
 }
 
 // Extra entry point: grouped_gemm with the SwiGLU activation fused into its epilogue (see moe_epilogue in
-// moe_gfx950.h): weight columns in groups of (gate 2j, gate 2j+1, up 2j, up 2j+1), output [M, N/2].
+// moe_gfx950.h): weight columns in groups of (gate 2j, gate 2j+1, up 2j, up 2j+1) on the N-contiguous containers, weight rows
+// in blocks of (16 gate, 16 up) on the K-contiguous ones; output [M, N/2].
 void GroupedGemmSwiglu(at::Tensor x, at::Tensor weight, at::Tensor antiquantScaleOptional,
                        at::Tensor antiquantOffsetOptional, at::Tensor groupListOptional, const char* computeType,
                        at::Tensor output) {

@@ -16,12 +16,7 @@ inline bool fits_i32(int64_t v) { return v >= 0 && v <= 0x7fffffffLL; }
 int validate_grouped(const moe_grouped_args* a, int64_t k_mult, int64_t n_mult, bool allow_epilogue) {
     if (!a) return MOE_ERR_NULL_POINTER;
     if (a->format < 0 || a->format >= MOE_FMT_COUNT) return MOE_ERR_BAD_FORMAT;
-    if (a->epilogue != MOE_EPILOGUE_NONE) {
-        // the fused activation lives in the GEMM kernels' epilogue for containers whose lanes own 4 adjacent columns
-        const bool n_contiguous = a->format == MOE_FMT_FP4_REF || a->format == MOE_FMT_FP8_REF ||
-                                  a->format == MOE_FMT_INT8 || a->format == MOE_FMT_INT4;
-        if (a->epilogue != MOE_EPILOGUE_SWIGLU || !allow_epilogue || !n_contiguous) return MOE_ERR_BAD_FORMAT;
-    }
+    if (a->epilogue != MOE_EPILOGUE_NONE && (a->epilogue != MOE_EPILOGUE_SWIGLU || !allow_epilogue)) return MOE_ERR_BAD_FORMAT;
     if (a->M < 0 || a->K <= 0 || a->N <= 0 || a->G <= 0) return MOE_ERR_BAD_SHAPE;
     // same limit as the reference: grouped_matmul_antiquant_tiling.cpp:260-264
     if (!fits_i32(a->M) || !fits_i32(a->K) || !fits_i32(a->N) || !fits_i32(a->G)) return MOE_ERR_TOO_LARGE;

@@ -176,6 +176,22 @@ __device__ __forceinline__ void store_tile(const GemmParams& P, const BCtx& c, f
     // through a buffer resource that ends after the tile's last valid row: stores to padded
     // rows fall outside it and are dropped (the containers of this routine are K-contiguous: a lane's
     // 4 accumulators of a row are 16 columns apart)
+    if (P.epilogue == MOE_EPILOGUE_SWIGLU) {
+        // weight rows in blocks of 32 = (16 gate rows, 16 up rows): MFMAs (0, 1) and (2, 3); y has N / 2 columns
+        const int NO = P.N >> 1;
+        const rsrc_t ro = make_rsrc(P.y + row0 * (int64_t)NO, (int64_t)rows * NO * 2);
+        const int vo = (4 * c.q * NO + ((n0 + 64 * c.w) >> 1) + c.i) * 2;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+#pragma unroll
+                for (int u = 0; u < 2; ++u)
+                    __builtin_amdgcn_raw_buffer_store_b16(
+                        (uint16_t)(pack_bf16_rne(swiglu(acc[mt][2 * u][r], acc[mt][2 * u + 1][r]), 0.f) & 0xffffu), ro,
+                        vo + 32 * u, (16 * mt + r) * NO * 2, 0);
+        return;
+    }
     const rsrc_t ry = make_rsrc(P.y + row0 * (int64_t)P.N, (int64_t)rows * P.N * 2);
     const int vy = (4 * c.q * P.N + n0) * 2;
 #pragma unroll
@@ -425,7 +441,18 @@ __device__ __forceinline__ void pair_finish(const GemmParams& P, u32x4_t* smem, 
     const rsrc_t ry = make_rsrc(P.y + row0 * (int64_t)NO, (int64_t)rows * NO * 2);
     auto store_block = [&](int mt) {
         if (!live) return;
-        if (swi) {
+        if (swi && KC) {
+            // K-contiguous containers: the weight rows come in blocks of 32 = (16 gate rows, 16 up rows), which are
+            // the MFMAs t = (0, 1) and (2, 3) of this lane; y has N / 2 columns
+            const int vo = (4 * q * NO + ((n0 + 64 * cw) >> 1) + i) * 2;
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+#pragma unroll
+                for (int u = 0; u < 2; ++u)
+                    __builtin_amdgcn_raw_buffer_store_b16(
+                        (uint16_t)(pack_bf16_rne(swiglu(acc[mt][2 * u][r], acc[mt][2 * u + 1][r]), 0.f) & 0xffffu), ry,
+                        vo + 32 * u, (16 * mt + r) * NO * 2, 0);
+        } else if (swi) {
             // this lane's 4 columns are (gate, gate, up, up) of 2 output columns; y has N / 2 columns
             const int vo = (4 * q * NO + ((n0 + col0) >> 1)) * 2;
 #pragma unroll
@@ -1213,7 +1240,8 @@ int launch_gemm_exact(const moe_grouped_args* a, hipStream_t stream) {
 int launch_grouped_gemm(const moe_grouped_args* a, hipStream_t stream) {
     // Decode-sized batches on the K-contiguous containers go to the weight-streaming GEMV kernels,
     // run with this op's arithmetic.
-    if (gemv_preferred(a)) return launch_grouped_gemv(a, stream, true);
+    // (the GEMV kernels have no fused activation: such calls stay on the GEMM kernels)
+    if (a->epilogue == MOE_EPILOGUE_NONE && gemv_preferred(a)) return launch_grouped_gemv(a, stream, true);
     switch (a->format) {
         case MOE_FMT_FP4_REF: return launch_gemm_fmt<MOE_FMT_FP4_REF>(a, stream);
         case MOE_FMT_FP8_REF: return launch_gemm_fmt<MOE_FMT_FP8_REF>(a, stream);

@@ -110,11 +110,15 @@ typedef enum moe_weight_format {
 
 /* What the grouped GEMM writes.  MOE_EPILOGUE_SWIGLU fuses the activation that sits between the
  * gate_up and the down projection of an MoE layer into the GEMM (no counterpart in the reference,
- * whose caller runs it as a separate op on the [M, N] result): the weight's columns come in groups
- * of 4 = (gate 2j, gate 2j+1, up 2j, up 2j+1) and y is bf16 [M, N/2] with
- *     y[m, 2j + e] = silu(z[m, 4j + e]) * z[m, 4j + 2 + e],  e = 0, 1,
- * z the fp32 accumulators of x . dequant(W) and silu(v) = v / (1 + exp(-v)).  Grouped GEMM only,
- * on the N-contiguous containers (MOE_FMT_FP4_REF, MOE_FMT_FP8_REF, MOE_FMT_INT8, MOE_FMT_INT4). */
+ * whose caller runs it as a separate op on the [M, N] result): y is bf16 [M, N/2] with
+ *     y[m, c] = silu(z[m, gate(c)]) * z[m, up(c)],   silu(v) = v / (1 + exp(-v)),
+ * z the fp32 accumulators of x . dequant(W).  The gate and up columns are interleaved the way each
+ * container's lanes hold them:
+ *   N-contiguous containers (MOE_FMT_FP4_REF, MOE_FMT_FP8_REF, MOE_FMT_INT8, MOE_FMT_INT4): groups of 4
+ *   columns = (gate 2j, gate 2j+1, up 2j, up 2j+1): gate(2j+e) = 4j+e, up(2j+e) = 4j+2+e;
+ *   K-contiguous containers (MOE_FMT_FP4_B32, MOE_FMT_FP4_B16, MOE_FMT_BF16): blocks of 32 weight rows =
+ *   (gate 16j .. 16j+15, up 16j .. 16j+15): gate(16j+i) = 32j+i, up(16j+i) = 32j+16+i.
+ * Grouped GEMM only. */
 typedef enum moe_epilogue {
     MOE_EPILOGUE_NONE = 0,
     MOE_EPILOGUE_SWIGLU = 1

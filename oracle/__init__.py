@@ -194,3 +194,16 @@ def swiglu_interleaved(z: np.ndarray) -> np.ndarray:
     gate, up = q[:, :, 0:2], q[:, :, 2:4]
     out = (gate / (1.0 + np.exp(-gate)) * up).reshape(M, N // 2)
     return f32_to_bf16_bits(out.astype(np.float32))
+
+
+def swiglu_blocked16(z: np.ndarray) -> np.ndarray:
+    """The fused activation on the K-contiguous containers: the weight rows (columns of z) come in blocks of
+    32 = (gate 16j..16j+15, up 16j..16j+15); out[:, 16j+i] = silu(z[:, 32j+i]) * z[:, 32j+16+i], float64, one
+    rounding to bf16.  Same definition of silu as swiglu_interleaved; pinned to torch in tests/test_oracle.py."""
+    z = np.asarray(z, dtype=np.float64)
+    M, N = z.shape
+    assert N % 32 == 0
+    b = z.reshape(M, N // 32, 2, 16)
+    gate, up = b[:, :, 0, :], b[:, :, 1, :]
+    out = (gate / (1.0 + np.exp(-gate)) * up).reshape(M, N // 2)
+    return f32_to_bf16_bits(out.astype(np.float32))

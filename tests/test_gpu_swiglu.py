@@ -12,6 +12,7 @@ import oracle
 
 pytestmark = pytest.mark.gpu
 N_CONTIG = ["fp4", "fp8", "int8", "int4"]
+K_CONTIG = ["fp4_b32", "fp4_b16", "bf16"]
 
 
 def _say(msg):
@@ -37,7 +38,7 @@ def _run(case):
 def _expected(case):
     _, z = oracle.grouped_gemm(oracle.FMT_BY_NAME[case["fmt"]], case["x"], case["weight"], case["scale"], case["offset"],
                                case["group_list"], want_f32=True)
-    return oracle.swiglu_interleaved(z)
+    return oracle.swiglu_blocked16(z) if case["fmt"] in K_CONTIG else oracle.swiglu_interleaved(z)
 
 
 @pytest.mark.parametrize("fmt", N_CONTIG)
@@ -48,6 +49,21 @@ def test_swiglu_epilogue(fmt, gl):
     case = H.make_case(fmt, len(gl), K, 512, gl, seed=len(gl) * 7 + K, extra_rows=2)
     if fmt in ("int4", "int8"):
         # larger outputs so that silu is exercised away from 0 as well
+        case["x"] = oracle.f32_to_bf16_bits(oracle.bf16_bits_to_f32(case["x"]) * 4.0)
+    got = _run(case)
+    H.assert_close(got, _expected(case), rows=slice(0, gl[-1]), what=f"swiglu {fmt}")
+    assert (got[gl[-1]:] == 0x7FC0).all(), "rows beyond group_list[-1] were written"
+
+
+@pytest.mark.parametrize("fmt", K_CONTIG)
+@pytest.mark.parametrize("gl", [[2, 3, 4, 40], [130, 130, 143, 300, 301], [0, 7, 7, 8], [0, 200, 200, 200]],
+                         ids=["small", "prefill", "decode", "one_big"])
+def test_swiglu_epilogue_k_contiguous(fmt, gl):
+    """K-contiguous containers: gate and up rows interleaved in blocks of 16 (the decode-sized batches stay on
+    the GEMM kernels: the weight-streaming GEMV kernels have no fused activation)."""
+    _say(f"swiglu fmt={fmt} gl={gl}")
+    case = H.make_case(fmt, len(gl), 512, 512, gl, seed=len(gl) * 11 + len(fmt), extra_rows=2)
+    if fmt == "bf16":
         case["x"] = oracle.f32_to_bf16_bits(oracle.bf16_bits_to_f32(case["x"]) * 4.0)
     got = _run(case)
     H.assert_close(got, _expected(case), rows=slice(0, gl[-1]), what=f"swiglu {fmt}")
@@ -87,13 +103,8 @@ def test_swiglu_via_module_and_rejections():
                                        torch.zeros(1, dtype=torch.bfloat16, device="cuda"), dev["group_list"], "int4", out)
     torch.cuda.synchronize()
     H.assert_close(H.bits(out.cpu()), _expected(case), what="module swiglu")
-    # K-contiguous containers and the GEMV op have no fused epilogue
+    # the GEMV op has no fused epilogue
     t = torch.zeros(4096, dtype=torch.uint8, device="cuda")
-    a = mg.grouped_args(mg.FMT_BF16, t.data_ptr(), t.data_ptr(), 0, 0, t.data_ptr(), t.data_ptr(), 4, 256, 256, 2, 1,
-                        epilogue=mg.EPILOGUE_SWIGLU)
-    with pytest.raises(mg.MoeError) as e:
-        mg.grouped_gemm(a)
-    assert e.value.status == mg.ERR_BAD_FORMAT
     a = mg.grouped_args(mg.FMT_INT4, t.data_ptr(), t.data_ptr(), t.data_ptr(), 0, t.data_ptr(), t.data_ptr(), 4, 256, 256, 2,
                         2, epilogue=mg.EPILOGUE_SWIGLU)
     with pytest.raises(mg.MoeError) as e:

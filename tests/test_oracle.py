@@ -314,6 +314,17 @@ def test_swiglu_interleaved_against_torch_silu_and_explicit_columns():
     assert np.allclose(one, [[1.0 / (1.0 + np.exp(-1.0)) * 3.0, -2.0 / (1.0 + np.exp(2.0)) * 4.0]], rtol=2 ** -8)
 
 
+def test_swiglu_blocked16_against_torch_silu():
+    rng = np.random.default_rng(32)
+    z = (rng.standard_normal((3, 64)) * 3).astype(np.float32)
+    got = oracle.bf16_bits_to_f32(oracle.swiglu_blocked16(z))
+    zt = torch.from_numpy(z).double()
+    gate = torch.cat([zt[:, 0:16], zt[:, 32:48]], dim=1)     # first 16 columns of every block of 32
+    up = torch.cat([zt[:, 16:32], zt[:, 48:64]], dim=1)
+    ref = (torch.nn.functional.silu(gate) * up).float().to(torch.bfloat16).float().numpy()
+    assert np.array_equal(got, ref)
+
+
 # ---------------------------------------------------------------- grouped_gemm
 @pytest.mark.parametrize("group_list", [[2, 3, 4, 256], [12, 25, 44, 48], [1, 2, 3, 4], [0, 0, 5, 5], [3, 3, 3, 3]])
 def test_grouped_gemm_against_torch_fp64(group_list):
