@@ -358,6 +358,28 @@ def test_gemv_matches_gemm_on_the_same_inputs():
 
 
 # -------------------------------------------------- error behaviour through the module
+@pytest.mark.parametrize("gl_name,gl", [("decode", [3, 3, 7, 9]), ("prefill", [40, 90, 130, 200])])
+@pytest.mark.parametrize("fmt", ["int4", "fp4", "fp8", "fp4_b32", "fp4_b16"])
+def test_each_op_uses_its_own_weight_rounding(fmt, gl_name, gl):
+    """The GEMM op multiplies weights rounded to bf16 (the reference's phase 1), the GEMV op un-rounded fp32
+    weights (gemv_impl.h:147-199).  The two differ by about a quarter of an output ulp, far inside the parity
+    tolerance, so they are told apart by counting outputs whose bf16 bits differ: against the oracle of its own
+    arithmetic an op differs only where the summation order moves a sum across a rounding boundary, against the
+    other arithmetic in a sizeable share of the outputs.  Covers every dispatch: k-split tiles, the matrix-core
+    GEMV kernels run with either rounding, decode and prefill sized batches."""
+    _say(f"rounding fmt={fmt} gl={gl_name}")
+    case = H.make_case(fmt, len(gl), 2048, 512, gl, seed=len(fmt) + gl[0])
+    dev = H.upload(case)
+    ref = {False: H.oracle_out(case, gemv=False), True: H.oracle_out(case, gemv=True)}
+    apart = float(np.mean(ref[False] != ref[True]))
+    assert apart > 0.03, "the case does not separate the two arithmetics"
+    for op in ("gemm", "gemv"):
+        got = H.run_cabi(case, dev, op)
+        own = float(np.mean(got != ref[op == "gemv"]))
+        other = float(np.mean(got != ref[op != "gemv"]))
+        assert own < 0.25 * other, f"{fmt}/{op}: {own:.4f} of the outputs differ from its own arithmetic, {other:.4f} from the other"
+
+
 def test_module_errors_on_gpu_tensors():
     import cinfer_ascendc
 
