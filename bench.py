@@ -48,6 +48,19 @@ def measured_traffic():
         return None, None
 
 
+def board_state():
+    """Socket power (W) and mean shader clock over the XCDs (MHz) as amd-smi reports them right now, or Nones."""
+    import re
+    import subprocess
+    try:
+        out = subprocess.run(["/opt/rocm/bin/amd-smi", "metric", "-p", "-c"], capture_output=True, text=True, timeout=30).stdout
+        p = re.search(r"SOCKET_POWER: *(\d+) *W", out)
+        clk = [int(v) for v in re.findall(r"GFX_\d+:\s*\n\s*CLK: *(\d+) *MHz", out)]
+        return (int(p.group(1)) if p else None), (sum(clk) / len(clk) if clk else None)
+    except Exception:  # noqa: BLE001
+        return None, None
+
+
 def routed_counts(torch, tokens, experts, topk, gen, max_rows=None):
     """Rows per expert for top-k routing of softmax(N(0,1)) logits (softmax is monotone)."""
     while True:
@@ -543,6 +556,8 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="dsv3_int4_prefill")
+    ap.add_argument("--settle-ms", type=float, default=300.0,
+                    help="untimed run of the workload before the warmup steps, until the clocks have settled")
     ap.add_argument("--no-extra", action="store_true", help="skip the other benchmark configurations")
     ap.add_argument("--only", choices=("headline",) + EXTRA, default=None,
                     help="run just this workload's GPU launches and print its figures (for profiles of one kernel)")
@@ -582,6 +597,25 @@ def main():
 
     wl = build_dsv3_int4_prefill(torch, mg, gen)
     ops = wl["ops"]
+    # The board settles its clocks over the first tenths of a second under this load (measured: the first 20
+    # launches after an idle phase run about 5 % slower than the following ones), so the workload runs untimed for
+    # --settle-ms before the W warmup steps.
+    torch.cuda.synchronize()
+    board = {"socket_power_w_idle": None, "sclk_mhz_idle": None, "socket_power_w_under_load": None, "sclk_mhz_under_load": None,
+             "board_power_limit_w": 1400}
+    if args.settle_ms > 0:
+        board["socket_power_w_idle"], board["sclk_mhz_idle"] = board_state()
+    t_settle = time.perf_counter()
+    while (time.perf_counter() - t_settle) * 1e3 < args.settle_ms:
+        first = board["socket_power_w_under_load"] is None
+        for _ in range(600 if first else 40):         # about 2 s (the first time) / 130 ms of queued launches
+            for op in ops:
+                op()
+        if first:
+            time.sleep(0.5)                               # let the board settle under the load, then read it
+            pw, ck = board_state()                        # while the queue is still running
+            board["socket_power_w_under_load"], board["sclk_mhz_under_load"] = pw or 0, ck
+        torch.cuda.synchronize()
     for _ in range(args.warmup):
         for op in ops:
             op()
@@ -627,12 +661,14 @@ def main():
     result = {
         "metric": "grouped-GEMM TFLOPS + GEMV/dequant HBM GB/s (% of MI355X peak), DSV3 MoE",
         "value": value, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": dt / args.steps * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "settle_ms": args.settle_ms, "ms_per_step": dt / args.steps * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "dsv3_int4_prefill: 256 experts, 4096 tokens x top-8 (32768 rows), gate_up "
                                "7168->4096 + down 2048->7168, int4 zp8 group-128 bf16 scales, bf16 activations",
                    "flops_per_step": step_flops},
         "roofline": roofline,
+        # socket power and shader clock before and during the settle phase: this workload runs at the board's power limit
+        "board": board,
     }
     if not args.no_extra:
         result["workloads"] = run_extra(torch, mg, gen, max(args.steps, 20), args.warmup)
