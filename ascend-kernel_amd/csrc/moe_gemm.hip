@@ -370,9 +370,10 @@ __device__ __forceinline__ void lds_load16(rsrc_t r, const u32x4_t* dst, int vof
 // LDS-direct loads into a ring of S = 5 stages.  The loads of stage kt+4 (it replaces stage kt-1,
 // last read before barrier kt-1) and the LDS reads of the packed dwords of stage kt+1 are
 // spread between the MFMAs of step kt; before barrier kt each wavefront waits until its own
-// loads of stage kt+2 have landed.  vmcnt counts a wavefront's loads in order and a
-// wavefront issues the same number of them in every step (NI, or NI - 1 for those without a row block of
-// their own in the last round of x loads), so "at most S - 3 groups outstanding" is a fixed count.
+// loads of stage kt+2 have landed.  vmcnt counts a wavefront's loads in order and every
+// wavefront issues the same number NI of them per step (waves without a row block of their
+// own repeat one: measured, the repeated loads cost nothing, a branch around them does), so "at most
+// (S - 3) NI outstanding" means exactly that.
 //
 // Decode of a k-row pair (a, b) of one dword column: v_perm gathers the two bytes of each row
 // this lane owns, the low nibbles (& 0x0f0f0f0f) and high nibbles (>> 4 & 0x0f0f0f0f) are bytes
@@ -583,13 +584,11 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
     int ja[NA], ca[NA];
 #pragma unroll
     for (int m = 0; m < NA; ++m) {
-        const int j = wv + 8 * m;
+        int j = wv + 8 * m;
+        if (8 * NA > 2 * MT) j = j % (2 * MT);   // repeat a block rather than issue fewer loads
         ja[m] = j * 64;
         ca[m] = 8 * j * P.K * 2;
     }
-    // the tile has 2 MT blocks of 8 rows: the wavefronts whose last block lies beyond them issue one load less
-    // per step, and count one less per group in their waits
-    const bool skip_last = wv + 8 * (NA - 1) >= 2 * MT;
     const int cb = KC ? n0 * (P.K >> 1) : B8 ? 8 * wv * P.N + n0 : 8 * wv * (P.N >> 1) + (n0 >> 1);
     const int kb_step = KC ? BK / 2 : B8 ? BK * P.N : BK * (P.N >> 1);
     // K-contiguous fp4 scales.  Fetching the 4 or 8 bytes a weight row needs per step costs a request per
@@ -614,11 +613,7 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
     // m-th load of group kt (stage kt+AHEAD of x, packed tile and scales), into LDS stage ST
     auto issue = [&](int m, int kt, int ST) {
         if (m < NA) {
-            if (m == NA - 1 && skip_last) return;
-            // past K a row's next bytes are the following row's (valid memory, real traffic): the loads of the last
-            // AHEAD steps are sent beyond the end of the resource instead, where they cost nothing and return 0
-            const int koff = kt + AHEAD < nk ? (kt + AHEAD) * (BK * 2) : 0x7ff00000;
-            lds_load16(rx, lds_a + ST * PAIR_A_UNITS + ja[m], va, ca[m] + koff);
+            lds_load16(rx, lds_a + ST * PAIR_A_UNITS + ja[m], va, ca[m] + (kt + AHEAD) * (BK * 2));
         } else if (m < NA + NB) {
             const int e = m - NA;
             lds_load16(rw, lds_b + ST * PAIR_B_UNITS + wv * (PAIR_B_UNITS / 8) + e * 64, vb,
@@ -681,12 +676,7 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
     // (WAITN: the loads of the S - 3 youngest groups may still be in flight at a barrier)
     constexpr int WAITN = (S - 3) * NI;
     // wait until this wavefront's loads of all but the S - 3 youngest groups have landed, then the step's barrier
-    auto ring_barrier = [&]() {
-        if (skip_last)
-            asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(WAITN - (S - 3)) : "memory");
-        else
-            asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(WAITN) : "memory");
-    };
+    auto ring_barrier = [&]() { asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(WAITN) : "memory"); };
     if constexpr (KC) {
         // the scale loads the groups below do not cover (older than all of them: landed by the first barrier)
 #pragma unroll
