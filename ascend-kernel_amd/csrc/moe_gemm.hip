@@ -7,16 +7,18 @@
 // global memory and then runs a bf16 matmul on it; here the packed weights are decoded
 // in registers straight into bf16 MFMA fragments and never go back to HBM.
 //
-// Work decomposition.  A tile is (expert, chunk of <= 192 rows, 256 columns).  The
-// tile list is derived inside the kernel from the device-resident cumulative
-// group_list (no host sync); a persistent grid walks it with an XCD-aware order so
-// that the workgroups of one XCD share the x rows of the same experts in that XCD's
-// L2.  A workgroup has 4 wavefronts; every wavefront owns 64 of the 256 columns for
-// ALL rows of the tile, so each weight element is dequantized exactly once per tile.
-// x tiles go through a double-buffered, XOR-swizzled LDS tile shared by the 4 waves.
-// (That is gemm_tile, used by the bf16 container.  The quantized ones -- int4, int8, the K-contiguous fp4 containers and
-// the reference's fp4 and fp8 containers -- use a tile routine with 8 wavefronts and LDS-direct loads
-// instead, see gemm_tile_pair.)
+// Work decomposition.  A tile is (expert, chunk of rows, 256 columns).  The tile list is derived
+// inside the kernel from the device-resident cumulative group_list (no host sync); a persistent
+// grid walks it with an XCD-aware order so that the workgroups of one XCD share the x rows and
+// weight slices of the same experts in that XCD's L2.  Every wavefront owns its columns for ALL
+// rows of the tile, so each weight element is dequantized exactly once per tile.  Two tile routines:
+//   gemm_tile_pair  every quantized container (int4, int8, the K-contiguous fp4 containers, the
+//                   reference's fp4 and fp8): 8 wavefronts, the two of a SIMD split the k range;
+//                   x, packed weights and scales arrive by LDS-direct loads into a ring of stages;
+//                   tiles of up to 160 rows (32 with the GEMV op's arithmetic)
+//   gemm_tile       the bf16 container: 4 wavefronts of 64 columns, x through a double-buffered,
+//                   XOR-swizzled LDS tile, weights from registers; tiles of up to 176 rows, or 32 rows
+//                   and several workgroups per CU for decode-sized batches
 //
 // MFMA: v_mfma_f32_16x16x32_bf16.  Lane l = 16*q + i holds, for A, row i and
 // k = 8q..8q+7 of the 16x32 block; for B, column i and the same k; for the result,
@@ -1003,7 +1005,7 @@ __device__ __forceinline__ void expert_chunks(int m, int& chunks, int& bpc) {
 }
 
 // Kernel variants.
-//   GK_GENERAL  4 wavefronts of 64 columns, one workgroup per CU, tiles of up to 192 rows
+//   GK_GENERAL  4 wavefronts of 64 columns, one workgroup per CU, tiles of up to 176 rows (bf16 only)
 //   GK_SKINNY   the same tile routine with tiles of at most 32 rows and several workgroups per CU
 //               (decode-sized batches are HBM bound: more weight bytes in flight)
 //   GK_PAIR     N-contiguous containers: 8 wavefronts, k range split between the two wavefronts of a SIMD
