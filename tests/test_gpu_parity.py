@@ -66,6 +66,33 @@ def test_dequant_full_size_config():
     assert np.array_equal(_dequant_gpu(codes, scale, 32), oracle.dequant_fp4_bf16(codes, scale, 32))
 
 
+@pytest.mark.parametrize("block", [32, 16])
+def test_dequant_large_tensor_path(block):
+    """Tensors of 128 Mi elements and more run on 1024-thread workgroups: bit-identical to the same rows taken
+    through the small-tensor path slice by slice, and to the oracle on a sample of rows."""
+    import moe_gfx950 as mg
+
+    _say(f"dequant large block={block}")
+    R, C = 16384 + 3, 8192                     # 134 Mi elements, not a multiple of the workgroup's span
+    gen = torch.Generator(device="cuda").manual_seed(block)
+    codes = torch.randint(0, 256, (R, C // 2), dtype=torch.uint8, device="cuda", generator=gen)
+    scale = (torch.rand(R, C // block, device="cuda", generator=gen) * 0.24 + 2.0 ** -8).to(torch.bfloat16)
+    whole = torch.full((R, C), 0x7FC0, dtype=torch.int16, device="cuda")
+    parts = torch.full((R, C), 0x7FC0, dtype=torch.int16, device="cuda")
+    st = torch.cuda.current_stream().cuda_stream
+    mg.dequant_fp4_bf16(codes.data_ptr(), scale.data_ptr(), whole.data_ptr(), R, C, block, st)
+    step = 2048
+    for r0 in range(0, R, step):
+        n = min(step, R - r0)
+        mg.dequant_fp4_bf16(codes[r0:].data_ptr(), scale[r0:].data_ptr(), parts[r0:].data_ptr(), n, C, block, st)
+    torch.cuda.synchronize()
+    assert torch.equal(whole, parts)
+    rows = [0, 1, 4095, 8192, R - 1]
+    got = whole[rows].cpu().numpy().view(np.uint16)
+    want = oracle.dequant_fp4_bf16(codes[rows].cpu().numpy(), H.bits(scale[rows].cpu()), block)
+    assert np.array_equal(got, want)
+
+
 def test_dequant_module_entry_point_and_empty():
     import cinfer_ascendc
 
