@@ -376,3 +376,18 @@ def test_grouped_gemm_rejects_bad_group_list():
         oracle.grouped_gemm(oracle.FMT_FP4_REF, x, w, bf16_bits(scale), None, [3, 2])
     with pytest.raises(RuntimeError):
         oracle.grouped_gemm(oracle.FMT_FP4_REF, x, w, bf16_bits(scale), None, [2, 9])
+
+
+def test_oracle_under_address_and_ub_sanitizers():
+    """`make -C oracle asan`: every entry point of the C oracle on exactly sized heap buffers under
+    AddressSanitizer and UBSan (host code only; the GPU side has no sanitizer on this pool)."""
+    import os
+    import subprocess
+
+    here = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "oracle")
+    r = subprocess.run(["make", "-C", here, "-B", "asan"], capture_output=True, text=True, timeout=300)
+    out = r.stdout + r.stderr
+    if "ASan runtime does not come first" in out:
+        pytest.skip("another preloaded library keeps AddressSanitizer from starting in this environment")
+    assert r.returncode == 0, out[-2000:]
+    assert "sanitize_check ok" in out
