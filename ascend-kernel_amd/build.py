@@ -2,6 +2,7 @@
 
   libmoe_gfx950.so          HIP kernels + the C ABI declared in include/moe_gfx950.h
   cinfer_ascendc.*.so       pybind11/torch module with the reference's Python API
+  cabi_driver               torch-free C++ test driver of the C ABI (tests/cabi_driver.cpp)
 
 Run as `python ascend-kernel_amd/build.py [--no-ext]`; hipcc cross-compiles for
 gfx950 without a GPU.
@@ -190,11 +191,21 @@ def build_extension() -> str:
     return out
 
 
+def build_cabi_driver() -> str:
+    """tests/cabi_driver.cpp: the torch-free C++ caller of the C ABI (a test binary, kept beside the library so that it
+    travels with it and finds it through its rpath)."""
+    out = os.path.join(HERE, "cabi_driver")
+    _run([HIPCC, "-O2", "-std=c++17", "--offload-arch=gfx950", "-I", os.path.join(ROOT, "include"),
+          os.path.join(ROOT, "tests", "cabi_driver.cpp"), "-o", out, f"-L{HERE}", "-lmoe_gfx950", "-ldl", "-Wl,-rpath,$ORIGIN"])
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--no-ext", action="store_true", help="skip the torch/pybind11 module")
     args = ap.parse_args()
     build_kernels()
+    build_cabi_driver()
     if not args.no_ext:
         build_extension()
 
