@@ -398,16 +398,38 @@ __device__ __forceinline__ void lds_load16(rsrc_t r, const u32x4_t* dst, int vof
 // weight row 64 cw + 16 t + i, whose 8 codes of the sub-step are one dword; the scales [N, K/block] are
 // fetched 16 bytes per row at a time into buffers of their own (see kc_issue_scale).
 // ---------------------------------------------------------------------------------
+// Kernel variants.
+//   GK_GENERAL  4 wavefronts of 64 columns, one workgroup per CU, tiles of up to 176 rows (bf16 only)
+//   GK_SKINNY   the same tile routine with tiles of at most 32 rows and several workgroups per CU
+//               (decode-sized batches are HBM bound: more weight bytes in flight)
+//   GK_PAIR     quantized containers: 8 wavefronts, k range split between the two wavefronts of a SIMD, tiles of
+//               up to 160 rows
+//   GK_PAIR_SMALL  GK_PAIR with tiles of at most 32 rows: x stages of 4 KB leave LDS for a second workgroup per
+//               CU (decode-sized batches on the 4-bit containers)
+//   GK_PAIR_EXACT  GK_PAIR_SMALL with the GEMV op's arithmetic (weights not rounded to bf16)
+enum { GK_GENERAL = 0, GK_SKINNY = 1, GK_PAIR = 2, GK_PAIR_EXACT = 3, GK_PAIR_SMALL = 4 };
+
 constexpr int PAIR_CAPB = 10;                         // x stages hold 160 rows
 constexpr int PAIR_MT_MAX = 10;
-constexpr int PAIR_EXACT_MT_MAX = 2;                  // row blocks per tile with the GEMV op's arithmetic
-// 16-byte units of one x stage: 160 rows, or the 32 rows of the GEMV op's tiles (whose small stages let two
-// workgroups share a CU: one computes while the other waits at its barrier)
-constexpr int pair_a_units(bool exact) { return 16 * (exact ? PAIR_EXACT_MT_MAX : PAIR_CAPB) * 8; }
+constexpr int PAIR_SMALL_MT_MAX = 2;                  // row blocks per tile of the small-stage kinds
+constexpr bool pair_small(int kind) { return kind != GK_PAIR; }
+// 16-byte units of one x stage: 160 rows, or the 32 rows of the small-stage kinds
+constexpr int pair_a_units(int kind) { return 16 * (pair_small(kind) ? PAIR_SMALL_MT_MAX : PAIR_CAPB) * 8; }
 // packed tile of one k step: 64 rows of 128 bytes (4-bit codes) or of 256 bytes (int8, fp8)
 template <int FMT>
 constexpr int pair_b_units() { return (FMT == MOE_FMT_INT8 || FMT == MOE_FMT_FP8_REF) ? 64 * 16 : 64 * 8; }
-// ring depth: what fits into LDS next to the x stages
+// Small-stage kinds on the 4-bit N-contiguous containers: two workgroups per CU, one computes while the other
+// waits at its barrier or between two tiles (512 rows over 256 experts of 7168 x 2048: int4 425 -> 387 us, fp4
+// 440 -> 425 us; the fp4 tile routine with the GEMV op's arithmetic needs 151 registers, too many for four
+// wavefronts per SIMD).  A deeper ring in the LDS the small x stages free does not pay instead (fp4 10 stages
+// 515 us against 510 us with 5; fp8 7 stages 572 us against 552 us with 4: a tile's first stages take longer
+// to fill), and the one-byte containers at two workgroups per CU are left with 3 stages (fp8 641 us).
+template <int FMT>
+constexpr int pair_wg_per_cu(int kind) {
+    if (!pair_small(kind)) return 1;
+    return (FMT == MOE_FMT_INT4 || (FMT == MOE_FMT_FP4_REF && kind == GK_PAIR_SMALL)) ? 2 : 1;
+}
+// ring depth: what fits into LDS next to the 160-row x stages
 template <int FMT>
 constexpr int pair_stages() { return (FMT == MOE_FMT_INT8 || FMT == MOE_FMT_FP8_REF) ? 4 : 5; }
 // 16-byte units of scales per k step: rows of 256 bf16, int4 one per 32-k sub-step (groups are multiples
@@ -420,8 +442,8 @@ constexpr int pair_sc_units() { return FMT == MOE_FMT_FP4_REF ? 128 : FMT == MOE
 template <int FMT>
 constexpr int pair_kc_scale_units() { return (FMT == MOE_FMT_FP4_B32 || FMT == MOE_FMT_FP4_B16) ? 3 * 256 : 0; }
 template <int FMT>
-constexpr int pair_lds_units(bool exact) {
-    return pair_stages<FMT>() * (pair_a_units(exact) + pair_b_units<FMT>() + pair_sc_units<FMT>()) + pair_kc_scale_units<FMT>();
+constexpr int pair_lds_units(int kind) {
+    return pair_stages<FMT>() * (pair_a_units(kind) + pair_b_units<FMT>() + pair_sc_units<FMT>()) + pair_kc_scale_units<FMT>();
 }
 
 // End of a k-split tile.  The two wavefronts of a pair (same columns, the two k halves) hold partial sums of the
@@ -520,9 +542,10 @@ __device__ __forceinline__ void pair_finish(const GemmParams& P, u32x4_t* smem, 
 // scale on the way into the accumulators.  The fp4 container has a scale per 16 k, half an MFMA: the x
 // fragment is split into its lanes q < 2 and q >= 2 (the other half zeroed) and each half takes its
 // own MFMA.  These MFMAs are compiler-visible builtins (their results feed ordinary VALU code).
-template <int FMT, int MT, bool EXACT = false>
+template <int FMT, int MT, int KIND>
 __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* smem, int g, int64_t row0, int rows, int n0) {
     static_assert(FMT != MOE_FMT_BF16, "the k-split tile routine decodes quantized containers");
+    constexpr bool EXACT = KIND == GK_PAIR_EXACT;
     static_assert(!EXACT || FMT == MOE_FMT_INT4 || FMT == MOE_FMT_FP4_REF || FMT == MOE_FMT_FP8_REF,
                   "un-rounded weights: the N-contiguous containers of the GEMV op");
     constexpr bool FP4 = FMT == MOE_FMT_FP4_REF, I8 = FMT == MOE_FMT_INT8, F8 = FMT == MOE_FMT_FP8_REF;
@@ -533,7 +556,7 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
     constexpr int BK = 64, S = pair_stages<FMT>(), PAIR_SC_UNITS = pair_sc_units<FMT>();
     constexpr int PAIR_B_UNITS = pair_b_units<FMT>();
     constexpr int AHEAD = S - 1;   // a step's loads fill the stage of step kt + AHEAD
-    constexpr int PAIR_A_UNITS = pair_a_units(EXACT);
+    constexpr int PAIR_A_UNITS = pair_a_units(KIND);
     static_assert(16 * MT * 8 <= PAIR_A_UNITS, "tile rows beyond the x stage");
     u32x4_t* lds_a = smem;
     u32x4_t* lds_b = lds_a + S * PAIR_A_UNITS;
@@ -1004,28 +1027,22 @@ __device__ __forceinline__ void expert_chunks(int m, int& chunks, int& bpc) {
     bpc = chunks ? (nblk + chunks - 1) / chunks : 0;
 }
 
-// Kernel variants.
-//   GK_GENERAL  4 wavefronts of 64 columns, one workgroup per CU, tiles of up to 176 rows (bf16 only)
-//   GK_SKINNY   the same tile routine with tiles of at most 32 rows and several workgroups per CU
-//               (decode-sized batches are HBM bound: more weight bytes in flight)
-//   GK_PAIR     N-contiguous containers: 8 wavefronts, k range split between the two wavefronts of a SIMD
-//   GK_PAIR_EXACT  GK_PAIR with the GEMV op's arithmetic (weights not rounded to bf16), tiles of at most 32 rows
-enum { GK_GENERAL = 0, GK_SKINNY = 1, GK_PAIR = 2, GK_PAIR_EXACT = 3 };
 template <int FMT, int KIND>
 struct KernelCfg {
-    static constexpr bool PAIR = KIND == GK_PAIR || KIND == GK_PAIR_EXACT;
+    static constexpr bool PAIR = KIND == GK_PAIR || KIND == GK_PAIR_EXACT || KIND == GK_PAIR_SMALL;
     static constexpr bool SKINNY = KIND == GK_SKINNY;
     static_assert(!PAIR || FMT != MOE_FMT_BF16, "the k-split tile routine decodes quantized containers");
     static constexpr int WAVES = PAIR ? 8 : 4;
     static constexpr int BN = GM_BN;                                             // columns per tile
-    // the 4-bit containers with the GEMV op's arithmetic: two workgroups per CU (their stages hold 32 rows of x)
-    static constexpr bool TWO_PER_CU = KIND == GK_PAIR_EXACT && FMT == MOE_FMT_INT4;
-    static constexpr int WG_PER_CU = SKINNY ? GM_SKINNY_WAVES : TWO_PER_CU ? 2 : 1;
+    static constexpr int pair_wgs() {
+        if constexpr (PAIR) return pair_wg_per_cu<FMT>(KIND); else return 1;
+    }
+    static constexpr int WG_PER_CU = SKINNY ? GM_SKINNY_WAVES : pair_wgs();
     static constexpr int WAVES_PER_SIMD = WG_PER_CU * (PAIR ? 2 : 1);
     static constexpr int CAPB = SKINNY ? GM_SKINNY_BLOCKS : PAIR ? PAIR_CAPB : GM_MT_MAX;
     static constexpr int fmt_mt_max() {
         if constexpr (PAIR)
-            return KIND == GK_PAIR ? PAIR_MT_MAX : PAIR_EXACT_MT_MAX;
+            return KIND == GK_PAIR ? PAIR_MT_MAX : PAIR_SMALL_MT_MAX;
         else
             return BTraits<FMT>::MT_MAX;
     }
@@ -1033,7 +1050,7 @@ struct KernelCfg {
     // 16-byte LDS units of the tile routine (the tile prefix array follows them)
     static constexpr int lds_units() {
         if constexpr (PAIR)
-            return pair_lds_units<FMT>(KIND == GK_PAIR_EXACT);
+            return pair_lds_units<FMT>(KIND);
         else
             return 2 * 16 * CAPB * (BTraits<FMT>::BK / 8);
     }
@@ -1043,7 +1060,7 @@ template <int FMT, int MT, int KIND>
 __device__ __forceinline__ void run_tile(const GemmParams& P, u32x4_t* smem, int g, int64_t row0, int rows, int n0) {
     using C = KernelCfg<FMT, KIND>;
     if constexpr (C::PAIR)
-        gemm_tile_pair<FMT, MT, KIND == GK_PAIR_EXACT>(P, smem, g, row0, rows, n0);
+        gemm_tile_pair<FMT, MT, KIND>(P, smem, g, row0, rows, n0);
     else
         gemm_tile<FMT, MT, C::CAPB>(P, smem, g, row0, rows, n0);
 }
@@ -1209,6 +1226,11 @@ static int launch_gemm_fmt(const moe_grouped_args* a, hipStream_t stream) {
     // small-tile kernel down to decode batches of 1-2 rows per expert (256 experts of 7168 x 2048: int4
     // 243 vs 344 us at 128 rows, fp4 476 vs 519 us and fp8 610 vs 784 us at 512 rows).
     if constexpr (FMT != MOE_FMT_BF16) {
+        // decode-like batches (on average at most 12 rows per expert) on the 4-bit N-contiguous containers: the
+        // small-stage kind (at 8 rows per expert int4 409 vs 506 us, fp4 448 vs 474 us; at 24 the large tiles win,
+        // 531 vs 549 us and 512 vs 609 us).  The one-byte containers gain nothing from it.
+        if constexpr (FMT == MOE_FMT_INT4 || FMT == MOE_FMT_FP4_REF)
+            if (a->M <= 12 * a->G) return launch_gemm_kind<FMT, GK_PAIR_SMALL>(P, a, stream);
         return launch_gemm_kind<FMT, GK_PAIR>(P, a, stream);
     } else {
         // Decode-like batches (on average at most 24 rows per expert; group_list itself stays on the
