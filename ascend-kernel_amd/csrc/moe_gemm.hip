@@ -48,6 +48,27 @@ struct GemmParams {
     int64_t M;
     int K, N, G, scale_rows;
     int epilogue;   // moe_epilogue
+    int slot;       // this launch's pair of counters in tile_queue
+};
+
+// Work queue of the persistent grid.  Workgroups do not run at one speed (of two that share a CU the one
+// placed first runs about 1.5 times as fast as the other while both are resident, and the XCDs differ by a few
+// per cent), so an even split of the tiles leaves most of the chip waiting for the slowest workgroup.  All but
+// the last two or three tiles of a workgroup's share are handed out in a fixed, XCD-aware order; the rest
+// are taken one at a time from a counter.  Every launch gets a slot (next tile, workgroups done) of its
+// own, so that launches on different streams do not share a counter; the last workgroup to finish puts both
+// back to zero, the state device memory starts in.  Two launches collide only if GM_QUEUE_SLOTS launches
+// later the first is still running.
+constexpr int GM_QUEUE_SLOTS = 1024;
+constexpr int GM_QUEUE_TAIL_SWEEPS = 2;   // tiles per workgroup that are left to the counter (plus the remainder)
+__device__ unsigned int tile_queue[GM_QUEUE_SLOTS * 2];
+static std::atomic<unsigned> queue_launches{0};   // launches of every kind of kernel in this file, for the slot
+// A tile routine that is handed a counter takes the workgroup's next tile from it while it finishes its own
+// (the counter's round trip, about 3 us under load, overlaps the tile's reduction and stores) and leaves the
+// result in *out behind its last barrier.
+struct Ticket {
+    unsigned int* counter;   // null: the caller takes the next tile itself
+    int* out;
 };
 
 // Buffer resources keep the addressing compact: one 128-bit descriptor in SGPRs per
@@ -453,8 +474,11 @@ constexpr int pair_lds_units(int kind) {
 // blocks (8 wavefronts x 4 blocks x 4 KB fit the x stage area, free now).
 template <int MT, bool KC>
 __device__ __forceinline__ void pair_finish(const GemmParams& P, u32x4_t* smem, f32x4_t (&acc)[MT][4], int h, int cw, int lane,
-                                            int col0, int64_t row0, int rows, int n0) {
+                                            int col0, int64_t row0, int rows, int n0, const Ticket& tk) {
     const int i = lane & 15, q = lane >> 4;
+    const bool takes = tk.counter != nullptr && threadIdx.x == 0;
+    unsigned int next_tile = 0;
+    if (takes) next_tile = atomicAdd(tk.counter, 1u);
     constexpr int MH = (MT + 1) / 2, RR = MH < 4 ? MH : 4, ROUNDS = (MH + RR - 1) / RR;
     // the last tile of an N that is not a multiple of 256 (the reference's fp8 container: multiples of 128)
     // computes columns past N from whatever follows in the slab: they are not stored
@@ -533,6 +557,7 @@ __device__ __forceinline__ void pair_finish(const GemmParams& P, u32x4_t* smem, 
         finish(std::integral_constant<int, 0>{});
     else
         finish(std::integral_constant<int, 1>{});
+    if (takes) *tk.out = (int)next_tile;
     __syncthreads();   // the slots are read: the next tile may load into the ring
 }
 
@@ -543,7 +568,7 @@ __device__ __forceinline__ void pair_finish(const GemmParams& P, u32x4_t* smem, 
 // fragment is split into its lanes q < 2 and q >= 2 (the other half zeroed) and each half takes its
 // own MFMA.  These MFMAs are compiler-visible builtins (their results feed ordinary VALU code).
 template <int FMT, int MT, int KIND>
-__device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* smem, int g, int64_t row0, int rows, int n0) {
+__device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* smem, int g, int64_t row0, int rows, int n0, const Ticket& tk) {
     static_assert(FMT != MOE_FMT_BF16, "the k-split tile routine decodes quantized containers");
     constexpr bool EXACT = KIND == GK_PAIR_EXACT;
     static_assert(!EXACT || FMT == MOE_FMT_INT4 || FMT == MOE_FMT_FP4_REF || FMT == MOE_FMT_FP8_REF,
@@ -1010,7 +1035,7 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
     // accumulators were last written by MFMAs the compiler cannot see: wait out their latency
     asm volatile("s_waitcnt vmcnt(0)\n\ts_nop 15\n\ts_nop 15\n\ts_barrier" ::: "memory");
 
-    pair_finish<MT, KC>(P, smem, acc, h, cw, lane, col0, row0, rows, n0);
+    pair_finish<MT, KC>(P, smem, acc, h, cw, lane, col0, row0, rows, n0, tk);
 }
 
 // ---------------------------------------------------------------------------------
@@ -1057,10 +1082,10 @@ struct KernelCfg {
 };
 
 template <int FMT, int MT, int KIND>
-__device__ __forceinline__ void run_tile(const GemmParams& P, u32x4_t* smem, int g, int64_t row0, int rows, int n0) {
+__device__ __forceinline__ void run_tile(const GemmParams& P, u32x4_t* smem, int g, int64_t row0, int rows, int n0, const Ticket& tk) {
     using C = KernelCfg<FMT, KIND>;
     if constexpr (C::PAIR)
-        gemm_tile_pair<FMT, MT, KIND>(P, smem, g, row0, rows, n0);
+        gemm_tile_pair<FMT, MT, KIND>(P, smem, g, row0, rows, n0, tk);
     else
         gemm_tile<FMT, MT, C::CAPB>(P, smem, g, row0, rows, n0);
 }
@@ -1075,10 +1100,10 @@ __global__ __launch_bounds__((64 * KernelCfg<FMT, KIND>::WAVES), (KernelCfg<FMT,
     int* prefix = reinterpret_cast<int*>(smem + C::lds_units());      // [G + 1]
     const int tid = threadIdx.x;
     const int ntile_n = (P.N + C::BN - 1) / C::BN;
+    __shared__ int part[THREADS];   // scan partials; part[0] later carries the tile taken from the queue
 
     // exclusive scan of tiles per expert: each thread takes a contiguous run of experts
     {
-        __shared__ int part[THREADS];
         const int per = (P.G + THREADS - 1) / THREADS;
         const int g0 = tid * per, g1 = min(P.G, g0 + per);
         int sum = 0;
@@ -1115,9 +1140,29 @@ __global__ __launch_bounds__((64 * KernelCfg<FMT, KIND>::WAVES), (KernelCfg<FMT,
     const int nwg = gridDim.x;
     const int per_xcd = (nwg + 7) / 8;
     const int vid = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
-    const int sweep = per_xcd * 8;
+    const int sweep = per_xcd * 8;   // == nwg: the grid is a multiple of 8
+    const int fixed_sweeps = max(0, total / sweep - GM_QUEUE_TAIL_SWEEPS);
+    unsigned int* q_next = tile_queue + 2 * P.slot;
+    unsigned int* q_done = q_next + 1;
 
-    for (int T = vid; T < total; T += sweep) {
+    bool have_ticket = false;   // the previous tile routine left the next tile in part[0]
+    for (int sw = 0;; ++sw) {
+        int T;
+        if (sw < fixed_sweeps) {
+            T = sw * sweep + vid;
+        } else {
+            if (!have_ticket) {
+                __syncthreads();   // part[0] of the previous round is read (the scan's part[], the first time)
+                if (tid == 0) part[0] = (int)atomicAdd(q_next, 1u);
+                __syncthreads();
+            }
+            T = fixed_sweeps * sweep + __builtin_amdgcn_readfirstlane(part[0]);
+            if (T >= total) break;
+        }
+        // from the last tile of the fixed order on, the k-split tile routines fetch the next tile themselves
+        const bool take = C::PAIR && sw + 1 >= fixed_sweeps;
+        const Ticket tk = {take ? q_next : nullptr, part};
+        have_ticket = take;
         // largest g with prefix[g] <= T (empty experts have prefix[g] == prefix[g+1])
         int lo = 0, hi = P.G;
         while (hi - lo > 1) {
@@ -1143,43 +1188,48 @@ __global__ __launch_bounds__((64 * KernelCfg<FMT, KIND>::WAVES), (KernelCfg<FMT,
         const int n0 = nt * C::BN;
         switch (mt) {
             case 1:
-                if constexpr (MTM >= 1) run_tile<FMT, 1, KIND>(P, smem, g, row0, rows, n0);
+                if constexpr (MTM >= 1) run_tile<FMT, 1, KIND>(P, smem, g, row0, rows, n0, tk);
                 break;
             case 2:
-                if constexpr (MTM >= 2) run_tile<FMT, 2, KIND>(P, smem, g, row0, rows, n0);
+                if constexpr (MTM >= 2) run_tile<FMT, 2, KIND>(P, smem, g, row0, rows, n0, tk);
                 break;
             case 3:
-                if constexpr (MTM >= 3) run_tile<FMT, 3, KIND>(P, smem, g, row0, rows, n0);
+                if constexpr (MTM >= 3) run_tile<FMT, 3, KIND>(P, smem, g, row0, rows, n0, tk);
                 break;
             case 4:
-                if constexpr (MTM >= 4) run_tile<FMT, 4, KIND>(P, smem, g, row0, rows, n0);
+                if constexpr (MTM >= 4) run_tile<FMT, 4, KIND>(P, smem, g, row0, rows, n0, tk);
                 break;
             case 5:
-                if constexpr (MTM >= 5) run_tile<FMT, 5, KIND>(P, smem, g, row0, rows, n0);
+                if constexpr (MTM >= 5) run_tile<FMT, 5, KIND>(P, smem, g, row0, rows, n0, tk);
                 break;
             case 6:
-                if constexpr (MTM >= 6) run_tile<FMT, 6, KIND>(P, smem, g, row0, rows, n0);
+                if constexpr (MTM >= 6) run_tile<FMT, 6, KIND>(P, smem, g, row0, rows, n0, tk);
                 break;
             case 7:
-                if constexpr (MTM >= 7) run_tile<FMT, 7, KIND>(P, smem, g, row0, rows, n0);
+                if constexpr (MTM >= 7) run_tile<FMT, 7, KIND>(P, smem, g, row0, rows, n0, tk);
                 break;
             case 8:
-                if constexpr (MTM >= 8) run_tile<FMT, 8, KIND>(P, smem, g, row0, rows, n0);
+                if constexpr (MTM >= 8) run_tile<FMT, 8, KIND>(P, smem, g, row0, rows, n0, tk);
                 break;
             case 9:
-                if constexpr (MTM >= 9) run_tile<FMT, 9, KIND>(P, smem, g, row0, rows, n0);
+                if constexpr (MTM >= 9) run_tile<FMT, 9, KIND>(P, smem, g, row0, rows, n0, tk);
                 break;
             case 10:
-                if constexpr (MTM >= 10) run_tile<FMT, 10, KIND>(P, smem, g, row0, rows, n0);
+                if constexpr (MTM >= 10) run_tile<FMT, 10, KIND>(P, smem, g, row0, rows, n0, tk);
                 break;
             case 11:
-                if constexpr (MTM >= 11) run_tile<FMT, 11, KIND>(P, smem, g, row0, rows, n0);
+                if constexpr (MTM >= 11) run_tile<FMT, 11, KIND>(P, smem, g, row0, rows, n0, tk);
                 break;
             case 12:
-                if constexpr (MTM >= 12) run_tile<FMT, 12, KIND>(P, smem, g, row0, rows, n0);
+                if constexpr (MTM >= 12) run_tile<FMT, 12, KIND>(P, smem, g, row0, rows, n0, tk);
                 break;
-            default: break;
+            default: have_ticket = false; break;
         }
+    }
+    // every workgroup has taken its last (failed) ticket; the last one to arrive here re-arms the slot
+    if (tid == 0 && atomicAdd(q_done, 1u) == (unsigned)nwg - 1u) {
+        atomicExch(q_next, 0u);
+        atomicExch(q_done, 0u);
     }
 }
 
@@ -1202,7 +1252,9 @@ static int launch_gemm_kind(const GemmParams& P, const moe_grouped_args* a, hipS
     const int64_t want = max_tiles < (int64_t)cus * C::WG_PER_CU ? max_tiles : (int64_t)cus * C::WG_PER_CU;
     // a multiple of 8 so that the XCD-aware order covers every tile index
     const int64_t grid = want > 0 ? (want + 7) / 8 * 8 : 8;
-    hipLaunchKernelGGL((grouped_gemm_kernel<FMT, KIND>), dim3((unsigned)grid), dim3(64 * C::WAVES), lds, stream, P);
+    GemmParams Q = P;
+    Q.slot = (int)(queue_launches.fetch_add(1, std::memory_order_relaxed) % GM_QUEUE_SLOTS);
+    hipLaunchKernelGGL((grouped_gemm_kernel<FMT, KIND>), dim3((unsigned)grid), dim3(64 * C::WAVES), lds, stream, Q);
     return hipGetLastError() == hipSuccess ? MOE_OK : MOE_ERR_LAUNCH;
 }
 
@@ -1216,6 +1268,7 @@ static GemmParams gemm_params(const moe_grouped_args* a) {
     P.y = static_cast<uint16_t*>(a->y);
     P.M = a->M; P.K = (int)a->K; P.N = (int)a->N; P.G = (int)a->G; P.scale_rows = (int)a->scale_rows;
     P.epilogue = a->epilogue;
+    P.slot = 0;
     return P;
 }
 

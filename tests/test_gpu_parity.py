@@ -197,6 +197,38 @@ def test_gemm_decode_batches_on_the_small_tile_kind(fmt, shape):
     assert (got[gl[-1]:] == 0x7FC0).all()
 
 
+def test_gemm_tile_queue_is_rearmed_after_every_launch():
+    """The persistent grid takes its last tiles from a counter in device memory; every launch uses one of 1024
+    counter slots and must leave it at zero.  More launches than slots, on two streams, with more tiles than
+    workgroups: a slot that was not put back would make a later launch skip tiles (rows left unwritten)."""
+    import moe_gfx950 as mg
+    _say("gemm tile queue: 2300 launches")
+    rng = np.random.default_rng(5)
+    counts = rng.choice([0, 1, 3, 16, 17, 33], 40)
+    gl = list(np.cumsum(counts))
+    cases = [H.make_case(fmt, len(gl), 128, 2048, gl, seed=7 + i, group=64) for i, fmt in enumerate(("int4", "bf16"))]
+    devs = [H.upload(c) for c in cases]
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    p = lambda t: 0 if t is None else t.data_ptr()
+    ys, argss = [], []
+    for c, d in zip(cases, devs):
+        y = torch.full((c["M"], c["N"]), 0x7FC0, dtype=torch.int16, device="cuda")
+        ys.append(y)
+        argss.append(mg.grouped_args(mg.format_from_compute_type(c["fmt"]), p(d["x"]), p(d["weight"]), p(d["scale"]),
+                                     p(d["offset"]), p(d["group_list"]), p(y), c["M"], c["K"], c["N"], c["G"], c["scale_rows"]))
+    torch.cuda.synchronize()
+    for it in range(1150):
+        for st, args in zip(streams, argss):
+            mg.grouped_gemm(args, st.cuda_stream)
+        if it in (0, 600, 1149):
+            torch.cuda.synchronize()
+            for c, y in zip(cases, ys):
+                got = y.cpu().numpy().view(np.uint16)
+                H.assert_close(got, H.oracle_out(c), rows=slice(0, gl[-1]), what=f"launch {it} {c['fmt']}")
+                y.fill_(0x7FC0)
+            torch.cuda.synchronize()
+
+
 def test_gemm_int4_group_size_32_and_64():
     for group in (32, 64, 256):
         _say(f"gemm int4 group={group}")
