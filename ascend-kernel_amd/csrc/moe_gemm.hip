@@ -428,27 +428,31 @@ __device__ __forceinline__ void lds_load16(rsrc_t r, const u32x4_t* dst, int vof
 //   GK_PAIR_SMALL  GK_PAIR with tiles of at most 32 rows: x stages of 4 KB leave LDS for a second workgroup per
 //               CU (decode-sized batches on the 4-bit containers)
 //   GK_PAIR_EXACT  GK_PAIR_SMALL with the GEMV op's arithmetic (weights not rounded to bf16)
-enum { GK_GENERAL = 0, GK_SKINNY = 1, GK_PAIR = 2, GK_PAIR_EXACT = 3, GK_PAIR_SMALL = 4 };
+//   GK_PAIR_EXACT16  GK_PAIR_EXACT with tiles of at most 16 rows (the fp4 container: its 32-row tile routine
+//               needs 153 registers, the 16-row one 97, which lets two workgroups share a CU)
+enum { GK_GENERAL = 0, GK_SKINNY = 1, GK_PAIR = 2, GK_PAIR_EXACT = 3, GK_PAIR_SMALL = 4, GK_PAIR_EXACT16 = 5 };
+constexpr bool pair_exact(int kind) { return kind == GK_PAIR_EXACT || kind == GK_PAIR_EXACT16; }
 
 constexpr int PAIR_CAPB = 10;                         // x stages hold 160 rows
 constexpr int PAIR_MT_MAX = 10;
 constexpr int PAIR_SMALL_MT_MAX = 2;                  // row blocks per tile of the small-stage kinds
 constexpr bool pair_small(int kind) { return kind != GK_PAIR; }
 // 16-byte units of one x stage: 160 rows, or the 32 rows of the small-stage kinds
-constexpr int pair_a_units(int kind) { return 16 * (pair_small(kind) ? PAIR_SMALL_MT_MAX : PAIR_CAPB) * 8; }
+constexpr int pair_mt_max(int kind) { return kind == GK_PAIR ? PAIR_MT_MAX : kind == GK_PAIR_EXACT16 ? 1 : PAIR_SMALL_MT_MAX; }
+constexpr int pair_a_units(int kind) { return 16 * (pair_small(kind) ? pair_mt_max(kind) : PAIR_CAPB) * 8; }
 // packed tile of one k step: 64 rows of 128 bytes (4-bit codes) or of 256 bytes (int8, fp8)
 template <int FMT>
 constexpr int pair_b_units() { return (FMT == MOE_FMT_INT8 || FMT == MOE_FMT_FP8_REF) ? 64 * 16 : 64 * 8; }
 // Small-stage kinds on the 4-bit N-contiguous containers: two workgroups per CU, one computes while the other
 // waits at its barrier or between two tiles (512 rows over 256 experts of 7168 x 2048: int4 425 -> 387 us, fp4
-// 440 -> 425 us; the fp4 tile routine with the GEMV op's arithmetic needs 151 registers, too many for four
-// wavefronts per SIMD).  A deeper ring in the LDS the small x stages free does not pay instead (fp4 10 stages
+// 440 -> 425 us; the fp4 tile routine with the GEMV op's arithmetic fits four wavefronts per SIMD only in its
+// 16-row form).  A deeper ring in the LDS the small x stages free does not pay instead (fp4 10 stages
 // 515 us against 510 us with 5; fp8 7 stages 572 us against 552 us with 4: a tile's first stages take longer
 // to fill), and the one-byte containers at two workgroups per CU are left with 3 stages (fp8 641 us).
 template <int FMT>
 constexpr int pair_wg_per_cu(int kind) {
     if (!pair_small(kind)) return 1;
-    return (FMT == MOE_FMT_INT4 || (FMT == MOE_FMT_FP4_REF && kind == GK_PAIR_SMALL)) ? 2 : 1;
+    return (FMT == MOE_FMT_INT4 || (FMT == MOE_FMT_FP4_REF && kind != GK_PAIR_EXACT)) ? 2 : 1;
 }
 // ring depth: what fits into LDS next to the 160-row x stages
 template <int FMT>
@@ -567,10 +571,19 @@ __device__ __forceinline__ void pair_finish(const GemmParams& P, u32x4_t* smem, 
 // scale on the way into the accumulators.  The fp4 container has a scale per 16 k, half an MFMA: the x
 // fragment is split into its lanes q < 2 and q >= 2 (the other half zeroed) and each half takes its
 // own MFMA.  These MFMAs are compiler-visible builtins (their results feed ordinary VALU code).
-template <int FMT, int MT, int KIND>
+//
+// STACK2 (that arithmetic on the fp4 container, tiles of at most 8 rows): the two scale groups of an MFMA's 32 k
+// are told apart by the row of the 16 x 16 product instead of by two MFMAs.  Row r < 8 of the x fragment holds
+// x row r in its first 16 k and zeros in the others, row 8 + r holds x row r in the last 16 k only (the zeros are
+// read from the rows 8..15 of the x stage, which are padding for such a tile).  One MFMA per 16 columns then
+// leaves the first group's sums in the lanes q < 2 and the second group's in q >= 2, each lane applies the
+// scale of its own group, and the two halves are added once at the end of the tile: half the MFMAs and half
+// the multiplies of the general case, and no masking.
+template <int FMT, int MT, int KIND, bool STACK2 = false>
 __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* smem, int g, int64_t row0, int rows, int n0, const Ticket& tk) {
     static_assert(FMT != MOE_FMT_BF16, "the k-split tile routine decodes quantized containers");
-    constexpr bool EXACT = KIND == GK_PAIR_EXACT;
+    constexpr bool EXACT = pair_exact(KIND);
+    static_assert(!STACK2 || (EXACT && FMT == MOE_FMT_FP4_REF && MT == 1), "two scale groups stacked in one MFMA: fp4, at most 8 rows");
     static_assert(!EXACT || FMT == MOE_FMT_INT4 || FMT == MOE_FMT_FP4_REF || FMT == MOE_FMT_FP8_REF,
                   "un-rounded weights: the N-contiguous containers of the GEMV op");
     constexpr bool FP4 = FMT == MOE_FMT_FP4_REF, I8 = FMT == MOE_FMT_INT8, F8 = FMT == MOE_FMT_FP8_REF;
@@ -695,6 +708,8 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
     asm volatile("" : "+s"(mask), "+s"(sel));   // kept opaque so that each stays one SGPR operand
     const int d = 16 * (cw >> 1) + i;            // dword column of this lane
     const int unit = (d >> 2) ^ (4 * (q & 1));
+    // row of the x stage this lane's fragment row i comes from (STACK2: see above)
+    const int xrow = STACK2 ? (((i >> 3) == (q >> 1)) ? (i & 7) : 8 + (i & 7)) : i;
 
     // The accumulators are zeroed by asm so that the compiler cannot re-materialize the zeros
     // right in front of the first MFMA that accumulates into them: a VALU write of an MFMA's
@@ -757,7 +772,7 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
             const u32x4_t lo4 = tb[(2 * (i & 3)) ^ swz], hi4 = tb[(2 * (i & 3) + 1) ^ swz];
 #pragma unroll
             for (int j = 0; j < 4; ++j) { r[j] = lo4[j]; r[4 + j] = hi4[j]; }
-            if constexpr (EXACT) {
+            if constexpr (EXACT && !STACK2) {
                 sc = *reinterpret_cast<const u32x2_t*>(sc16 + 256 * (2 * h) + col0);
                 sc2 = *reinterpret_cast<const u32x2_t*>(sc16 + 256 * (2 * h + 1) + col0);
             } else {
@@ -830,7 +845,7 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
                 }
                 // first x fragments of the MFMA phase, read under the rest of the decode
 #pragma unroll
-                for (int f = 0; f < R; ++f) afr[f & 3] = la[a_lds_unit<BK>(16 * f + i, 4 * h + q)];
+                for (int f = 0; f < R; ++f) afr[f & 3] = la[a_lds_unit<BK>(16 * f + xrow, 4 * h + q)];
             }
             if constexpr (KC) {
                 // dword r[t] = 8 consecutive k of MFMA t's weight row: byte p = the k pair p
@@ -978,10 +993,18 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
         // barrier) are fetched between the MFMAs.
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
-            if (mt + R < MT) afr[(mt + R) & 3] = la[a_lds_unit<BK>(16 * (mt + R) + i, 4 * h + q)];
+            if (mt + R < MT) afr[(mt + R) & 3] = la[a_lds_unit<BK>(16 * (mt + R) + xrow, 4 * h + q)];
             if constexpr (EXACT) {
                 const f32x4_t zero = {0.f, 0.f, 0.f, 0.f};
-                if constexpr (FP4) {
+                if constexpr (STACK2) {
+#pragma unroll
+                    for (int t = 0; t < 4; ++t) {
+                        const f32x4_t dd = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                            __builtin_bit_cast(bf16x8_t, afr[mt & 3]), __builtin_bit_cast(bf16x8_t, bf[t]), zero, 0, 0, 0);
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) acc[mt][t][e] = fmaf(dd[e], sa[t], acc[mt][t][e]);
+                    }
+                } else if constexpr (FP4) {
                     const uint32_t mlo = q < 2 ? 0xffffffffu : 0u;
                     u32x4_t xlo, xhi;
 #pragma unroll
@@ -1035,6 +1058,13 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
     // accumulators were last written by MFMAs the compiler cannot see: wait out their latency
     asm volatile("s_waitcnt vmcnt(0)\n\ts_nop 15\n\ts_nop 15\n\ts_barrier" ::: "memory");
 
+    if constexpr (STACK2) {
+        // the lanes q and q + 2 hold the two scale groups' sums of the same rows
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) acc[0][t][e] += __shfl_xor(acc[0][t][e], 32);
+    }
     pair_finish<MT, KC>(P, smem, acc, h, cw, lane, col0, row0, rows, n0, tk);
 }
 
@@ -1054,7 +1084,7 @@ __device__ __forceinline__ void expert_chunks(int m, int& chunks, int& bpc) {
 
 template <int FMT, int KIND>
 struct KernelCfg {
-    static constexpr bool PAIR = KIND == GK_PAIR || KIND == GK_PAIR_EXACT || KIND == GK_PAIR_SMALL;
+    static constexpr bool PAIR = KIND == GK_PAIR || KIND == GK_PAIR_SMALL || pair_exact(KIND);
     static constexpr bool SKINNY = KIND == GK_SKINNY;
     static_assert(!PAIR || FMT != MOE_FMT_BF16, "the k-split tile routine decodes quantized containers");
     static constexpr int WAVES = PAIR ? 8 : 4;
@@ -1067,7 +1097,7 @@ struct KernelCfg {
     static constexpr int CAPB = SKINNY ? GM_SKINNY_BLOCKS : PAIR ? PAIR_CAPB : GM_MT_MAX;
     static constexpr int fmt_mt_max() {
         if constexpr (PAIR)
-            return KIND == GK_PAIR ? PAIR_MT_MAX : PAIR_SMALL_MT_MAX;
+            return pair_mt_max(KIND);
         else
             return BTraits<FMT>::MT_MAX;
     }
@@ -1084,8 +1114,12 @@ struct KernelCfg {
 template <int FMT, int MT, int KIND>
 __device__ __forceinline__ void run_tile(const GemmParams& P, u32x4_t* smem, int g, int64_t row0, int rows, int n0, const Ticket& tk) {
     using C = KernelCfg<FMT, KIND>;
-    if constexpr (C::PAIR)
+    if constexpr (C::PAIR) {
+        if constexpr (FMT == MOE_FMT_FP4_REF && pair_exact(KIND) && MT == 1) {
+            if (rows <= 8) return gemm_tile_pair<FMT, MT, KIND, true>(P, smem, g, row0, rows, n0, tk);
+        }
         gemm_tile_pair<FMT, MT, KIND>(P, smem, g, row0, rows, n0, tk);
+    }
     else
         gemm_tile<FMT, MT, C::CAPB>(P, smem, g, row0, rows, n0);
 }
@@ -1297,7 +1331,11 @@ static int launch_gemm_fmt(const moe_grouped_args* a, hipStream_t stream) {
 int launch_gemm_exact(const moe_grouped_args* a, hipStream_t stream) {
     const GemmParams P = gemm_params(a);
     switch (a->format) {
-        case MOE_FMT_FP4_REF: return launch_gemm_kind<MOE_FMT_FP4_REF, GK_PAIR_EXACT>(P, a, stream);
+        case MOE_FMT_FP4_REF:
+            // decode-like batches (on average at most 12 rows per expert): 16-row tiles, two workgroups per CU; an
+            // expert with more rows than that costs a pass over its weights per 16 rows
+            if (a->M <= 12 * a->G) return launch_gemm_kind<MOE_FMT_FP4_REF, GK_PAIR_EXACT16>(P, a, stream);
+            return launch_gemm_kind<MOE_FMT_FP4_REF, GK_PAIR_EXACT>(P, a, stream);
         case MOE_FMT_INT4: return launch_gemm_kind<MOE_FMT_INT4, GK_PAIR_EXACT>(P, a, stream);
         case MOE_FMT_FP8_REF: return launch_gemm_kind<MOE_FMT_FP8_REF, GK_PAIR_EXACT>(P, a, stream);
         default: return MOE_ERR_BAD_FORMAT;

@@ -177,23 +177,25 @@ def test_several_tiles_per_workgroup(fmt, op):
     assert (got[gl[-1]:] == 0x7FC0).all()
 
 
+@pytest.mark.parametrize("op", ["gemm", "gemv"])
 @pytest.mark.parametrize("fmt", ["int4", "fp4"])
 @pytest.mark.parametrize("shape", ["row_counts", "many_tiles"])
-def test_gemm_decode_batches_on_the_small_tile_kind(fmt, shape):
+def test_decode_batches_on_the_small_tile_kinds(fmt, shape, op):
     """Batches of at most 12 rows per expert on average run the 4-bit N-contiguous containers in tiles of at most
-    32 rows, two workgroups per CU: experts of 0 to 70 rows (several row chunks per expert), and more tiles than
-    the grid has workgroups."""
-    _say(f"gemm small tiles fmt={fmt} {shape}")
+    32 rows (the GEMV op on fp4: 16 rows, with the two scale groups of an MFMA stacked for tiles of at most 8),
+    two workgroups per CU: experts of 0 to 70 rows (several row chunks per expert), and more tiles than the grid
+    has workgroups."""
+    _say(f"{op} small tiles fmt={fmt} {shape}")
     if shape == "row_counts":
-        counts, K, N = [1, 0, 4, 5, 16, 17, 32, 33, 70, 0, 3] + [0] * 6, 1024, 512
+        counts, K, N = [1, 0, 4, 5, 16, 17, 32, 33, 70, 0, 3, 8, 9, 7] + [0] * 8, 1024, 512
     else:
         rng = np.random.default_rng(zlib.crc32(f"small/{fmt}".encode()))
         counts, K, N = list(rng.choice([0] * 6 + [1, 3, 16, 17, 33, 40], 160)), 256, 2048
     gl = list(np.cumsum(counts))
     assert gl[-1] <= 12 * len(gl)
     case = H.make_case(fmt, len(gl), K, N, gl, seed=len(gl), extra_rows=2, group=64)
-    got = H.run_cabi(case, H.upload(case), "gemm")
-    H.assert_close(got, H.oracle_out(case), rows=slice(0, gl[-1]), what=f"small tiles {fmt}/{shape}")
+    got = H.run_cabi(case, H.upload(case), op)
+    H.assert_close(got, H.oracle_out(case, gemv=op == "gemv"), rows=slice(0, gl[-1]), what=f"small tiles {op} {fmt}/{shape}")
     assert (got[gl[-1]:] == 0x7FC0).all()
 
 
