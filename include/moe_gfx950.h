@@ -6,9 +6,13 @@
  * Every launch is asynchronous on the given stream, never synchronizes the
  * device, never copies group_list to the host and allocates nothing.  The only
  * state between calls is set-up done once per process or GPU (a kernel attribute,
- * the address of moe_route_static's scratch array); calls are re-entrant except
- * where moe_route_static says otherwise.  All functions return MOE_OK (0) or a
- * negative moe_status; nothing throws across this boundary.
+ * the address of moe_route_static's scratch array) and the tile counters of the
+ * grouped GEMM kernels: 8 KB of the library's own device memory, 1024 slots, each
+ * launch takes the next slot and its kernel leaves it at zero again, so launches
+ * may overlap on different streams and replay from HIP graphs (a launch would
+ * collide with another only if that one were still running 1024 launches later).
+ * Calls are re-entrant except where moe_route_static says otherwise.  All functions
+ * return MOE_OK (0) or a negative moe_status; nothing throws across this boundary.
  *
  * What each entry point replaces in the reference (paths relative to its tree):
  *   moe_grouped_gemm            aclnnGroupedMatmulAntiquant{GetWorkspaceSize,}

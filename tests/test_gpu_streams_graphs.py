@@ -1,4 +1,4 @@
-"""The C ABI's launch contract: asynchronous on the caller's stream, no allocation, no hidden state.
+"""The C ABI's launch contract: asynchronous on the caller's stream, no allocation, no state that outlives a launch.
 Checked by capturing the ops into a HIP graph and replaying it, and by calling them from several
 host threads on their own streams; results must equal the eager, single-stream ones bit for bit
 (every kernel here is deterministic)."""
