@@ -10,12 +10,14 @@
 // Work decomposition.  A tile is (expert, chunk of rows, 256 columns).  The tile list is derived
 // inside the kernel from the device-resident cumulative group_list (no host sync); a persistent
 // grid walks it with an XCD-aware order so that the workgroups of one XCD share the x rows and
-// weight slices of the same experts in that XCD's L2.  Every wavefront owns its columns for ALL
+// weight slices of the same experts in that XCD's L2, and takes the last two or three tiles of every
+// workgroup from a work counter (see tile_queue).  Every wavefront owns its columns for ALL
 // rows of the tile, so each weight element is dequantized exactly once per tile.  Two tile routines:
 //   gemm_tile_pair  every quantized container (int4, int8, the K-contiguous fp4 containers, the
 //                   reference's fp4 and fp8): 8 wavefronts, the two of a SIMD split the k range;
 //                   x, packed weights and scales arrive by LDS-direct loads into a ring of stages;
-//                   tiles of up to 160 rows (32 with the GEMV op's arithmetic)
+//                   tiles of up to 160 rows, or of up to 32 / 16 rows with small stages (decode batches,
+//                   and the GEMV op's arithmetic on the N-contiguous containers)
 //   gemm_tile       the bf16 container: 4 wavefronts of 64 columns, x through a double-buffered,
 //                   XOR-swizzled LDS tile, weights from registers; tiles of up to 176 rows, or 32 rows
 //                   and several workgroups per CU for decode-sized batches
