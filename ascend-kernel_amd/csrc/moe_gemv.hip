@@ -447,6 +447,10 @@ __device__ __forceinline__ uint32_t e2m1_pair_bf16(uint32_t word, int sel) {
 // q < 2 of a column hold its first half, q >= 2 the second, so with the GEMM's rounding each lane
 // simply uses its half's scale, and with the GEMV's arithmetic the block takes two MFMAs, each on
 // one half of the lanes' codes (the other half zeroed), each partial sum scaled by its own scale.
+// With at most 8 activation rows (STACK below) one MFMA does: fragment row r < 8 of x keeps only the first
+// 16 k of x row r, row 8 + r only the last 16 k, so the product's rows < 8 (lanes q < 2) are the first
+// scale's partial sums and rows >= 8 (q >= 2) the second's; each lane applies its own half's scale and the
+// halves are added once at the end.
 template <int MB, bool ROUNDW, int BLK>
 __device__ __forceinline__ void gemv_fp4_mfma_rows(const uint8_t* __restrict__ wg, const uint16_t* __restrict__ sg,
                                                    const uint16_t* __restrict__ x, uint16_t* __restrict__ y,
@@ -464,6 +468,9 @@ __device__ __forceinline__ void gemv_fp4_mfma_rows(const uint8_t* __restrict__ w
     const uint32_t soff = (uint32_t)nn * (uint32_t)(K / BLK) * 2;
     constexpr int PER = BLK / 8;                // loop iterations per 128 bytes (64 scales) of a scale row
     const bool hi_half = (q & 2) != 0;          // block 16: this lane's codes belong to the second scale of a block
+    constexpr bool STACK = BLK == 16 && !ROUNDW && MB <= 8;
+    // STACK: fragment row i of x is live only in the k half that matches i >> 3
+    const uint32_t x_keep = ((i >> 3) == (q >> 1)) ? 0xffffffffu : 0u;
     f32x4_t acc = {0.f, 0.f, 0.f, 0.f}, acc2 = {0.f, 0.f, 0.f, 0.f};
 
     for (int kc0 = 0; kc0 < K; kc0 += KC) {
@@ -496,7 +503,7 @@ __device__ __forceinline__ void gemv_fp4_mfma_rows(const uint8_t* __restrict__ w
                 if constexpr (BLK == 32) {
                     s[j] = (j & 1) ? bf16_hi(sd[j >> 1]) : bf16_lo(sd[j >> 1]);
                     s2[j] = 0.f;
-                } else if constexpr (ROUNDW) {
+                } else if constexpr (ROUNDW || STACK) {
                     s[j] = hi_half ? bf16_hi(sd[j]) : bf16_lo(sd[j]);
                     s2[j] = 0.f;
                 } else {
@@ -524,6 +531,24 @@ __device__ __forceinline__ void gemv_fp4_mfma_rows(const uint8_t* __restrict__ w
                                                                   __builtin_bit_cast(bf16x8_t, bw[0]), acc, 0, 0, 0);
                     acc2 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, aw[1]),
                                                                    __builtin_bit_cast(bf16x8_t, bw[1]), acc2, 0, 0, 0);
+                } else if constexpr (STACK) {
+                    f32x4_t part[2];
+#pragma unroll
+                    for (int j = 0; j < 2; ++j)
+#pragma unroll
+                        for (int d = 0; d < 4; ++d) {
+                            bw[j][d] = e2m1_pair_bf16(b[j0 + j], d);
+                            aw[j][d] &= x_keep;
+                        }
+#pragma unroll
+                    for (int j = 0; j < 2; ++j)
+                        part[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, aw[j]),
+                                                                          __builtin_bit_cast(bf16x8_t, bw[j]),
+                                                                          f32x4_t{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+#pragma unroll
+                    for (int j = 0; j < 2; ++j)
+#pragma unroll
+                        for (int rr = 0; rr < 4; ++rr) acc[rr] = fmaf(part[j][rr], s[j0 + j], acc[rr]);
                 } else if constexpr (BLK == 16) {
                     // per block: first-half lanes' codes, then second-half lanes' codes
                     const uint32_t keep_lo = hi_half ? 0u : 0xffffffffu;
@@ -627,6 +652,11 @@ __device__ __forceinline__ void gemv_fp4_mfma_rows(const uint8_t* __restrict__ w
                 iteration(wb, it + 1);
             }
         }
+    }
+    if constexpr (STACK) {
+        // lanes q and q + 2 hold the two scales' sums of the same rows
+#pragma unroll
+        for (int r = 0; r < 4; ++r) acc[r] += __shfl_xor(acc[r], 32);
     }
     // lane (i, q) holds column n, rows 4 q .. 4 q + 3
 #pragma unroll
