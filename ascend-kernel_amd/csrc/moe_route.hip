@@ -23,16 +23,20 @@ constexpr int RT_BLOCK = 1024;     // choices per block of the count / rank kern
 constexpr int RT_MAX_E = 1024;     // experts (one thread each in the scan kernel)
 constexpr int RT_MAX_PER_LANE = RT_MAX_E / 64;
 
+// PL = logits per lane (E <= 64 PL).  The arg-max over the wavefront is lexicographic in (value descending, expert
+// ascending): a max-reduction of the lanes' best values, then the expert of the one lane that holds it (read with
+// v_readlane); only when several lanes hold the maximum a second reduction picks the lowest expert among them.
+template <int PL>
 __global__ __launch_bounds__(256) void route_topk_kernel(const float* __restrict__ logits, float* __restrict__ weight,
                                                          int32_t* __restrict__ ids, int T, int E, int topk) {
     const int lane = threadIdx.x & 63;
     const int t = blockIdx.x * 4 + (threadIdx.x >> 6);
     if (t >= T) return;
     const float* row = logits + (int64_t)t * E;
-    float v[RT_MAX_PER_LANE];
+    float v[PL];
     float mx = -INFINITY;
 #pragma unroll
-    for (int c = 0; c < RT_MAX_PER_LANE; ++c) {
+    for (int c = 0; c < PL; ++c) {
         const int e = c * 64 + lane;
         v[c] = e < E ? row[e] : -INFINITY;
         mx = fmaxf(mx, v[c]);
@@ -41,7 +45,7 @@ __global__ __launch_bounds__(256) void route_topk_kernel(const float* __restrict
     for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off, 64));
     float sum = 0.f;
 #pragma unroll
-    for (int c = 0; c < RT_MAX_PER_LANE; ++c)
+    for (int c = 0; c < PL; ++c)
         if (c * 64 + lane < E) sum += __expf(v[c] - mx);
     sum = wave_reduce_sum(sum);
     const float inv = 1.f / sum;
@@ -50,23 +54,29 @@ __global__ __launch_bounds__(256) void route_topk_kernel(const float* __restrict
         float bv = -INFINITY;
         int be = 0x7fffffff;
 #pragma unroll
-        for (int c = 0; c < RT_MAX_PER_LANE; ++c) {
+        for (int c = 0; c < PL; ++c) {
             const int e = c * 64 + lane;
             if (e < E && (v[c] > bv || (v[c] == bv && e < be))) { bv = v[c]; be = e; }
         }
+        float gv = bv;
 #pragma unroll
-        for (int off = 32; off > 0; off >>= 1) {
-            const float ov = __shfl_xor(bv, off, 64);
-            const int oe = __shfl_xor(be, off, 64);
-            if (ov > bv || (ov == bv && oe < be)) { bv = ov; be = oe; }
+        for (int off = 32; off > 0; off >>= 1) gv = fmaxf(gv, __shfl_xor(gv, off, 64));
+        const unsigned long long holders = __ballot(bv == gv);
+        int ge;
+        if (__popcll(holders) == 1) {
+            ge = __shfl(be, __ffsll(holders) - 1, 64);
+        } else {
+            ge = bv == gv ? be : 0x7fffffff;
+#pragma unroll
+            for (int off = 32; off > 0; off >>= 1) ge = min(ge, __shfl_xor(ge, off, 64));
         }
         if (lane == 0) {
-            ids[(int64_t)t * topk + j] = be;
-            weight[(int64_t)t * topk + j] = __expf(bv - mx) * inv;
+            ids[(int64_t)t * topk + j] = ge;
+            weight[(int64_t)t * topk + j] = __expf(gv - mx) * inv;
         }
 #pragma unroll
-        for (int c = 0; c < RT_MAX_PER_LANE; ++c)
-            if (c * 64 + lane == be) v[c] = -INFINITY;
+        for (int c = 0; c < PL; ++c)
+            if (c * 64 + lane == ge) v[c] = -INFINITY;
     }
 }
 
@@ -222,9 +232,15 @@ int launch_route(const moe_route_args* a, hipStream_t stream) {
     int32_t* ids = static_cast<int32_t*>(a->topk_ids);
     int32_t* counts = static_cast<int32_t*>(a->workspace);
     if (a->logits && a->T > 0) {
-        hipLaunchKernelGGL(route_topk_kernel, dim3((unsigned)((a->T + 3) / 4)), dim3(256), 0, stream,
-                           static_cast<const float*>(a->logits), static_cast<float*>(a->topk_weight), ids, (int)a->T,
-                           (int)a->E, (int)a->topk);
+        const dim3 grid((unsigned)((a->T + 3) / 4));
+        const float* lg = static_cast<const float*>(a->logits);
+        float* tw = static_cast<float*>(a->topk_weight);
+        const int T = (int)a->T, E = (int)a->E, topk = (int)a->topk;
+        if (E <= 64) hipLaunchKernelGGL(route_topk_kernel<1>, grid, dim3(256), 0, stream, lg, tw, ids, T, E, topk);
+        else if (E <= 128) hipLaunchKernelGGL(route_topk_kernel<2>, grid, dim3(256), 0, stream, lg, tw, ids, T, E, topk);
+        else if (E <= 256) hipLaunchKernelGGL(route_topk_kernel<4>, grid, dim3(256), 0, stream, lg, tw, ids, T, E, topk);
+        else if (E <= 512) hipLaunchKernelGGL(route_topk_kernel<8>, grid, dim3(256), 0, stream, lg, tw, ids, T, E, topk);
+        else hipLaunchKernelGGL(route_topk_kernel<RT_MAX_PER_LANE>, grid, dim3(256), 0, stream, lg, tw, ids, T, E, topk);
         if (hipGetLastError() != hipSuccess) return MOE_ERR_LAUNCH;
     }
     if (nblocks > 0)

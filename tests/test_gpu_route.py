@@ -58,6 +58,20 @@ def test_route_from_logits(T, E, K, topk):
     assert np.array_equal(xs, x[ref_rt])
 
 
+@pytest.mark.parametrize("E", [48, 200, 300, 1000])
+def test_route_topk_with_many_equal_logits(E):
+    """Few distinct logit values: every arg-max has several holders, in different lanes and in different
+    64-expert slices of a lane; ties go to the lower expert id."""
+    _say(f"route ties E={E}")
+    T, topk = 130, 6
+    rng = np.random.default_rng(E)
+    logits = rng.integers(0, 4, (T, E)).astype(np.float32)
+    ids, w, gl, rt, roc, _ = _route(logits, None, None, T, E, 0, topk)
+    ref_ids, ref_w = R.route_topk(logits, topk)
+    assert np.array_equal(ids, ref_ids)
+    assert np.allclose(w, ref_w, rtol=1e-5, atol=1e-9)
+
+
 def test_route_ties_and_given_ids_with_dropped_choices():
     _say("route ties / given ids")
     # all-equal logits: the k lowest expert ids, in order
