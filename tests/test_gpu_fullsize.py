@@ -159,3 +159,44 @@ def test_fused_fp4_decode_against_separate_path_and_oracle():
     g = experts[0]
     ref_w = oracle.dequant_fp4_bf16(w[g].cpu().numpy(), H.bits(s[g].cpu()), 32)
     assert np.array_equal(H.bits(wd[g].cpu()), ref_w)
+
+
+@pytest.mark.parametrize("fmt", ["fp4", "int4", "fp8"])
+def test_decode_batch_on_the_n_contiguous_containers(fmt):
+    """256 experts of 7168 x 2048, 512 routed rows, through both ops on the reference's own containers and on
+    int4: the small-tile kinds with two workgroups per CU and tiles taken from the work counter.  The oracle
+    checks whole experts (the largest, the first and the last with rows); every other row must agree between
+    the two ops up to the rounding of the weights, be finite, and rows past group_list[-1] stay untouched."""
+    _say(f"full size: decode batch on {fmt}")
+    gen = torch.Generator().manual_seed(11)
+    torch.manual_seed(11)
+    G, K, N = 256, 7168, 2048
+    counts = _routed(64, G, 8, gen)
+    gl = counts.cumsum(0).to(torch.int64).cuda()
+    M = int(counts.sum())
+    x = _bf16_normal((M + 3, K))
+    if fmt == "fp8":
+        w = torch.randint(0, 255, (G, K, N), dtype=torch.uint8, device="cuda")
+        s = torch.rand((G, K // 128, N // 128), device="cuda") * 1e-2 + 1e-3
+        srows = K // 128
+    else:
+        group = 16 if fmt == "fp4" else 128
+        w = torch.randint(0, 256, (G, K, N // 2), dtype=torch.uint8, device="cuda")
+        w = w.view(torch.int8) if fmt == "fp4" else w
+        s = _bf16_uniform((G, K // group, N), 2.0 ** -8, 2.0 ** -2)
+        srows = K // group
+    active = torch.nonzero(counts > 0).flatten().tolist()
+    experts = sorted({int(torch.argmax(counts)), active[0], active[-1]})
+    ys = {}
+    for op in ("gemm", "gemv"):
+        y = torch.full((M + 3, N), float("nan"), dtype=torch.bfloat16, device="cuda")
+        _launch(op, fmt, x, w, s, None, gl, y, scale_rows=srows)
+        assert torch.isnan(y[M:]).all(), "rows beyond group_list[-1] were written"
+        assert torch.isfinite(y[:M].float()).all()
+        rows, ref = _oracle_subset(fmt, x, w, s, None, counts, experts, gemv=op == "gemv")
+        H.assert_close(H.bits(y[rows.cuda()]), ref, what=f"{fmt} {op} vs oracle")
+        ys[op] = y[:M]
+    # the ops differ by the rounding of the weights to bf16 (2^-9 per weight, summed over K = 7168): small against
+    # the largest outputs, not against every single one
+    rel, _ = H.compare(H.bits(ys["gemm"]), H.bits(ys["gemv"]))
+    assert rel <= H.REL_TOL, f"{fmt}: GEMM op vs GEMV op rel {rel:.3e}"
