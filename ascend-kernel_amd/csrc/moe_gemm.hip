@@ -1153,15 +1153,26 @@ __global__ __launch_bounds__((64 * KernelCfg<FMT, KIND>::WAVES), (KernelCfg<FMT,
             expert_chunks<MTM>(e > s ? (int)(e - s) : 0, chunks, bpc);
             sum += chunks * ntile_n;
         }
-        part[tid] = sum;
-        __syncthreads();
-        if (tid == 0) {
-            int run = 0;
-            for (int t = 0; t < THREADS; ++t) { const int v = part[t]; part[t] = run; run += v; }
-            prefix[P.G] = run;
+        // scan over the threads: within a wavefront by shuffles, across wavefronts through their totals in
+        // LDS (a loop of one thread over all partial sums took 8 us at the start of every workgroup)
+        const int lane = tid & 63, wave = tid >> 6;
+        int incl = sum;
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) {
+            const int up = __shfl_up(incl, off, 64);
+            if (lane >= off) incl += up;
         }
+        if (lane == 63) part[wave] = incl;
         __syncthreads();
-        int run = part[tid];
+        int before = 0, all = 0;
+#pragma unroll
+        for (int w = 0; w < WAVES; ++w) {
+            const int v = part[w];
+            before += w < wave ? v : 0;
+            all += v;
+        }
+        if (tid == 0) prefix[P.G] = all;
+        int run = before + incl - sum;
         for (int g = g0; g < g1; ++g) {
             int64_t s = g ? P.gl[g - 1] : 0, e = P.gl[g];
             s = max((int64_t)0, s); e = min(e, P.M);
