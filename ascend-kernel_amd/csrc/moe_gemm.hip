@@ -51,6 +51,7 @@ struct GemmParams {
     int K, N, G, scale_rows;
     int epilogue;   // moe_epilogue
     int slot;       // this launch's pair of counters in tile_queue
+    int rows_in_lds;   // the scheduler keeps the experts' clamped row bounds in LDS (they fit next to the tile table)
 };
 
 // Work queue of the persistent grid.  Workgroups do not run at one speed (of two that share a CU the one
@@ -1136,21 +1137,40 @@ __global__ __launch_bounds__((64 * KernelCfg<FMT, KIND>::WAVES), (KernelCfg<FMT,
     extern __shared__ u32x4_t smem[];
     constexpr int THREADS = 64 * WAVES;
     constexpr int MTM = C::MTM;
-    int* prefix = reinterpret_cast<int*>(smem + C::lds_units());      // [G + 1]
+    int* prefix = reinterpret_cast<int*>(smem + C::lds_units());      // [G + 1] first tile of every expert
+    // [G + 1] row bounds: rowc[g] = group_list[g - 1] clamped to [0, M] (rowc[0] = 0); expert g owns the rows
+    // [rowc[g], rowc[g + 1]) if that is not empty (same result as clamping start and end separately).  Kept in
+    // LDS so that the scheduler does not wait for a global load per tile (2 to 4 us under a streaming kernel).
+    int* rowc = prefix + (P.G + 1);
     const int tid = threadIdx.x;
     const int ntile_n = (P.N + C::BN - 1) / C::BN;
     __shared__ int part[THREADS];   // scan partials; part[0] later carries the tile taken from the queue
+    auto clamp_row = [&](int64_t v) { return (int)min(max(v, (int64_t)0), P.M); };
+    auto expert_rows = [&](int g, int& first) {
+        int hi;
+        if (P.rows_in_lds) {
+            first = rowc[g];
+            hi = rowc[g + 1];
+        } else {
+            first = g ? clamp_row(P.gl[g - 1]) : 0;
+            hi = clamp_row(P.gl[g]);
+        }
+        return max(hi - first, 0);
+    };
 
     // exclusive scan of tiles per expert: each thread takes a contiguous run of experts
     {
         const int per = (P.G + THREADS - 1) / THREADS;
         const int g0 = tid * per, g1 = min(P.G, g0 + per);
+        if (P.rows_in_lds) {
+            for (int g = g0; g < g1; ++g) rowc[g + 1] = clamp_row(P.gl[g]);
+            if (tid == 0) rowc[0] = 0;
+            __syncthreads();
+        }
         int sum = 0;
         for (int g = g0; g < g1; ++g) {
-            int64_t s = g ? P.gl[g - 1] : 0, e = P.gl[g];
-            s = max((int64_t)0, s); e = min(e, P.M);
-            int chunks, bpc;
-            expert_chunks<MTM>(e > s ? (int)(e - s) : 0, chunks, bpc);
+            int first, chunks, bpc;
+            expert_chunks<MTM>(expert_rows(g, first), chunks, bpc);
             sum += chunks * ntile_n;
         }
         // scan over the threads: within a wavefront by shuffles, across wavefronts through their totals in
@@ -1174,10 +1194,8 @@ __global__ __launch_bounds__((64 * KernelCfg<FMT, KIND>::WAVES), (KernelCfg<FMT,
         if (tid == 0) prefix[P.G] = all;
         int run = before + incl - sum;
         for (int g = g0; g < g1; ++g) {
-            int64_t s = g ? P.gl[g - 1] : 0, e = P.gl[g];
-            s = max((int64_t)0, s); e = min(e, P.M);
-            int chunks, bpc;
-            expert_chunks<MTM>(e > s ? (int)(e - s) : 0, chunks, bpc);
+            int first, chunks, bpc;
+            expert_chunks<MTM>(expert_rows(g, first), chunks, bpc);
             prefix[g] = run;
             run += chunks * ntile_n;
         }
@@ -1213,22 +1231,27 @@ __global__ __launch_bounds__((64 * KernelCfg<FMT, KIND>::WAVES), (KernelCfg<FMT,
         const bool take = C::PAIR && sw + 1 >= fixed_sweeps;
         const Ticket tk = {take ? q_next : nullptr, part};
         have_ticket = take;
-        // largest g with prefix[g] <= T (empty experts have prefix[g] == prefix[g+1])
-        int lo = 0, hi = P.G;
-        while (hi - lo > 1) {
-            const int mid = (lo + hi) >> 1;
-            if (prefix[mid] <= T) lo = mid; else hi = mid;
-        }
+        // largest g with prefix[g] <= T (empty experts have prefix[g] == prefix[g+1]): every wavefront looks at 64
+        // evenly spaced entries at once, then at the entries between two of them -- two LDS round trips
+        // instead of the ten of a binary search
+        const int lane64 = tid & 63;
+        const int stride = (P.G + 63) >> 6;                      // entries per lane of the first step
+        const int probe = min(lane64 * stride, P.G);
+        const unsigned long long le1 = __ballot(prefix[probe] <= T && lane64 * stride <= P.G);
+        const int seg = 63 - __builtin_clzll(le1 | 1ull);        // last lane whose entry is <= T (lane 0: prefix[0] = 0)
+        const int idx2 = seg * stride + lane64;
+        const unsigned long long le2 = __ballot(lane64 < stride && idx2 < P.G && prefix[idx2] <= T);
         // everything below is wave-uniform; readfirstlane lets the compiler keep it in SGPRs
-        const int g = __builtin_amdgcn_readfirstlane(lo);
-        const int64_t gbeg = g ? max((int64_t)0, P.gl[g - 1]) : 0, gend = min(P.gl[g], P.M);
-        const int m = __builtin_amdgcn_readfirstlane((int)(gend - gbeg));
+        const int g = __builtin_amdgcn_readfirstlane(seg * stride + 63 - __builtin_clzll(le2 | 1ull));
+        int gfirst;
+        const int m = __builtin_amdgcn_readfirstlane(expert_rows(g, gfirst));
+        const int64_t gbeg = gfirst;
         int chunks, bpc;
         expert_chunks<MTM>(m, chunks, bpc);
         const int local = __builtin_amdgcn_readfirstlane(T - prefix[g]);
         // row chunks innermost: the tiles that share a weight column tile are neighbours in the order, run at
         // the same time on one XCD and pull that slice of the expert's weights into its L2 once
-        const int nt = local / chunks, chunk = local % chunks;
+        const int nt = chunks == 1 ? local : local / chunks, chunk = chunks == 1 ? 0 : local % chunks;
         const int rbeg = chunk * bpc * 16;
         const int rows = min(m - rbeg, bpc * 16);
         const int mt = (rows + 15) >> 4;
@@ -1286,8 +1309,11 @@ __global__ __launch_bounds__((64 * KernelCfg<FMT, KIND>::WAVES), (KernelCfg<FMT,
 template <int FMT, int KIND>
 static int launch_gemm_kind(const GemmParams& P, const moe_grouped_args* a, hipStream_t stream) {
     using C = KernelCfg<FMT, KIND>;
-    const size_t lds = (size_t)C::lds_units() * 16 + ((size_t)a->G + 1) * sizeof(int);
     const size_t lds_max = (160 * 1024 - 2048) / C::WG_PER_CU;
+    const size_t table = ((size_t)a->G + 1) * sizeof(int);
+    // tile table, and the row bounds next to it where they fit (else the scheduler reads group_list per tile)
+    const bool rows_in_lds = (size_t)C::lds_units() * 16 + 2 * table <= lds_max;
+    const size_t lds = (size_t)C::lds_units() * 16 + (rows_in_lds ? 2 : 1) * table;
     if (lds > lds_max) return MOE_ERR_TOO_LARGE;
     static std::atomic<uint64_t> lds_set{0};
     if (const int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(&grouped_gemm_kernel<FMT, KIND>), (int)lds_max, lds_set))
@@ -1304,6 +1330,7 @@ static int launch_gemm_kind(const GemmParams& P, const moe_grouped_args* a, hipS
     const int64_t grid = want > 0 ? (want + 7) / 8 * 8 : 8;
     GemmParams Q = P;
     Q.slot = (int)(queue_launches.fetch_add(1, std::memory_order_relaxed) % GM_QUEUE_SLOTS);
+    Q.rows_in_lds = rows_in_lds ? 1 : 0;
     hipLaunchKernelGGL((grouped_gemm_kernel<FMT, KIND>), dim3((unsigned)grid), dim3(64 * C::WAVES), lds, stream, Q);
     return hipGetLastError() == hipSuccess ? MOE_OK : MOE_ERR_LAUNCH;
 }
@@ -1319,6 +1346,7 @@ static GemmParams gemm_params(const moe_grouped_args* a) {
     P.M = a->M; P.K = (int)a->K; P.N = (int)a->N; P.G = (int)a->G; P.scale_rows = (int)a->scale_rows;
     P.epilogue = a->epilogue;
     P.slot = 0;
+    P.rows_in_lds = 0;
     return P;
 }
 
