@@ -52,6 +52,8 @@ struct GemmParams {
     int epilogue;   // moe_epilogue
     int slot;       // this launch's pair of counters in tile_queue
     int rows_in_lds;   // the scheduler keeps the experts' clamped row bounds in LDS (they fit next to the tile table)
+    uint32_t sub_per_group;   // 32-k sub-steps per scale group of the N-contiguous 4-bit containers ...
+    uint32_t sub_to_group;    // ... and the multiplier that turns a sub-step index into its scale row (0: identity)
 };
 
 // Work queue of the persistent grid.  Workgroups do not run at one speed (of two that share a CU the one
@@ -627,8 +629,9 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
     const rsrc_t rs8 = make_rsrc(static_cast<const float*>(P.scale) + (int64_t)g * (P.K >> 7) * (P.N >> 7),
                                  (int64_t)(P.K >> 7) * (P.N >> 7) * 4);
     const int cs8 = ((n0 + 64 * cw) >> 7) * 4;
-    const uint32_t per = (B8 || KC) ? 1u : (uint32_t)((P.K / P.scale_rows) >> 5);      // 32-k sub-steps per scale group
-    const uint32_t gmul = per == 1 ? 0u : 0xffffffffu / per + 1u;   // sub-step -> scale row as a multiply
+    // 32-k sub-steps per scale group, and sub-step -> scale row as a multiply (both worked out on the host)
+    const uint32_t per = (B8 || KC) ? 1u : P.sub_per_group;
+    const uint32_t gmul = (B8 || KC) ? 0u : P.sub_to_group;
     auto scale_row = [&](uint32_t sub) { return gmul ? (int)__umulhi(sub, gmul) : (int)sub; };
     // x rows through a buffer resource that ends after the last valid row (padded rows read as
     // zeros).  Load instruction j covers rows 8j + (lane >> 3); position lane & 7 of a row
@@ -720,17 +723,8 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
     // The accumulators are zeroed by asm so that the compiler cannot re-materialize the zeros
     // right in front of the first MFMA that accumulates into them: a VALU write of an MFMA's
     // accumulator input needs wait states the compiler only inserts for MFMAs it can see.
+    // (Done behind the prologue's loads, below: up to 160 moves that would otherwise delay the first request.)
     f32x4_t acc[MT][4];
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-        for (int t = 0; t < 4; ++t) {
-            if constexpr (EXACT)
-                acc[mt][t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-            else
-                asm volatile("v_mov_b32 %0, 0\n\tv_mov_b32 %1, 0\n\tv_mov_b32 %2, 0\n\tv_mov_b32 %3, 0"
-                             : "=v"(acc[mt][t][0]), "=v"(acc[mt][t][1]), "=v"(acc[mt][t][2]), "=v"(acc[mt][t][3]));
-        }
     u32x4_t bf[4], afr[4];
     constexpr int RING = 3;
     constexpr int R = RING < MT ? RING : MT;   // x fragments read ahead of their MFMAs
@@ -755,6 +749,16 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
     }
 #pragma unroll
     for (int st0 = 0; st0 < AHEAD; ++st0) issue_group(st0 - AHEAD, st0);
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            if constexpr (EXACT)
+                acc[mt][t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+            else
+                asm volatile("v_mov_b32 %0, 0\n\tv_mov_b32 %1, 0\n\tv_mov_b32 %2, 0\n\tv_mov_b32 %3, 0"
+                             : "=v"(acc[mt][t][0]), "=v"(acc[mt][t][1]), "=v"(acc[mt][t][2]), "=v"(acc[mt][t][3]));
+        }
     ring_barrier();
     if constexpr (I8) {
         ch_s[0] = bf16_lo(ch_sb[0]); ch_s[1] = bf16_hi(ch_sb[0]); ch_s[2] = bf16_lo(ch_sb[1]); ch_s[3] = bf16_hi(ch_sb[1]);
@@ -1084,8 +1088,13 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
 template <int MT_MAX>
 __device__ __forceinline__ void expert_chunks(int m, int& chunks, int& bpc) {
     const int nblk = (m + 15) >> 4;
+    if (nblk <= MT_MAX) {   // the usual case, without the division
+        chunks = nblk ? 1 : 0;
+        bpc = nblk;
+        return;
+    }
     chunks = (nblk + MT_MAX - 1) / MT_MAX;
-    bpc = chunks ? (nblk + chunks - 1) / chunks : 0;
+    bpc = (nblk + chunks - 1) / chunks;
 }
 
 template <int FMT, int KIND>
@@ -1347,6 +1356,9 @@ static GemmParams gemm_params(const moe_grouped_args* a) {
     P.epilogue = a->epilogue;
     P.slot = 0;
     P.rows_in_lds = 0;
+    const uint32_t per = a->scale_rows > 0 ? (uint32_t)((a->K / a->scale_rows) >> 5) : 1u;
+    P.sub_per_group = per ? per : 1u;
+    P.sub_to_group = P.sub_per_group == 1 ? 0u : 0xffffffffu / P.sub_per_group + 1u;
     return P;
 }
 
