@@ -760,9 +760,24 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
                              : "=v"(acc[mt][t][0]), "=v"(acc[mt][t][1]), "=v"(acc[mt][t][2]), "=v"(acc[mt][t][3]));
         }
     ring_barrier();
+    // int8: (q + offset) * scale is defined as two rounded fp32 operations.  Where q + offset cannot round (an
+    // offset of 0, or of a magnitude in [2^-8, 2^22]: the sum of an 8-bit integer and an 8-bit significand then fits
+    // 24 bits) and offset * scale is exact and normal (scale positive and far from the ends of the range), one fma
+    // q * scale + offset * scale rounds the same real number once and gives the same bits: 2.5 instead of 3.5
+    // instructions per weight.  Decided per wavefront and tile from its lanes' channels.
+    float ch_os[4] = {0.f, 0.f, 0.f, 0.f};
+    bool i8_one_rounding = false;
     if constexpr (I8) {
         ch_s[0] = bf16_lo(ch_sb[0]); ch_s[1] = bf16_hi(ch_sb[0]); ch_s[2] = bf16_lo(ch_sb[1]); ch_s[3] = bf16_hi(ch_sb[1]);
         ch_o[0] = bf16_lo(ch_ob[0]); ch_o[1] = bf16_hi(ch_ob[0]); ch_o[2] = bf16_lo(ch_ob[1]); ch_o[3] = bf16_hi(ch_ob[1]);
+        bool ok = true;
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            const float ao = fabsf(ch_o[t]);
+            ok = ok && ch_s[t] >= 0x1p-60f && ch_s[t] <= 0x1p60f && (ao == 0.f || (ao >= 0x1p-8f && ao <= 0x1p22f));
+            ch_os[t] = ch_o[t] * ch_s[t];
+        }
+        i8_one_rounding = __all(ok);
     }
 
     // this lane's packed dwords and scales of its sub-step of LDS stage st
@@ -899,15 +914,27 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
             }
             if constexpr (I8) {
                 // byte t of the dwords of k rows 2p, 2p+1 -> (q + offset) * scale as two rounded fp32
-                // operations -> bf16 pair along k
+                // operations (or the one fma that equals them, see i8_one_rounding) -> bf16 pair along k
+                if (i8_one_rounding) {
 #pragma unroll
-                for (int p = 0; p < 2; ++p) {
-                    const uint32_t a = r[2 * (p0 + p)], b = r[2 * (p0 + p) + 1];
+                    for (int p = 0; p < 2; ++p) {
+                        const uint32_t a = r[2 * (p0 + p)], b = r[2 * (p0 + p) + 1];
 #pragma unroll
-                    for (int t = 0; t < 4; ++t) {
-                        const float qa = (float)(int)(int8_t)(a >> (8 * t)), qb = (float)(int)(int8_t)(b >> (8 * t));
-                        bf[t][p0 + p] = pack_bf16_rne(__fmul_rn(__fadd_rn(qa, ch_o[t]), ch_s[t]),
-                                                      __fmul_rn(__fadd_rn(qb, ch_o[t]), ch_s[t]));
+                        for (int t = 0; t < 4; ++t) {
+                            const float qa = (float)(int)(int8_t)(a >> (8 * t)), qb = (float)(int)(int8_t)(b >> (8 * t));
+                            bf[t][p0 + p] = pack_bf16_rne(__fmaf_rn(qa, ch_s[t], ch_os[t]), __fmaf_rn(qb, ch_s[t], ch_os[t]));
+                        }
+                    }
+                } else {
+#pragma unroll
+                    for (int p = 0; p < 2; ++p) {
+                        const uint32_t a = r[2 * (p0 + p)], b = r[2 * (p0 + p) + 1];
+#pragma unroll
+                        for (int t = 0; t < 4; ++t) {
+                            const float qa = (float)(int)(int8_t)(a >> (8 * t)), qb = (float)(int)(int8_t)(b >> (8 * t));
+                            bf[t][p0 + p] = pack_bf16_rne(__fmul_rn(__fadd_rn(qa, ch_o[t]), ch_s[t]),
+                                                          __fmul_rn(__fadd_rn(qb, ch_o[t]), ch_s[t]));
+                        }
                     }
                 }
                 __builtin_amdgcn_sched_barrier(0);

@@ -391,3 +391,31 @@ def test_oracle_under_address_and_ub_sanitizers():
         pytest.skip("another preloaded library keeps AddressSanitizer from starting in this environment")
     assert r.returncode == 0, out[-2000:]
     assert "sanitize_check ok" in out
+
+
+def test_int8_one_fma_equals_the_two_rounded_operations_where_the_kernel_uses_it():
+    """The int8 decode of the GPU kernel replaces (q + offset) * scale, two rounded fp32 operations, by one fma
+    q * scale + offset * scale where the sum cannot round: offset 0 or |offset| in [2^-8, 2^22], scale in
+    [2^-60, 2^60].  Checked here on every q against random bf16 offsets and scales of that domain, bit for bit;
+    the fma is evaluated exactly in float64 (16-bit products at most 2^30 apart) and rounded once."""
+    rng = np.random.default_rng(77)
+    n = 20000
+    def bf16_of(mag_lo, mag_hi, signed):
+        e = rng.integers(mag_lo, mag_hi, n)                     # exponent
+        m = rng.integers(128, 256, n).astype(np.float64) / 128  # 8-bit significand in [1, 2)
+        v = np.ldexp(m, e)
+        if signed:
+            v *= rng.choice([-1.0, 1.0], n)
+        return v.astype(np.float32)
+    off = bf16_of(-8, 22, True)
+    off[: n // 10] = 0.0
+    off[n // 10: n // 10 + 50] = np.float32(2.0 ** -8)
+    off[n // 10 + 50: n // 10 + 100] = np.float32(255.0 / 128 * 2.0 ** 21)   # largest allowed bf16 below 2^22
+    scale = bf16_of(-60, 60, False)
+    assert (oracle.bf16_bits_to_f32(oracle.f32_to_bf16_bits(off)) == off).all()
+    assert (oracle.bf16_bits_to_f32(oracle.f32_to_bf16_bits(scale)) == scale).all()
+    for q in range(-128, 128):
+        qf = np.float32(q)
+        two = (qf + off) * scale                                             # float32 add, float32 multiply
+        one = (np.float64(q) * scale.astype(np.float64) + off.astype(np.float64) * scale.astype(np.float64)).astype(np.float32)
+        assert np.array_equal(two.view(np.uint32), one.view(np.uint32)), q
