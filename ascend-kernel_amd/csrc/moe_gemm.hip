@@ -416,7 +416,8 @@ __device__ __forceinline__ void lds_load16(rsrc_t r, const u32x4_t* dst, int vof
 //
 // int8 and the reference fp8 container: a step's tile is 64 rows of 256 bytes (two load instructions
 // per wavefront), which leaves room for S = 4 stages; a lane's 4 columns are one dword of each of its 8 k
-// rows.  int8 keeps its per-channel scale and offset in registers; fp8 decodes two codes at a time through
+// rows.  int8 keeps its per-channel scale and offset in registers (and folds them into one fma where that gives
+// the bits of the two rounded operations, see i8_one_rounding); fp8 decodes two codes at a time through
 // fp16 (see e4m3_ref_pair_over_256_fp16) and gets the fp32 scale of its 128 x 128 block through the ring,
 // 4 bytes per wavefront and step.
 //
