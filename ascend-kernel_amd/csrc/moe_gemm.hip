@@ -50,7 +50,8 @@ struct GemmParams {
     int64_t M;
     int K, N, G, scale_rows;
     int epilogue;   // moe_epilogue
-    int slot;       // this launch's pair of counters in tile_queue
+    int slot;       // this launch's counters in tile_queue; -1: none, every tile in the fixed order
+    unsigned epoch; // stamp of this launch's counters
     int rows_in_lds;   // the scheduler keeps the experts' clamped row bounds in LDS (they fit next to the tile table)
     uint32_t sub_per_group;   // 32-k sub-steps per scale group of the N-contiguous 4-bit containers ...
     uint32_t sub_to_group;    // ... and the multiplier that turns a sub-step index into its scale row (0: identity)
@@ -60,19 +61,71 @@ struct GemmParams {
 // placed first runs about 1.5 times as fast as the other while both are resident, and the XCDs differ by a few
 // per cent), so an even split of the tiles leaves most of the chip waiting for the slowest workgroup.  All but
 // the last two or three tiles of a workgroup's share are handed out in a fixed, XCD-aware order; the rest
-// are taken one at a time from a counter.  Every launch gets a slot (next tile, workgroups done) of its
-// own, so that launches on different streams do not share a counter; the last workgroup to finish puts both
-// back to zero, the state device memory starts in.  Two launches collide only if GM_QUEUE_SLOTS launches
-// later the first is still running.
+// (the tail) are taken one at a time from counters in the library's device memory.
+//
+// The tail is cut into 8 contiguous runs, one per XCD, each with a counter of its own: the workgroups of an
+// XCD keep drawing neighbouring tiles (the same experts' x rows and weight slices in that XCD's L2) and only
+// when their run is used up take tiles from the XCD that has most left.
+//
+// A launch owns one slot of 8 counters.  The host numbers the launches; launch L uses slot L % GM_QUEUE_SLOTS
+// and stamps every counter it touches with its epoch (L / GM_QUEUE_SLOTS, never 0) in the upper bits: a counter
+// that carries another epoch is left over from an earlier launch and counts as zero, so nothing has to be
+// cleared at the end of a kernel and no state a kernel leaves behind can mislead a later one.  Two launches
+// share a slot only if GM_QUEUE_SLOTS launches after the first one it is still running.  A launch that is
+// being captured into a HIP graph gets no slot at all (slot -1): its kernel node would keep the slot for every
+// replay while the ring moves on, so it walks all of its tiles in the fixed order instead.
 constexpr int GM_QUEUE_SLOTS = 1024;
-constexpr int GM_QUEUE_TAIL_SWEEPS = 2;   // tiles per workgroup that are left to the counter (plus the remainder)
-__device__ unsigned int tile_queue[GM_QUEUE_SLOTS * 2];
-static std::atomic<unsigned> queue_launches{0};   // launches of every kind of kernel in this file, for the slot
-// A tile routine that is handed a counter takes the workgroup's next tile from it while it finishes its own
-// (the counter's round trip, about 3 us under load, overlaps the tile's reduction and stores) and leaves the
-// result in *out behind its last barrier.
+constexpr int GM_QUEUE_TAIL_SWEEPS = 2;   // tiles per workgroup that are left to the counters (plus the remainder)
+constexpr unsigned GM_QUEUE_COUNT_BITS = 20, GM_QUEUE_COUNT_MASK = (1u << GM_QUEUE_COUNT_BITS) - 1u;
+constexpr unsigned GM_QUEUE_EPOCHS = (1u << (32 - GM_QUEUE_COUNT_BITS)) - 1u;   // epochs 1 .. GM_QUEUE_EPOCHS
+__device__ unsigned int tile_queue[GM_QUEUE_SLOTS * 8];
+static std::atomic<unsigned> queue_launches{0};   // launches of every kind of kernel in this file, for slot and epoch
+
+// The ticket a fetch-and-add on counter q returned (raw), for a launch of the given epoch: the count
+// before the add if the counter was this launch's already, else the counter is stamped first (compare-and-
+// swap, so that exactly one workgroup gets ticket 0 of a stale counter).  Every path ends after at most as
+// many rounds as there are workgroups.
+__device__ __forceinline__ unsigned queue_ticket(unsigned int* q, unsigned raw, unsigned epoch) {
+    if ((raw >> GM_QUEUE_COUNT_BITS) == epoch) return raw & GM_QUEUE_COUNT_MASK;
+    for (;;) {
+        const unsigned v = __hip_atomic_load(q, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if ((v >> GM_QUEUE_COUNT_BITS) == epoch) return atomicAdd(q, 1u) & GM_QUEUE_COUNT_MASK;
+        if (atomicCAS(q, v, (epoch << GM_QUEUE_COUNT_BITS) | 1u) == v) return 0u;
+    }
+}
+// The tail [lo, lo + n) of a launch as the 8 runs of its XCDs
+struct TailRuns {
+    int lo, n;
+    __device__ __forceinline__ int first(int x) const { return lo + (int)(((int64_t)n * x) >> 3); }
+    __device__ __forceinline__ int size(int x) const { return first(x + 1) - first(x); }
+};
+// One thread resolves the workgroup's next tail tile from the raw value its fetch-and-add on the own XCD's
+// counter returned; -1 when the tail is used up.
+__device__ __forceinline__ int queue_resolve(unsigned int* slot, int xcd, unsigned raw, unsigned epoch, const TailRuns& tr) {
+    unsigned t = queue_ticket(slot + xcd, raw, epoch);
+    if ((int)t < tr.size(xcd)) return tr.first(xcd) + (int)t;
+    for (;;) {
+        // the XCD with most tiles left (the 8 loads are independent: one round trip)
+        unsigned v[8];
+#pragma unroll
+        for (int x = 0; x < 8; ++x) v[x] = __hip_atomic_load(slot + x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        int best = -1, left = 0;
+#pragma unroll
+        for (int x = 0; x < 8; ++x) {
+            const int used = (v[x] >> GM_QUEUE_COUNT_BITS) == epoch ? (int)(v[x] & GM_QUEUE_COUNT_MASK) : 0;
+            const int l = tr.size(x) - used;
+            if (l > left) { left = l; best = x; }
+        }
+        if (best < 0) return -1;
+        t = queue_ticket(slot + best, atomicAdd(slot + best, 1u), epoch);
+        if ((int)t < tr.size(best)) return tr.first(best) + (int)t;
+    }
+}
+// A tile routine that is handed a counter draws the workgroup's next ticket from it while it finishes its own
+// tile (the counter's round trip, about 3 us under load, overlaps the tile's reduction and stores) and leaves
+// the raw value in *out behind its last barrier.
 struct Ticket {
-    unsigned int* counter;   // null: the caller takes the next tile itself
+    unsigned int* counter;   // null: the caller draws the ticket itself
     int* out;
 };
 
@@ -1246,27 +1299,42 @@ __global__ __launch_bounds__((64 * KernelCfg<FMT, KIND>::WAVES), (KernelCfg<FMT,
     const int per_xcd = (nwg + 7) / 8;
     const int vid = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
     const int sweep = per_xcd * 8;   // == nwg: the grid is a multiple of 8
-    const int fixed_sweeps = max(0, total / sweep - GM_QUEUE_TAIL_SWEEPS);
-    unsigned int* q_next = tile_queue + 2 * P.slot;
-    unsigned int* q_done = q_next + 1;
+    // a launch without counters (captured into a HIP graph) walks every tile in the fixed order
+    const bool queued = P.slot >= 0;
+    const int fixed_sweeps = queued ? max(0, total / sweep - GM_QUEUE_TAIL_SWEEPS) : (total + sweep - 1) / sweep;
+    const int xcd = blockIdx.x % 8;
+    unsigned int* q_slot = tile_queue + 8 * max(P.slot, 0);
+    const TailRuns tail = {fixed_sweeps * sweep, max(total - fixed_sweeps * sweep, 0)};
 
-    bool have_ticket = false;   // the previous tile routine left the next tile in part[0]
+    bool have_ticket = false;   // the previous tile routine left the raw ticket in part[0]
     for (int sw = 0;; ++sw) {
         int T;
         if (sw < fixed_sweeps) {
             T = sw * sweep + vid;
+            if (T >= total) break;
         } else {
+            if (!queued) break;
             if (!have_ticket) {
-                __syncthreads();   // part[0] of the previous round is read (the scan's part[], the first time)
-                if (tid == 0) part[0] = (int)atomicAdd(q_next, 1u);
+                __syncthreads();   // part[] of the previous round is read (the scan's part[], the first time)
+                if (tid == 0) part[0] = (int)atomicAdd(q_slot + xcd, 1u);
                 __syncthreads();
             }
-            T = fixed_sweeps * sweep + __builtin_amdgcn_readfirstlane(part[0]);
-            if (T >= total) break;
+            // the usual case needs no second exchange: a ticket of this launch inside the XCD's own run
+            const unsigned raw = (unsigned)__builtin_amdgcn_readfirstlane(part[0]);
+            const int own = (int)(raw & GM_QUEUE_COUNT_MASK);
+            if ((raw >> GM_QUEUE_COUNT_BITS) == P.epoch && own < tail.size(xcd)) {
+                T = tail.first(xcd) + own;
+            } else {
+                __syncthreads();
+                if (tid == 0) part[1] = queue_resolve(q_slot, xcd, raw, P.epoch, tail);
+                __syncthreads();
+                T = __builtin_amdgcn_readfirstlane(part[1]);
+                if (T < 0) break;
+            }
         }
-        // from the last tile of the fixed order on, the k-split tile routines fetch the next tile themselves
-        const bool take = C::PAIR && sw + 1 >= fixed_sweeps;
-        const Ticket tk = {take ? q_next : nullptr, part};
+        // from the last tile of the fixed order on, the k-split tile routines draw the next ticket themselves
+        const bool take = C::PAIR && queued && sw + 1 >= fixed_sweeps;
+        const Ticket tk = {take ? q_slot + xcd : nullptr, part};
         have_ticket = take;
         // largest g with prefix[g] <= T (empty experts have prefix[g] == prefix[g+1]): every wavefront looks at 64
         // evenly spaced entries at once, then at the entries between two of them -- two LDS round trips
@@ -1336,11 +1404,19 @@ __global__ __launch_bounds__((64 * KernelCfg<FMT, KIND>::WAVES), (KernelCfg<FMT,
             default: have_ticket = false; break;
         }
     }
-    // every workgroup has taken its last (failed) ticket; the last one to arrive here re-arms the slot
-    if (tid == 0 && atomicAdd(q_done, 1u) == (unsigned)nwg - 1u) {
-        atomicExch(q_next, 0u);
-        atomicExch(q_done, 0u);
+}
+
+// Compute units of the current device, looked up once per device.
+static int device_cu_count() {
+    static std::atomic<int> cached[64];
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return -1;
+    int cus = cached[dev].load(std::memory_order_relaxed);
+    if (cus == 0) {
+        if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) return -1;
+        cached[dev].store(cus, std::memory_order_relaxed);
     }
+    return cus;
 }
 
 template <int FMT, int KIND>
@@ -1355,9 +1431,8 @@ static int launch_gemm_kind(const GemmParams& P, const moe_grouped_args* a, hipS
     static std::atomic<uint64_t> lds_set{0};
     if (const int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(&grouped_gemm_kernel<FMT, KIND>), (int)lds_max, lds_set))
         return rc;
-    int dev = 0, cus = 256;
-    if (hipGetDevice(&dev) != hipSuccess) return MOE_ERR_NO_DEVICE;
-    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return MOE_ERR_NO_DEVICE;
+    const int cus = device_cu_count();
+    if (cus <= 0) return MOE_ERR_NO_DEVICE;
     // persistent grid: as many workgroups as the CUs hold, but no more than an upper bound on the
     // tile count that needs no look at group_list (every expert adds at most one partly filled chunk)
     const int64_t max_chunks = a->M / (16 * C::MTM) + a->G;
@@ -1366,7 +1441,21 @@ static int launch_gemm_kind(const GemmParams& P, const moe_grouped_args* a, hipS
     // a multiple of 8 so that the XCD-aware order covers every tile index
     const int64_t grid = want > 0 ? (want + 7) / 8 * 8 : 8;
     GemmParams Q = P;
-    Q.slot = (int)(queue_launches.fetch_add(1, std::memory_order_relaxed) % GM_QUEUE_SLOTS);
+    // A launch that is being captured into a graph gets no counters (see tile_queue); so does one whose
+    // stream cannot be queried.  (The null stream cannot be captured and is not asked.)
+    hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+    if (stream != nullptr && hipStreamIsCapturing(stream, &capture) != hipSuccess) {
+        (void)hipGetLastError();
+        capture = hipStreamCaptureStatusActive;
+    }
+    if (capture == hipStreamCaptureStatusNone) {
+        const unsigned launch = queue_launches.fetch_add(1, std::memory_order_relaxed);
+        Q.slot = (int)(launch % GM_QUEUE_SLOTS);
+        Q.epoch = (launch / GM_QUEUE_SLOTS) % GM_QUEUE_EPOCHS + 1u;
+    } else {
+        Q.slot = -1;
+        Q.epoch = 0;
+    }
     Q.rows_in_lds = rows_in_lds ? 1 : 0;
     hipLaunchKernelGGL((grouped_gemm_kernel<FMT, KIND>), dim3((unsigned)grid), dim3(64 * C::WAVES), lds, stream, Q);
     return hipGetLastError() == hipSuccess ? MOE_OK : MOE_ERR_LAUNCH;
@@ -1382,7 +1471,8 @@ static GemmParams gemm_params(const moe_grouped_args* a) {
     P.y = static_cast<uint16_t*>(a->y);
     P.M = a->M; P.K = (int)a->K; P.N = (int)a->N; P.G = (int)a->G; P.scale_rows = (int)a->scale_rows;
     P.epilogue = a->epilogue;
-    P.slot = 0;
+    P.slot = -1;
+    P.epoch = 0;
     P.rows_in_lds = 0;
     const uint32_t per = a->scale_rows > 0 ? (uint32_t)((a->K / a->scale_rows) >> 5) : 1u;
     P.sub_per_group = per ? per : 1u;

@@ -9,6 +9,7 @@
 //
 //   route_topk_kernel     one wavefront per token: softmax statistics and top-k by repeated arg-max
 //   route_count_kernel    per 1024-choice block, a histogram over experts (LDS atomics)
+//   route_scan_kernel     (many blocks only) the counts' prefix over the blocks, per expert
 //   route_rank_kernel     per block: prefix of the counts over experts and earlier blocks (group_list), then every
 //                         choice's rank among the earlier choices of its expert -> its sorted row
 //   route_scatter_kernel  a token's x row read once and written to the sorted row of each of its choices
@@ -49,6 +50,9 @@ __global__ __launch_bounds__(256) void route_topk_kernel(const float* __restrict
         if (c * 64 + lane < E) sum += __expf(v[c] - mx);
     sum = wave_reduce_sum(sum);
     const float inv = 1.f / sum;
+    // experts already chosen, one bit per logit of this lane (a chosen expert cannot be marked with -inf: a
+    // masked logit is -inf too, and a row with fewer than topk finite logits would pick it twice)
+    unsigned taken = 0;
     for (int j = 0; j < topk; ++j) {
         // arg-max over what is left; ties go to the lower expert id
         float bv = -INFINITY;
@@ -56,7 +60,7 @@ __global__ __launch_bounds__(256) void route_topk_kernel(const float* __restrict
 #pragma unroll
         for (int c = 0; c < PL; ++c) {
             const int e = c * 64 + lane;
-            if (e < E && (v[c] > bv || (v[c] == bv && e < be))) { bv = v[c]; be = e; }
+            if (e < E && !((taken >> c) & 1u) && (v[c] > bv || (v[c] == bv && e < be))) { bv = v[c]; be = e; }
         }
         float gv = bv;
 #pragma unroll
@@ -76,7 +80,7 @@ __global__ __launch_bounds__(256) void route_topk_kernel(const float* __restrict
         }
 #pragma unroll
         for (int c = 0; c < PL; ++c)
-            if (c * 64 + lane == ge) v[c] = -INFINITY;
+            if (c * 64 + lane == ge) taken |= 1u << c;
     }
 }
 
@@ -94,16 +98,42 @@ __global__ __launch_bounds__(RT_BLOCK) void route_count_kernel(const int32_t* __
     for (int e = threadIdx.x; e < E; e += RT_BLOCK) block_counts[(int64_t)blockIdx.x * E + e] = hist[e];
 }
 
+// Many blocks: the per-block counts [nblocks][E] become, in place, each expert's exclusive prefix over the
+// blocks, and row nblocks receives the experts' totals.  One wavefront per expert, 64 blocks per round
+// (wavefront scan by shuffles, the running total carried from round to round).
+constexpr int RT_FUSED_SCAN_MAX_BLOCKS = 64;   // up to here every rank block sums the counts itself
+__global__ __launch_bounds__(256) void route_scan_kernel(int32_t* __restrict__ block_counts, int E, int nblocks) {
+    const int lane = threadIdx.x & 63;
+    const int e = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (e >= E) return;
+    int carry = 0;
+    for (int b0 = 0; b0 < nblocks; b0 += 64) {
+        const int b = b0 + lane;
+        const int c = b < nblocks ? block_counts[(int64_t)b * E + e] : 0;
+        int incl = c;
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) {
+            const int up = __shfl_up(incl, off, 64);
+            if (lane >= off) incl += up;
+        }
+        if (b < nblocks) block_counts[(int64_t)b * E + e] = carry + incl - c;
+        carry += __shfl(incl, 63, 64);
+    }
+    if (lane == 0) block_counts[(int64_t)nblocks * E + e] = carry;
+}
+
 // Rank of every choice of block b among the choices of its expert, and with it the sorted row:
 //   row = (choices of lower experts) + (choices of this expert in earlier blocks) + (in earlier wavefronts of
 //         this block) + (in lower lanes of this wavefront)
-// Every block derives the first two terms from the per-block counts itself (nblocks x E integers: cheaper than
-// a kernel of its own for the scan); block 0 also writes group_list.  The third comes from per-wavefront
-// histograms in LDS, the fourth from comparing with the lanes below.  Dynamic LDS: (16 + 2) * E integers.
+// With few blocks every block derives the first two terms from the per-block counts itself (nblocks x E integers
+// per block: cheaper than a kernel of its own for the scan, but quadratic in the number of blocks); with more than
+// RT_FUSED_SCAN_MAX_BLOCKS of them route_scan_kernel has turned the counts into prefixes and totals (prefixed != 0).
+// Block 0 also writes group_list.  The third term comes from per-wavefront histograms in LDS, the fourth from
+// comparing with the lanes below.  Dynamic LDS: (16 + 2) * E integers.
 __global__ __launch_bounds__(RT_BLOCK) void route_rank_kernel(const int32_t* __restrict__ ids, const int32_t* __restrict__ block_counts,
                                                               int64_t* __restrict__ group_list,
                                                               int32_t* __restrict__ row_token, int32_t* __restrict__ row_of_choice,
-                                                              int64_t n, int E, int topk, int nblocks) {
+                                                              int64_t n, int E, int topk, int nblocks, int prefixed) {
     extern __shared__ int rank_lds[];
     int* scan = rank_lds;            // [E] inclusive scan of the experts' totals
     int* base = scan + E;            // [E] first sorted row of this block's choices of expert e
@@ -111,7 +141,11 @@ __global__ __launch_bounds__(RT_BLOCK) void route_rank_kernel(const int32_t* __r
     const int e = threadIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int blk = blockIdx.x;
     int total = 0, before = 0;
-    if (e < E) {
+    if (e < E && prefixed) {
+        before = block_counts[(int64_t)blk * E + e];
+        total = block_counts[(int64_t)nblocks * E + e];
+        scan[e] = total;
+    } else if (e < E) {
         // independent loads, 4 blocks at a time
         int b = 0;
         for (; b + 4 <= nblocks; b += 4) {
@@ -198,10 +232,10 @@ __global__ __launch_bounds__(256) void route_scatter_kernel(const u32x4_t* __res
 size_t route_workspace_bytes(const moe_route_args* a) {
     const int64_t n = a->T * a->topk;
     const int64_t nblocks = (n + RT_BLOCK - 1) / RT_BLOCK;
-    return (size_t)(nblocks * a->E) * sizeof(int32_t);   // per-block counts
+    return (size_t)((nblocks + 1) * a->E) * sizeof(int32_t);   // per-block counts, and a row of totals
 }
 
-// Scratch of moe_route_static: the per-block counts and first rows live in this array instead of a
+// Scratch of moe_route_static: the per-block counts (and the row of totals) live in this array instead of a
 // caller-provided workspace.  One copy per GPU, held until the process ends; every call on a GPU uses
 // that GPU's copy (the count kernel rewrites all of the part a call reads, so nothing needs clearing,
 // but two calls that overlap in time on one GPU race on it).
@@ -245,6 +279,9 @@ int launch_route(const moe_route_args* a, hipStream_t stream) {
     }
     if (nblocks > 0)
         hipLaunchKernelGGL(route_count_kernel, dim3((unsigned)nblocks), dim3(RT_BLOCK), 0, stream, ids, counts, n, (int)a->E);
+    const int prefixed = nblocks > RT_FUSED_SCAN_MAX_BLOCKS ? 1 : 0;
+    if (prefixed)
+        hipLaunchKernelGGL(route_scan_kernel, dim3((unsigned)((a->E + 3) / 4)), dim3(256), 0, stream, counts, (int)a->E, nblocks);
     // one block even without choices: it writes group_list (all zeros then)
     const size_t lds = (size_t)18 * a->E * sizeof(int);
     static std::atomic<uint64_t> lds_set{0};
@@ -252,7 +289,7 @@ int launch_route(const moe_route_args* a, hipStream_t stream) {
         return rc;
     hipLaunchKernelGGL(route_rank_kernel, dim3((unsigned)(nblocks > 0 ? nblocks : 1)), dim3(RT_BLOCK), lds, stream, ids, counts,
                        static_cast<int64_t*>(a->group_list), static_cast<int32_t*>(a->row_token),
-                       static_cast<int32_t*>(a->row_of_choice), n, (int)a->E, (int)a->topk, nblocks);
+                       static_cast<int32_t*>(a->row_of_choice), n, (int)a->E, (int)a->topk, nblocks, prefixed);
     if (hipGetLastError() != hipSuccess) return MOE_ERR_LAUNCH;
     if (a->x && n > 0) {
         hipLaunchKernelGGL(route_scatter_kernel, dim3((unsigned)a->T), dim3(256), 0, stream,

@@ -6,11 +6,14 @@
  * Every launch is asynchronous on the given stream, never synchronizes the
  * device, never copies group_list to the host and allocates nothing.  The only
  * state between calls is set-up done once per process or GPU (a kernel attribute,
- * the address of moe_route_static's scratch array) and the tile counters of the
- * grouped GEMM kernels: 8 KB of the library's own device memory, 1024 slots, each
- * launch takes the next slot and its kernel leaves it at zero again, so launches
- * may overlap on different streams and replay from HIP graphs (a launch would
- * collide with another only if that one were still running 1024 launches later).
+ * the CU count, the address of moe_route_static's scratch array) and the tile counters
+ * of the grouped GEMM kernels: 32 KB of the library's own device memory, 1024 slots.
+ * An eager launch takes the next slot and stamps it with its own epoch, so nothing a
+ * kernel leaves in a slot can mislead a later one; launches may overlap on different
+ * streams (two eager launches would share a slot only if one were still running 1024
+ * launches after it was issued).  A launch made while its stream is being captured
+ * into a HIP graph takes no slot and walks its tiles in a fixed order, so graphs may
+ * be replayed any number of times, beside each other and beside eager launches.
  * Calls are re-entrant except where moe_route_static says otherwise.  All functions
  * return MOE_OK (0) or a negative moe_status; nothing throws across this boundary.
  *
@@ -241,7 +244,7 @@ int moe_route(const moe_route_args *args, moe_stream_t stream);
  * reference.  Same arguments and results as moe_route; args->workspace is ignored (may be NULL): the
  * scratch is a static device array inside the library, MOE_ROUTE_STATIC_SCRATCH_BYTES per GPU, held
  * until the process ends.  Calls whose moe_route_workspace_bytes() exceeds it return MOE_ERR_TOO_LARGE
- * (with 256 experts that is more than 2097152 routed choices T * topk).  Allocates nothing; the first
+ * (with 256 experts that is more than 2096128 routed choices T * topk).  Allocates nothing; the first
  * call on a GPU looks the array's address up (hipGetSymbolAddress), so make that call with the GPU
  * current and outside a stream capture.  All calls on one GPU share the array: calls that overlap in
  * time on the same GPU race on it -- keep them on one stream or otherwise ordered. */

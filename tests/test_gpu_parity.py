@@ -199,10 +199,11 @@ def test_decode_batches_on_the_small_tile_kinds(fmt, shape, op):
     assert (got[gl[-1]:] == 0x7FC0).all()
 
 
-def test_gemm_tile_queue_is_rearmed_after_every_launch():
-    """The persistent grid takes its last tiles from a counter in device memory; every launch uses one of 1024
-    counter slots and must leave it at zero.  More launches than slots, on two streams, with more tiles than
-    workgroups: a slot that was not put back would make a later launch skip tiles (rows left unwritten)."""
+def test_gemm_tile_queue_slots_are_reused_safely():
+    """The persistent grid takes its last tiles from counters in device memory; every launch uses one of 1024
+    slots and stamps it with its epoch, so whatever an earlier launch left in a slot counts as zero.  More
+    launches than slots, on two streams, with more tiles than workgroups: a launch misled by a slot's old
+    content would skip tiles (rows left unwritten)."""
     import moe_gfx950 as mg
     _say("gemm tile queue: 2300 launches")
     rng = np.random.default_rng(5)

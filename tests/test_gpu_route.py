@@ -124,6 +124,47 @@ def test_route_dropped_choices_with_rows_gathered():
     assert np.array_equal(xs[: ref_rt.size], x[ref_rt]) and (xs[ref_rt.size:] == 0x7FC0).all()
 
 
+def test_route_rows_with_fewer_finite_logits_than_topk():
+    """Masked experts carry -inf logits.  A row with fewer than topk finite logits fills up with masked experts in
+    ascending id order (a stable sort by descending logit) and never names an expert twice."""
+    _say("route masked logits")
+    rng = np.random.default_rng(21)
+    T, E, K, topk = 40, 200, 64, 6
+    logits = rng.standard_normal((T, E)).astype(np.float32)
+    for t in range(T):
+        keep = rng.choice(E, size=t % (topk + 2), replace=False)     # 0 .. topk + 1 finite logits
+        row = np.full(E, -np.inf, dtype=np.float32)
+        row[keep] = logits[t, keep]
+        logits[t] = row
+    x = oracle.f32_to_bf16_bits(rng.standard_normal((T, K)).astype(np.float32))
+    ids, w, gl, rt, roc, xs = _route(logits, None, x, T, E, K, topk)
+    for t in range(T):
+        assert len(set(ids[t])) == topk, f"row {t} names an expert twice: {ids[t]}"
+    finite = [t for t in range(T) if t % (topk + 2) > 0]          # a row of -inf only has no softmax (NaN weights)
+    ref_ids, ref_w = R.route_topk(logits[finite], topk)
+    assert np.array_equal(ids[finite], ref_ids)
+    assert np.allclose(w[finite], ref_w, rtol=1e-5, atol=1e-9)
+    all_ref = np.argsort(-logits, axis=1, kind="stable")[:, :topk].astype(np.int32)
+    assert np.array_equal(ids, all_ref)
+    ref_gl, ref_rt, ref_roc = R.route_sort(all_ref, E)
+    assert np.array_equal(gl, ref_gl) and np.array_equal(rt, ref_rt) and np.array_equal(roc, ref_roc)
+
+
+def test_route_many_blocks_uses_the_scan_kernel():
+    """More than 64 blocks of 1024 choices: the per-block counts go through a scan kernel of their own."""
+    _say("route many blocks")
+    rng = np.random.default_rng(22)
+    T, E, K, topk = 20000, 160, 64, 8                  # 157 blocks
+    logits = rng.standard_normal((T, E)).astype(np.float32)
+    x = oracle.f32_to_bf16_bits(rng.standard_normal((T, K)).astype(np.float32))
+    ids, w, gl, rt, roc, xs = _route(logits, None, x, T, E, K, topk)
+    ref_ids, _ = R.route_topk(logits, topk)
+    assert np.array_equal(ids, ref_ids)
+    ref_gl, ref_rt, ref_roc = R.route_sort(ref_ids, E)
+    assert np.array_equal(gl, ref_gl) and np.array_equal(rt, ref_rt) and np.array_equal(roc, ref_roc)
+    assert np.array_equal(xs, x[ref_rt])
+
+
 def test_routed_rows_feed_the_grouped_gemm():
     """End to end on the device: logits -> routing -> grouped GEMM on the sorted rows with the
     group_list the routing wrote; expected value from the oracle on the oracle's own sort."""

@@ -120,7 +120,7 @@ def test_fp8_accepts_n_multiple_of_128(op):
 
 
 def test_route_static_limit_is_checked_on_the_host():
-    # ceil(T * topk / 1024) * E * 4 bytes of scratch: 1024 experts, 2^20 choices -> 4 MiB > 2 MiB
+    # (ceil(T * topk / 1024) + 1) * E * 4 bytes of scratch: 1024 experts, 2^20 choices -> 4 MiB > 2 MiB
     a = mg.route_args(P, 0, P, P, P, P, P, 0, 0, 1 << 17, 1024, 0, 8)
     assert mg.route_workspace_bytes(a) > mg.ROUTE_STATIC_SCRATCH_BYTES
     assert mg.lib.moe_route_static(ctypes.byref(a), None) == mg.ERR_TOO_LARGE

@@ -54,10 +54,56 @@ def test_route_static_matches_route_twice_second_smaller():
         assert got[2][-1] == T * topk
 
 
+def test_route_static_allocates_nothing_and_replays_from_a_graph():
+    """The contract of the entry point: after its first call on a GPU (the one that looks the scratch array's
+    address up) it allocates no device memory -- the free memory the driver reports does not change over
+    further calls -- and it can be captured into a HIP graph; every replay must give moe_route's result."""
+    import moe_gfx950 as mg
+    import oracle
+
+    T, E, K, topk = 1500, 96, 256, 4
+    print(f"route_static no-alloc / graph T={T} E={E}", flush=True)
+    sys.stdout.flush()
+    rng = np.random.default_rng(3)
+    logits = rng.standard_normal((T, E)).astype(np.float32)
+    x = oracle.f32_to_bf16_bits(rng.standard_normal((T, K)).astype(np.float32))
+    want = _run("plain", logits, x, T, E, K, topk)
+    _run("static", logits, x, T, E, K, topk)                 # first call on this GPU, outside any capture
+    dev = torch.device("cuda")
+    n = T * topk
+    d_logits = torch.from_numpy(logits).to(dev)
+    d_x = torch.from_numpy(x.view(np.int16)).to(dev)
+    outs = [torch.empty((n,), dtype=torch.int32, device=dev), torch.empty((n,), dtype=torch.float32, device=dev),
+            torch.empty((E,), dtype=torch.int64, device=dev), torch.empty((n,), dtype=torch.int32, device=dev),
+            torch.empty((n,), dtype=torch.int32, device=dev), torch.empty((n, K), dtype=torch.int16, device=dev)]
+    args = mg.route_args(d_logits.data_ptr(), d_x.data_ptr(), outs[0].data_ptr(), outs[1].data_ptr(), outs[2].data_ptr(),
+                         outs[3].data_ptr(), outs[4].data_ptr(), outs[5].data_ptr(), 0, T, E, K, topk)
+    side = torch.cuda.Stream()
+    mg.route_static(args, side.cuda_stream)                   # the runtime's own set-up of a new stream happens here
+    torch.cuda.synchronize()
+    free_before = torch.cuda.mem_get_info()[0]
+    reserved_before = torch.cuda.memory_reserved()
+    for _ in range(3):
+        mg.route_static(args, side.cuda_stream)
+    side.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free_before and torch.cuda.memory_reserved() == reserved_before
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g, stream=side):
+        mg.route_static(args, torch.cuda.current_stream().cuda_stream)
+    for rep in range(3):
+        for t in outs:
+            t.fill_(-3)                                       # eager work between the replays
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        for t, w, name in zip(outs, want, ("topk_ids", "topk_weight", "group_list", "row_token", "row_of_choice", "x_sorted")):
+            assert np.array_equal(t.cpu().numpy(), w), f"replay {rep}: {name}"
+
+
 def test_route_static_rejects_sizes_beyond_its_scratch():
     import moe_gfx950 as mg
 
-    # ceil(T * topk / 1024) * E * 4 bytes of scratch: 1024 experts, 2^20 choices -> 4 MiB > 2 MiB
+    # (ceil(T * topk / 1024) + 1) * E * 4 bytes of scratch: 1024 experts, 2^20 choices -> 4 MiB > 2 MiB
     args = mg.route_args(16, 0, 16, 16, 16, 16, 16, 0, 0, 1 << 17, 1024, 0, 8)
     assert mg.route_workspace_bytes(args) > mg.ROUTE_STATIC_SCRATCH_BYTES
     with pytest.raises(mg.MoeError) as e:
