@@ -127,6 +127,7 @@ __device__ __forceinline__ int queue_resolve(unsigned int* slot, int xcd, unsign
 struct Ticket {
     unsigned int* counter;   // null: the caller draws the ticket itself
     int* out;
+    int* arrivals;           // a word of LDS for the tile routine's arrival counter (see gemm_tile_pair)
 };
 
 // Buffer resources keep the addressing compact: one 128-bit descriptor in SGPRs per
@@ -426,6 +427,19 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& P, u32x4_t* lds_a, i
 __device__ __forceinline__ void lds_load16(rsrc_t r, const u32x4_t* dst, int voff, int soff) {
     __builtin_amdgcn_raw_ptr_buffer_load_lds(r, MOE_LDS_PTR(const_cast<u32x4_t*>(dst)), 16, voff, soff, 0, 0);
 }
+// The same with the destination as a byte address in LDS (wave-uniform).
+__device__ __forceinline__ uint32_t lds_address(const void* p) {
+    return (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(uintptr_t)MOE_LDS_PTR(p));
+}
+__device__ __forceinline__ void lds_load16_at(rsrc_t r, uint32_t dst, int voff, int soff) {
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (__attribute__((address_space(3))) void*)(uintptr_t)dst, 16, voff, soff, 0, 0);
+}
+// A wave-uniform value the compiler must take as it finds it: whatever is derived from the result is computed
+// where it is used instead of once per variant ahead of an unrolled loop (where it would occupy an SGPR each).
+__device__ __forceinline__ uint32_t here(uint32_t v) {
+    asm volatile("" : "+s"(v));
+    return v;
+}
 
 // ---------------------------------------------------------------------------------
 // Tile routine for the quantized containers (int4, int8, reference fp4 / fp8, K-contiguous fp4) with two
@@ -442,16 +456,16 @@ __device__ __forceinline__ void lds_load16(rsrc_t r, const u32x4_t* dst, int vof
 // element), and each wavefront reads half of the x fragments.
 //
 // Each wavefront alternates a decode phase (its sub-step of the packed stage -> 4 bf16 B
-// fragments in registers) and an MFMA phase.  The phases of a pair are kept in opposition by
-// the position of the step's barrier: the wavefronts of sub-step 0 take it after their MFMA
-// phase, those of sub-step 1 half way through their decode phase, so that after every
-// barrier one wavefront of the SIMD starts decoding while the other starts multiplying.
+// fragments in registers) and an MFMA phase; one wavefront of a SIMD multiplies while the other
+// decodes.  The steps of the 8 wavefronts are tied together by a split barrier, an arrival counter
+// in LDS (see ring_arrive / ring_wait in gemm_tile_pair): a wavefront that is done with a step says
+// so and goes on decoding the next one; it waits for the others only in front of its next MFMA phase.
 //
 // Everything the k loop consumes -- x tile, packed weight tile, scales -- is brought in by
 // LDS-direct loads into a ring of S = 5 stages.  The loads of stage kt+4 (it replaces stage kt-1,
-// last read before barrier kt-1) and the LDS reads of the packed dwords of stage kt+1 are
-// spread between the MFMAs of step kt; before barrier kt each wavefront waits until its own
-// loads of stage kt+2 have landed.  vmcnt counts a wavefront's loads in order and every
+// which every wavefront has left when all have arrived kt times) and the LDS reads of the packed
+// dwords of stage kt+1 are spread between the MFMAs of step kt; before it arrives at the end of step
+// kt each wavefront waits until its own loads of stage kt+2 have landed.  vmcnt counts a wavefront's loads in order and every
 // wavefront issues the same number NI of them per step (waves without a row block of their
 // own repeat one: measured, the repeated loads cost nothing, a branch around them does), so "at most
 // (S - 3) NI outstanding" means exactly that.
@@ -656,19 +670,27 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
     constexpr int BK = 64, S = pair_stages<FMT>(), PAIR_SC_UNITS = pair_sc_units<FMT>();
     constexpr int PAIR_B_UNITS = pair_b_units<FMT>();
     constexpr int AHEAD = S - 1;   // a step's loads fill the stage of step kt + AHEAD
+    // Kinds of which two workgroups share a CU (decode batches, HBM bound) keep one s_barrier per step, placed so
+    // that the two wavefronts of a SIMD alternate (those of sub-step 0 take it after their MFMA phase, those of
+    // sub-step 1 half way through their decode); with one workgroup per CU the split barrier described below is
+    // faster (measured on 512 rows over 256 experts of 7168 x 2048: two per CU 335 against 340 us (int4), 390 against
+    // 395 us (fp4) with the plain barrier; one per CU, fp8, 555 against 580 us with the split one).
+    constexpr bool SPLIT_BARRIER = pair_wg_per_cu<FMT>(KIND) == 1;
     constexpr int PAIR_A_UNITS = pair_a_units(KIND);
     static_assert(16 * MT * 8 <= PAIR_A_UNITS, "tile rows beyond the x stage");
     u32x4_t* lds_a = smem;
     u32x4_t* lds_b = lds_a + S * PAIR_A_UNITS;
     u32x4_t* lds_s = lds_b + S * PAIR_B_UNITS;
 
-    const int tid = threadIdx.x, lane = tid & 63;
+    // (the thread id is taken as found: what is derived from it is worked out per tile and does not hold
+    // registers from tile to tile, where the routine has none to spare)
+    int tid = threadIdx.x;
+    asm volatile("" : "+v"(tid));
+    const int lane = tid & 63;
     const int i = lane & 15, q = lane >> 4;
     const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int cw = wv & 3;                                    // column group: 64 columns
-    // the sub-step of every step this wavefront owns.  The SIMD's issue arbitration favours the
-    // wavefront in the lower slot (wv < 4); measured, the pair runs 20 % faster when that one takes
-    // the role whose barrier sits inside the decode phase
+    // the sub-step of every step this wavefront owns
     const int h = 1 - (wv >> 2);
     // this lane's 4 columns (MFMA t = column col0 + t): half of a dword of 8 4-bit codes, or a dword of 4 bytes
     const int col0 = B8 ? 64 * cw + 4 * i : 128 * (cw >> 1) + 8 * i + 4 * (cw & 1);
@@ -736,24 +758,31 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
     const int cs = FP4 ? n0 * 2 + (wv & 1) * 256 : n0 * 2 + (wv & 3) * 128;
     const int lane16 = lane * 16;
     const bool s_lane = lane < (FP4 ? 16 : 8);
+    // where this wavefront's loads land in stage 0 (byte addresses in LDS)
+    uint32_t a_at[NA];
+#pragma unroll
+    for (int m = 0; m < NA; ++m) a_at[m] = lds_address(lds_a + ja[m]);
+    const uint32_t b_at = lds_address(lds_b + wv * (PAIR_B_UNITS / 8));
+    const uint32_t s_at = lds_address(lds_s + wv * (F8 ? 1 : PAIR_SC_UNITS / 8));
     // m-th load of group kt (stage kt+AHEAD of x, packed tile and scales), into LDS stage ST
     auto issue = [&](int m, int kt, int ST) {
         if (m < NA) {
-            lds_load16(rx, lds_a + ST * PAIR_A_UNITS + ja[m], va, ca[m] + (kt + AHEAD) * (BK * 2));
+            lds_load16_at(rx, here(a_at[m]) + ST * (PAIR_A_UNITS * 16), va, ca[m] + (kt + AHEAD) * (BK * 2));
         } else if (m < NA + NB) {
             const int e = m - NA;
-            lds_load16(rw, lds_b + ST * PAIR_B_UNITS + wv * (PAIR_B_UNITS / 8) + e * 64, vb,
-                       cb + (B8 ? 4 * e * P.N : 0) + (kt + AHEAD) * kb_step);
+            lds_load16_at(rw, here(b_at) + ST * (PAIR_B_UNITS * 16) + e * 1024, vb,
+                          cb + (B8 ? 4 * e * P.N : 0) + (kt + AHEAD) * kb_step);
         } else if constexpr (KC) {
             kc_issue_scale(kt + KC_D);
         } else if constexpr (F8) {
             // the block scale of the stage's 128-k block, 4 bytes by lane 0 (past K: reads as 0, unused)
             if (lane == 0)
-                __builtin_amdgcn_raw_ptr_buffer_load_lds(rs8, MOE_LDS_PTR(lds_s + ST * PAIR_SC_UNITS + wv), 4, 0,
-                                                         ((kt + AHEAD) >> 1) * (P.N >> 7) * 4 + cs8, 0, 0);
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(
+                    rs8, (__attribute__((address_space(3))) void*)(uintptr_t)(here(s_at) + ST * (PAIR_SC_UNITS * 16)), 4, 0,
+                    ((kt + AHEAD) >> 1) * (P.N >> 7) * 4 + cs8, 0, 0);
         } else {
             const int grow = FP4 ? (kt + AHEAD) * 4 + (wv >> 1) : scale_row((uint32_t)((kt + AHEAD) * 2 + (wv >> 2)));
-            if (s_lane) lds_load16(rs, lds_s + ST * PAIR_SC_UNITS + wv * (PAIR_SC_UNITS / 8), lane16, grow * (P.N * 2) + cs);
+            if (s_lane) lds_load16_at(rs, here(s_at) + ST * (PAIR_SC_UNITS * 16), lane16, grow * (P.N * 2) + cs);
         }
     };
     auto issue_group = [&](int kt, int ST) {
@@ -794,8 +823,40 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
     // groups -AHEAD .. -1: stages 0 .. AHEAD-1; stages 0 and 1 must have landed before the first barrier
     // (WAITN: the loads of the S - 3 youngest groups may still be in flight at a barrier)
     constexpr int WAITN = (S - 3) * NI;
-    // wait until this wavefront's loads of all but the S - 3 youngest groups have landed, then the step's barrier
+    // wait until this wavefront's loads of all but the S - 3 youngest groups have landed, then a barrier (prologue)
     auto ring_barrier = [&]() { asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(WAITN) : "memory"); };
+    // Inside the k loop the step's barrier is split in two.  A wavefront "arrives" at the end of step kt: it is
+    // done with stage kt, and its loads of stage kt + 2 have landed; it adds 1 to a counter in LDS.  It only
+    // "waits" -- polls the counter until all 8 wavefronts have arrived kt times -- at the start of the MFMA phase
+    // of step kt + 1, in front of the first things that need the others: the loads that overwrite stage kt and
+    // the packed dwords of stage kt + 2.  A whole decode phase lies between the two, so a wavefront that is late
+    // by less than that stalls nobody (measured against one s_barrier per step: 7 % at K = 7168, 4 % at K = 2048).
+    // Everything is inline asm so that the compiler can move nothing across it; every wavefront arrives once in
+    // every step of a tile, so every wait ends.  The counter is zeroed per tile, ahead of the prologue's barrier.
+    // (the counter's address stays in an SGPR; the asm makes its vector operands on the spot, so that no vector
+    // register is held for them through the decode)
+    const uint32_t arrivals_at = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(uintptr_t)MOE_LDS_PTR(tk.arrivals));
+    const __attribute__((address_space(3))) uint32_t* arrivals_lds =
+        reinterpret_cast<const __attribute__((address_space(3))) uint32_t*>(MOE_LDS_PTR(tk.arrivals));
+    uint32_t arrivals_seen = 0u;
+    if (tid == 0) {
+        uint32_t va, vz;
+        asm volatile("v_mov_b32 %0, %2\n\tv_mov_b32 %1, 0\n\ts_nop 0\n\tds_write_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)"
+                     : "=&v"(va), "=&v"(vz) : "s"(arrivals_at) : "memory");
+    }
+    auto ring_arrive = [&]() {
+        uint32_t va, v1;
+        asm volatile("s_waitcnt vmcnt(%2)\n\tv_mov_b32 %0, %3\n\tv_mov_b32 %1, 1\n\ts_mov_b64 exec, 1\n\tds_add_u32 %0, %1\n\ts_mov_b64 exec, -1"
+                     : "=&v"(va), "=&v"(v1) : "n"(WAITN), "s"(arrivals_at) : "memory");
+    };
+    // early: the counter as read half a decode phase ago (usually enough, and its latency is hidden)
+    auto ring_wait = [&](uint32_t steps, uint32_t early) {
+        uint32_t seen_v, seen_s;
+        asm volatile("v_readfirstlane_b32 %1, %4\n\ts_cmp_ge_u32 %1, %3\n\ts_cbranch_scc1 2f\n"
+                     "1:\n\tv_mov_b32 %0, %2\n\ts_nop 0\n\tds_read_b32 %0, %0\n\ts_waitcnt lgkmcnt(0)\n\tv_readfirstlane_b32 %1, %0\n\ts_cmp_ge_u32 %1, %3\n\t"
+                     "s_cbranch_scc1 2f\n\ts_sleep 1\n\ts_branch 1b\n2:"
+                     : "=&v"(seen_v), "=&s"(seen_s) : "s"(arrivals_at), "s"(8u * steps), "v"(early) : "memory", "scc");
+    };
     if constexpr (KC) {
         // the scale loads the groups below do not cover (older than all of them: landed by the first barrier)
 #pragma unroll
@@ -891,7 +952,7 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
 
     // One data step; st = step mod S is its LDS stage, sn the next one, sl the stage this step's loads
     // go to (wave-uniform).
-    auto step = [&](int kt, int st, int sn, int sl) {
+    auto step = [&](int kt, int st, int sn, int sl) __attribute__((always_inline)) {
         const u32x4_t* la = lds_a + st * PAIR_A_UNITS;
         // ---- decode phase: this wavefront's sub-step of the packed stage -> bf[0..3]
         float m[4], z[4];
@@ -916,10 +977,11 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
 #pragma unroll
         for (int p0 = 0; p0 < 4; p0 += 2) {
             if (p0 == 2) {
-                if (h == 1) {
+                if constexpr (SPLIT_BARRIER) {
+                    arrivals_seen = *arrivals_lds;   // a first look at the counter, checked after the decode
+                } else if (h == 1) {
                     // barrier kt-1 for the wavefronts that own sub-step 1, half way through their decode
-                    // (not in the tile's first step: the barrier of the prologue stands for it); x stage
-                    // kt is visible behind it
+                    // (not in the tile's first step: the barrier of the prologue stands for it)
                     if (kt > 0) ring_barrier();
                 }
                 // first x fragments of the MFMA phase, read under the rest of the decode
@@ -1078,10 +1140,12 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
         // ---- MFMA phase, at raised issue priority: the other wavefront of the SIMD is decoding
         // meanwhile and would otherwise win the arbitration whenever both are ready, starving
         // the matrix pipe; its VALU instructions fit into the gaps the MFMAs leave
+        // every wavefront has arrived kt times (none in the tile's first step: the prologue's barrier stands for it)
+        if constexpr (SPLIT_BARRIER) ring_wait((uint32_t)kt, arrivals_seen);
+        __builtin_amdgcn_sched_barrier(0);
         __builtin_amdgcn_s_setprio(3);
-        // Both kinds of wavefront are past barrier kt-1 here: this step's loads (stage kt+4 replaces
-        // stage kt-1) and the packed dwords of the next step (stage kt+1, visible since that
-        // barrier) are fetched between the MFMAs.
+        // Everybody is done with stage kt-1 and has its part of stage kt+1 in LDS: this step's loads (stage kt+4
+        // replaces stage kt-1) and the packed dwords of the next step (stage kt+1) are fetched between the MFMAs.
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
             if (mt + R < MT) afr[(mt + R) & 3] = la[a_lds_unit<BK>(16 * (mt + R) + xrow, 4 * h + q)];
@@ -1136,18 +1200,37 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
             __builtin_amdgcn_sched_barrier(0);
         }
         __builtin_amdgcn_s_setprio(0);
-        if (h == 0) ring_barrier();   // barrier kt
+        if constexpr (SPLIT_BARRIER) {
+            ring_arrive();
+        } else if (h == 0) {
+            ring_barrier();   // barrier kt
+        }
     };
-    for (int kt = 0, st = 0, sl = S - 1; kt < nk; ++kt) {
-        const int sn = st == S - 1 ? 0 : st + 1;
-        step(kt, st, sn, sl);
-        st = sn;
-        sl = sl == S - 1 ? 0 : sl + 1;
+    // unrolled over the ring, so that every stage number is a constant and the LDS addresses of a step are
+    // immediate offsets (with run-time stage numbers a step spent 9 vector and about 25 scalar instructions on
+    // them: measured 10 % of the kernel's time at K = 7168); a tile starts at stage 0
+    // (the K-contiguous containers keep run-time stage numbers: their routine has no registers left for the
+    // unrolled form)
+    if constexpr (!KC) {
+        for (int kt0 = 0; kt0 < nk; kt0 += S) {
+#pragma unroll
+            for (int u = 0; u < S; ++u)
+                if (kt0 + u < nk) step(kt0 + u, u, (u + 1) % S, (u + S - 1) % S);
+        }
+    } else {
+        for (int kt = 0, st = 0, sl = S - 1; kt < nk; ++kt) {
+            const int sn = st == S - 1 ? 0 : st + 1;
+            step(kt, st, sn, sl);
+            st = sn;
+            sl = sl == S - 1 ? 0 : sl + 1;
+        }
     }
-    if (h == 1) ring_barrier();       // barrier nk-1
+    if constexpr (!SPLIT_BARRIER)
+        if (h == 1) ring_barrier();   // barrier nk-1
     // drain this wavefront's loads (they target stages past K and are never read); the
     // accumulators were last written by MFMAs the compiler cannot see: wait out their latency
-    asm volatile("s_waitcnt vmcnt(0)\n\ts_nop 15\n\ts_nop 15\n\ts_barrier" ::: "memory");
+    // (and the last arrivals are counted before anybody zeroes the counter for the next tile)
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_nop 15\n\ts_nop 15\n\ts_barrier" ::: "memory");
 
     if constexpr (STACK2) {
         // the lanes q and q + 2 hold the two scale groups' sums of the same rows
@@ -1334,7 +1417,7 @@ __global__ __launch_bounds__((64 * KernelCfg<FMT, KIND>::WAVES), (KernelCfg<FMT,
         }
         // from the last tile of the fixed order on, the k-split tile routines draw the next ticket themselves
         const bool take = C::PAIR && queued && sw + 1 >= fixed_sweeps;
-        const Ticket tk = {take ? q_slot + xcd : nullptr, part};
+        const Ticket tk = {take ? q_slot + xcd : nullptr, part, part + 2};
         have_ticket = take;
         // largest g with prefix[g] <= T (empty experts have prefix[g] == prefix[g+1]): every wavefront looks at 64
         // evenly spaced entries at once, then at the entries between two of them -- two LDS round trips
