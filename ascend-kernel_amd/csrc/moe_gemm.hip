@@ -238,6 +238,13 @@ __device__ __forceinline__ int a_lds_unit(int row, int c) {
     return row * (BK / 8) + (c ^ (row & 7));
 }
 
+// The same for tile rows of 32 k (four 16-byte chunks, 64 bytes): chunk c of row r at position c ^ ((r >> 2) & 3),
+// so that the 16 rows x 1 chunk a quarter of a wavefront reads, and the 16 rows x 4 chunks an LDS-direct load
+// writes, each cover all banks once.
+__device__ __forceinline__ int a_lds_unit32(int row, int c) {
+    return row * 4 + (c ^ ((row >> 2) & 3));
+}
+
 // Per-tile context: lane coordinates and the buffer resources of expert g.
 template <int FMT>
 __device__ __forceinline__ void make_ctx(BCtx& c, const GemmParams& P, int g, int n0) {
@@ -503,19 +510,26 @@ __device__ __forceinline__ uint32_t here(uint32_t v) {
 //   GK_PAIR_EXACT  GK_PAIR_SMALL with the GEMV op's arithmetic (weights not rounded to bf16)
 //   GK_PAIR_EXACT16  GK_PAIR_EXACT with tiles of at most 16 rows (the fp4 container: its 32-row tile routine
 //               needs 153 registers, the 16-row one 97, which lets two workgroups share a CU)
-enum { GK_GENERAL = 0, GK_SKINNY = 1, GK_PAIR = 2, GK_PAIR_EXACT = 3, GK_PAIR_SMALL = 4, GK_PAIR_EXACT16 = 5 };
+//   GK_QUAD     the large tiles of GK_PAIR without the k split: workgroups of 4 wavefronts, each wavefront takes its
+//               64 columns through the whole k range in steps of 32 k, two workgroups per CU.  The two wavefronts
+//               of a SIMD belong to different workgroups and work on different tiles: no partial sums to
+//               exchange, a barrier spans 4 wavefronts instead of 8, and while one workgroup is between two tiles
+//               (stores, tile search, first loads) the other has the SIMDs to itself.  (int4 and int8.)
+enum { GK_GENERAL = 0, GK_SKINNY = 1, GK_PAIR = 2, GK_PAIR_EXACT = 3, GK_PAIR_SMALL = 4, GK_PAIR_EXACT16 = 5, GK_QUAD = 6 };
 constexpr bool pair_exact(int kind) { return kind == GK_PAIR_EXACT || kind == GK_PAIR_EXACT16; }
+constexpr int pair_waves(int kind) { return kind == GK_QUAD ? 4 : 8; }
+constexpr int pair_bk(int kind) { return kind == GK_QUAD ? 32 : 64; }   // k per step
 
 constexpr int PAIR_CAPB = 10;                         // x stages hold 160 rows
 constexpr int PAIR_MT_MAX = 10;
 constexpr int PAIR_SMALL_MT_MAX = 2;                  // row blocks per tile of the small-stage kinds
-constexpr bool pair_small(int kind) { return kind != GK_PAIR; }
+constexpr bool pair_small(int kind) { return kind != GK_PAIR && kind != GK_QUAD; }
 // 16-byte units of one x stage: 160 rows, or the 32 rows of the small-stage kinds
-constexpr int pair_mt_max(int kind) { return kind == GK_PAIR ? PAIR_MT_MAX : kind == GK_PAIR_EXACT16 ? 1 : PAIR_SMALL_MT_MAX; }
-constexpr int pair_a_units(int kind) { return 16 * (pair_small(kind) ? pair_mt_max(kind) : PAIR_CAPB) * 8; }
-// packed tile of one k step: 64 rows of 128 bytes (4-bit codes) or of 256 bytes (int8, fp8)
+constexpr int pair_mt_max(int kind) { return !pair_small(kind) ? PAIR_MT_MAX : kind == GK_PAIR_EXACT16 ? 1 : PAIR_SMALL_MT_MAX; }
+constexpr int pair_a_units(int kind) { return 16 * (pair_small(kind) ? pair_mt_max(kind) : PAIR_CAPB) * (pair_bk(kind) / 8); }
+// packed tile of one k step: rows of 128 bytes (4-bit codes) or of 256 bytes (int8, fp8)
 template <int FMT>
-constexpr int pair_b_units() { return (FMT == MOE_FMT_INT8 || FMT == MOE_FMT_FP8_REF) ? 64 * 16 : 64 * 8; }
+constexpr int pair_b_units(int kind) { return pair_bk(kind) * ((FMT == MOE_FMT_INT8 || FMT == MOE_FMT_FP8_REF) ? 16 : 8); }
 // Small-stage kinds on the 4-bit N-contiguous containers: two workgroups per CU, one computes while the other
 // waits at its barrier or between two tiles (512 rows over 256 experts of 7168 x 2048: int4 425 -> 387 us, fp4
 // 440 -> 425 us; the fp4 tile routine with the GEMV op's arithmetic fits four wavefronts per SIMD only in its
@@ -524,6 +538,7 @@ constexpr int pair_b_units() { return (FMT == MOE_FMT_INT8 || FMT == MOE_FMT_FP8
 // to fill), and the one-byte containers at two workgroups per CU are left with 3 stages (fp8 641 us).
 template <int FMT>
 constexpr int pair_wg_per_cu(int kind) {
+    if (kind == GK_QUAD) return 2;
     if (!pair_small(kind)) return 1;
     return (FMT == MOE_FMT_INT4 || (FMT == MOE_FMT_FP4_REF && kind != GK_PAIR_EXACT)) ? 2 : 1;
 }
@@ -534,14 +549,16 @@ constexpr int pair_stages() { return (FMT == MOE_FMT_INT8 || FMT == MOE_FMT_FP8_
 // of 32), the reference fp4 container one per 16 k; fp8 one unit per wavefront holding the fp32 scale of
 // its 128 x 128 block; int8 none (per-channel scales stay in registers)
 template <int FMT>
-constexpr int pair_sc_units() { return FMT == MOE_FMT_FP4_REF ? 128 : FMT == MOE_FMT_INT4 ? 64 : FMT == MOE_FMT_FP8_REF ? 8 : 0; }
+constexpr int pair_sc_units(int kind) {
+    return (FMT == MOE_FMT_FP4_REF ? 128 : FMT == MOE_FMT_INT4 ? 64 : FMT == MOE_FMT_FP8_REF ? 8 : 0) * pair_bk(kind) / 64;
+}
 // The K-contiguous fp4 containers keep their scales [N, K/block] outside the stages: 16 bytes (2 or 4 steps'
 // worth) per weight row at a time, three buffers of 256 rows
 template <int FMT>
 constexpr int pair_kc_scale_units() { return (FMT == MOE_FMT_FP4_B32 || FMT == MOE_FMT_FP4_B16) ? 3 * 256 : 0; }
 template <int FMT>
 constexpr int pair_lds_units(int kind) {
-    return pair_stages<FMT>() * (pair_a_units(kind) + pair_b_units<FMT>() + pair_sc_units<FMT>()) + pair_kc_scale_units<FMT>();
+    return pair_stages<FMT>() * (pair_a_units(kind) + pair_b_units<FMT>(kind) + pair_sc_units<FMT>(kind)) + pair_kc_scale_units<FMT>();
 }
 
 // End of a k-split tile.  The two wavefronts of a pair (same columns, the two k halves) hold partial sums of the
@@ -549,7 +566,8 @@ constexpr int pair_lds_units(int kind) {
 // row blocks it keeps and stores those: the first half of the tile's 16-row blocks is finished by the h == 0
 // wavefront, the second by h == 1, so both reduce and store at the same time.  Rounds of at most 4 row
 // blocks (8 wavefronts x 4 blocks x 4 KB fit the x stage area, free now).
-template <int MT, bool KC>
+// WHOLE: the wavefront holds the whole sums (no k split): it stores all of its row blocks, nothing is exchanged.
+template <int MT, bool KC, bool WHOLE = false>
 __device__ __forceinline__ void pair_finish(const GemmParams& P, u32x4_t* smem, f32x4_t (&acc)[MT][4], int h, int cw, int lane,
                                             int col0, int64_t row0, int rows, int n0, const Ticket& tk) {
     const int i = lane & 15, q = lane >> 4;
@@ -633,10 +651,14 @@ __device__ __forceinline__ void pair_finish(const GemmParams& P, u32x4_t* smem, 
             }
         }
     };
-    if (h == 0)
+    if constexpr (WHOLE) {
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) store_block(mt);
+    } else if (h == 0) {
         finish(std::integral_constant<int, 0>{});
-    else
+    } else {
         finish(std::integral_constant<int, 1>{});
+    }
     if (takes) *tk.out = (int)next_tile;
     lds_barrier();   // the slots are read: the next tile may load into the ring (the stores are still in flight)
 }
@@ -667,8 +689,12 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
     constexpr bool KC = FMT == MOE_FMT_FP4_B32 || FMT == MOE_FMT_FP4_B16;
     constexpr int KBLK = FMT == MOE_FMT_FP4_B32 ? 32 : 16;
     constexpr bool B8 = I8 || F8;   // one byte per weight: tiles of 64 rows x 256 bytes
-    constexpr int BK = 64, S = pair_stages<FMT>(), PAIR_SC_UNITS = pair_sc_units<FMT>();
-    constexpr int PAIR_B_UNITS = pair_b_units<FMT>();
+    // Q4: the kind without the k split (GK_QUAD): 4 wavefronts, steps of 32 k, every wavefront in every step
+    constexpr bool Q4 = KIND == GK_QUAD;
+    static_assert(!Q4 || FMT == MOE_FMT_INT4 || FMT == MOE_FMT_INT8, "the 4-wavefront kind serves int4 and int8");
+    constexpr int NW = pair_waves(KIND);
+    constexpr int BK = pair_bk(KIND), S = pair_stages<FMT>(), PAIR_SC_UNITS = pair_sc_units<FMT>(KIND);
+    constexpr int PAIR_B_UNITS = pair_b_units<FMT>(KIND);
     constexpr int AHEAD = S - 1;   // a step's loads fill the stage of step kt + AHEAD
     // Kinds of which two workgroups share a CU (decode batches, HBM bound) keep one s_barrier per step, placed so
     // that the two wavefronts of a SIMD alternate (those of sub-step 0 take it after their MFMA phase, those of
@@ -677,7 +703,7 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
     // 395 us (fp4) with the plain barrier; one per CU, fp8, 555 against 580 us with the split one).
     constexpr bool SPLIT_BARRIER = pair_wg_per_cu<FMT>(KIND) == 1;
     constexpr int PAIR_A_UNITS = pair_a_units(KIND);
-    static_assert(16 * MT * 8 <= PAIR_A_UNITS, "tile rows beyond the x stage");
+    static_assert(16 * MT * (BK / 8) <= PAIR_A_UNITS, "tile rows beyond the x stage");
     u32x4_t* lds_a = smem;
     u32x4_t* lds_b = lds_a + S * PAIR_A_UNITS;
     u32x4_t* lds_s = lds_b + S * PAIR_B_UNITS;
@@ -690,8 +716,8 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
     const int i = lane & 15, q = lane >> 4;
     const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int cw = wv & 3;                                    // column group: 64 columns
-    // the sub-step of every step this wavefront owns
-    const int h = 1 - (wv >> 2);
+    // the sub-step of every step this wavefront owns (Q4: a step is one sub-step)
+    const int h = Q4 ? 0 : 1 - (wv >> 2);
     // this lane's 4 columns (MFMA t = column col0 + t): half of a dword of 8 4-bit codes, or a dword of 4 bytes
     const int col0 = B8 ? 64 * cw + 4 * i : 128 * (cw >> 1) + 8 * i + 4 * (cw & 1);
     const int nk = P.K / BK;
@@ -712,8 +738,11 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
     // x rows through a buffer resource that ends after the last valid row (padded rows read as
     // zeros).  Load instruction j covers rows 8j + (lane >> 3); position lane & 7 of a row
     // holds chunk (lane & 7) ^ (row & 7), the swizzle a_lds_unit expects.
+    // (Q4, rows of 64 bytes: instruction j covers rows 16j + (lane >> 2); position lane & 3 of a row holds
+    // chunk (lane & 3) ^ ((row >> 2) & 3), see a_lds_unit32)
     const rsrc_t rx = make_rsrc(P.x + row0 * (int64_t)P.K, (int64_t)rows * P.K * 2);
-    const int va = ((lane >> 3) * P.K + (((lane & 7) ^ (lane >> 3)) * 8)) * 2;
+    const int va = Q4 ? ((lane >> 2) * P.K + (((lane & 3) ^ ((lane >> 4) & 3)) * 8)) * 2
+                      : ((lane >> 3) * P.K + (((lane & 7) ^ (lane >> 3)) * 8)) * 2;
     // packed tile: instruction wv brings rows 8 wv + (lane >> 3) into the 1 KB block wv of the stage;
     // the two 64-byte halves of the rows with odd (row >> 3) are swapped, so that the four q groups
     // of a wavefront read from both halves of the banks
@@ -726,16 +755,18 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
     const int vb = KC   ? kc_n * (P.K >> 1) + 16 * ((lane & 1) ^ ((kc_n >> 3) & 1))
                    : B8 ? (lane >> 4) * P.N + (((lane & 15) ^ (4 * (wv & 3))) * 16)
                         : (lane >> 3) * (P.N >> 1) + (((lane & 7) ^ (4 * (wv & 1))) * 16);
-    constexpr int NA = (2 * MT + 7) / 8;   // x load instructions per wavefront per step
-    constexpr int NB = B8 ? 2 : 1;         // packed-tile instructions
-    constexpr int NI = NA + NB + ((PAIR_SC_UNITS || KC) ? 1 : 0);   // + an eighth of the step's scales
+    constexpr int XI = Q4 ? MT : 2 * MT;          // x load instructions per step (1 KB each: 16 or 8 rows)
+    constexpr int XROWS = Q4 ? 16 : 8;
+    constexpr int NA = (XI + NW - 1) / NW;        // ... per wavefront
+    constexpr int NB = B8 ? 2 : 1;                // packed-tile instructions
+    constexpr int NI = NA + NB + ((PAIR_SC_UNITS || KC) ? 1 : 0);   // + this wavefront's share of the step's scales
     int ja[NA], ca[NA];
 #pragma unroll
     for (int m = 0; m < NA; ++m) {
-        int j = wv + 8 * m;
-        if (8 * NA > 2 * MT) j = j % (2 * MT);   // repeat a block rather than issue fewer loads
+        int j = wv + NW * m;
+        if (NW * NA > XI) j = j % XI;   // repeat a block rather than issue fewer loads
         ja[m] = j * 64;
-        ca[m] = 8 * j * P.K * 2;
+        ca[m] = XROWS * j * P.K * 2;
     }
     const int cb = KC ? n0 * (P.K >> 1) : B8 ? 8 * wv * P.N + n0 : 8 * wv * (P.N >> 1) + (n0 >> 1);
     const int kb_step = KC ? BK / 2 : B8 ? BK * P.N : BK * (P.N >> 1);
@@ -762,8 +793,8 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
     uint32_t a_at[NA];
 #pragma unroll
     for (int m = 0; m < NA; ++m) a_at[m] = lds_address(lds_a + ja[m]);
-    const uint32_t b_at = lds_address(lds_b + wv * (PAIR_B_UNITS / 8));
-    const uint32_t s_at = lds_address(lds_s + wv * (F8 ? 1 : PAIR_SC_UNITS / 8));
+    const uint32_t b_at = lds_address(lds_b + wv * (PAIR_B_UNITS / NW));
+    const uint32_t s_at = lds_address(lds_s + wv * (F8 ? 1 : PAIR_SC_UNITS / NW));
     // m-th load of group kt (stage kt+AHEAD of x, packed tile and scales), into LDS stage ST
     auto issue = [&](int m, int kt, int ST) {
         if (m < NA) {
@@ -781,7 +812,9 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
                     rs8, (__attribute__((address_space(3))) void*)(uintptr_t)(here(s_at) + ST * (PAIR_SC_UNITS * 16)), 4, 0,
                     ((kt + AHEAD) >> 1) * (P.N >> 7) * 4 + cs8, 0, 0);
         } else {
-            const int grow = FP4 ? (kt + AHEAD) * 4 + (wv >> 1) : scale_row((uint32_t)((kt + AHEAD) * 2 + (wv >> 2)));
+            const int grow = FP4  ? (kt + AHEAD) * 4 + (wv >> 1)
+                             : Q4 ? scale_row((uint32_t)(kt + AHEAD))
+                                  : scale_row((uint32_t)((kt + AHEAD) * 2 + (wv >> 2)));
             if (s_lane) lds_load16_at(rs, here(s_at) + ST * (PAIR_SC_UNITS * 16), lane16, grow * (P.N * 2) + cs);
         }
     };
@@ -802,6 +835,13 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
     const int unit = (d >> 2) ^ (4 * (q & 1));
     // row of the x stage this lane's fragment row i comes from (STACK2: see above)
     const int xrow = STACK2 ? (((i >> 3) == (q >> 1)) ? (i & 7) : 8 + (i & 7)) : i;
+    // LDS unit (within a stage) of this lane's 8 k of tile row `row`
+    auto x_unit = [&](int row) {
+        if constexpr (Q4)
+            return a_lds_unit32(row, q);
+        else
+            return a_lds_unit<64>(row, 4 * h + q);
+    };
 
     // The accumulators are zeroed by asm so that the compiler cannot re-materialize the zeros
     // right in front of the first MFMA that accumulates into them: a VALU write of an MFMA's
@@ -855,7 +895,7 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
         asm volatile("v_readfirstlane_b32 %1, %4\n\ts_cmp_ge_u32 %1, %3\n\ts_cbranch_scc1 2f\n"
                      "1:\n\tv_mov_b32 %0, %2\n\ts_nop 0\n\tds_read_b32 %0, %0\n\ts_waitcnt lgkmcnt(0)\n\tv_readfirstlane_b32 %1, %0\n\ts_cmp_ge_u32 %1, %3\n\t"
                      "s_cbranch_scc1 2f\n\ts_sleep 1\n\ts_branch 1b\n2:"
-                     : "=&v"(seen_v), "=&s"(seen_s) : "s"(arrivals_at), "s"(8u * steps), "v"(early) : "memory", "scc");
+                     : "=&v"(seen_v), "=&s"(seen_s) : "s"(arrivals_at), "s"((uint32_t)NW * steps), "v"(early) : "memory", "scc");
     };
     if constexpr (KC) {
         // the scale loads the groups below do not cover (older than all of them: landed by the first barrier)
@@ -986,7 +1026,7 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
                 }
                 // first x fragments of the MFMA phase, read under the rest of the decode
 #pragma unroll
-                for (int f = 0; f < R; ++f) afr[f & 3] = la[a_lds_unit<BK>(16 * f + xrow, 4 * h + q)];
+                for (int f = 0; f < R; ++f) afr[f & 3] = la[x_unit(16 * f + xrow)];
             }
             if constexpr (KC) {
                 // dword r[t] = 8 consecutive k of MFMA t's weight row: byte p = the k pair p
@@ -1148,7 +1188,7 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
         // replaces stage kt-1) and the packed dwords of the next step (stage kt+1) are fetched between the MFMAs.
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
-            if (mt + R < MT) afr[(mt + R) & 3] = la[a_lds_unit<BK>(16 * (mt + R) + xrow, 4 * h + q)];
+            if (mt + R < MT) afr[(mt + R) & 3] = la[x_unit(16 * (mt + R) + xrow)];
             if constexpr (EXACT) {
                 const f32x4_t zero = {0.f, 0.f, 0.f, 0.f};
                 if constexpr (STACK2) {
@@ -1239,7 +1279,7 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
 #pragma unroll
             for (int e = 0; e < 4; ++e) acc[0][t][e] += __shfl_xor(acc[0][t][e], 32);
     }
-    pair_finish<MT, KC>(P, smem, acc, h, cw, lane, col0, row0, rows, n0, tk);
+    pair_finish<MT, KC, Q4>(P, smem, acc, h, cw, lane, col0, row0, rows, n0, tk);
 }
 
 // ---------------------------------------------------------------------------------
@@ -1263,16 +1303,16 @@ __device__ __forceinline__ void expert_chunks(int m, int& chunks, int& bpc) {
 
 template <int FMT, int KIND>
 struct KernelCfg {
-    static constexpr bool PAIR = KIND == GK_PAIR || KIND == GK_PAIR_SMALL || pair_exact(KIND);
+    static constexpr bool PAIR = KIND == GK_PAIR || KIND == GK_PAIR_SMALL || KIND == GK_QUAD || pair_exact(KIND);
     static constexpr bool SKINNY = KIND == GK_SKINNY;
     static_assert(!PAIR || FMT != MOE_FMT_BF16, "the k-split tile routine decodes quantized containers");
-    static constexpr int WAVES = PAIR ? 8 : 4;
+    static constexpr int WAVES = PAIR ? pair_waves(KIND) : 4;
     static constexpr int BN = GM_BN;                                             // columns per tile
     static constexpr int pair_wgs() {
         if constexpr (PAIR) return pair_wg_per_cu<FMT>(KIND); else return 1;
     }
     static constexpr int WG_PER_CU = SKINNY ? GM_SKINNY_WAVES : pair_wgs();
-    static constexpr int WAVES_PER_SIMD = WG_PER_CU * (PAIR ? 2 : 1);
+    static constexpr int WAVES_PER_SIMD = WG_PER_CU * WAVES / 4;
     static constexpr int CAPB = SKINNY ? GM_SKINNY_BLOCKS : PAIR ? PAIR_CAPB : GM_MT_MAX;
     static constexpr int fmt_mt_max() {
         if constexpr (PAIR)
@@ -1575,6 +1615,11 @@ static int launch_gemm_fmt(const moe_grouped_args* a, hipStream_t stream) {
         // 531 vs 549 us and 512 vs 609 us).  The one-byte containers gain nothing from it.
         if constexpr (FMT == MOE_FMT_INT4 || FMT == MOE_FMT_FP4_REF)
             if (a->M <= 12 * a->G) return launch_gemm_kind<FMT, GK_PAIR_SMALL>(P, a, stream);
+        // int4 and int8 prefill: workgroups of 4 wavefronts without the k split, two per CU
+        if constexpr (FMT == MOE_FMT_INT4 || FMT == MOE_FMT_INT8) {
+            const int rc = launch_gemm_kind<FMT, GK_QUAD>(P, a, stream);
+            if (rc != MOE_ERR_TOO_LARGE) return rc;   // (more experts than its half of the LDS holds a table for)
+        }
         return launch_gemm_kind<FMT, GK_PAIR>(P, a, stream);
     } else {
         // Decode-like batches (on average at most 24 rows per expert; group_list itself stays on the
