@@ -542,9 +542,10 @@ constexpr int pair_wg_per_cu(int kind) {
     if (!pair_small(kind)) return 1;
     return (FMT == MOE_FMT_INT4 || (FMT == MOE_FMT_FP4_REF && kind != GK_PAIR_EXACT)) ? 2 : 1;
 }
-// ring depth: what fits into LDS next to the 160-row x stages
+// ring depth: what fits into LDS next to the 160-row x stages; the 4-wavefront kind runs best with 4 stages (a tile's
+// first stages are filled sooner: int4 1790 against 1818 us at K = 7168, 949 against 952 us at K = 2048)
 template <int FMT>
-constexpr int pair_stages() { return (FMT == MOE_FMT_INT8 || FMT == MOE_FMT_FP8_REF) ? 4 : 5; }
+constexpr int pair_stages(int kind) { return (FMT == MOE_FMT_INT8 || FMT == MOE_FMT_FP8_REF || kind == GK_QUAD) ? 4 : 5; }
 // 16-byte units of scales per k step: rows of 256 bf16, int4 one per 32-k sub-step (groups are multiples
 // of 32), the reference fp4 container one per 16 k; fp8 one unit per wavefront holding the fp32 scale of
 // its 128 x 128 block; int8 none (per-channel scales stay in registers)
@@ -558,7 +559,7 @@ template <int FMT>
 constexpr int pair_kc_scale_units() { return (FMT == MOE_FMT_FP4_B32 || FMT == MOE_FMT_FP4_B16) ? 3 * 256 : 0; }
 template <int FMT>
 constexpr int pair_lds_units(int kind) {
-    return pair_stages<FMT>() * (pair_a_units(kind) + pair_b_units<FMT>(kind) + pair_sc_units<FMT>(kind)) + pair_kc_scale_units<FMT>();
+    return pair_stages<FMT>(kind) * (pair_a_units(kind) + pair_b_units<FMT>(kind) + pair_sc_units<FMT>(kind)) + pair_kc_scale_units<FMT>();
 }
 
 // End of a k-split tile.  The two wavefronts of a pair (same columns, the two k halves) hold partial sums of the
@@ -693,7 +694,7 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
     constexpr bool Q4 = KIND == GK_QUAD;
     static_assert(!Q4 || FMT == MOE_FMT_INT4 || FMT == MOE_FMT_INT8, "the 4-wavefront kind serves int4 and int8");
     constexpr int NW = pair_waves(KIND);
-    constexpr int BK = pair_bk(KIND), S = pair_stages<FMT>(), PAIR_SC_UNITS = pair_sc_units<FMT>(KIND);
+    constexpr int BK = pair_bk(KIND), S = pair_stages<FMT>(KIND), PAIR_SC_UNITS = pair_sc_units<FMT>(KIND);
     constexpr int PAIR_B_UNITS = pair_b_units<FMT>(KIND);
     constexpr int AHEAD = S - 1;   // a step's loads fill the stage of step kt + AHEAD
     // Kinds of which two workgroups share a CU (decode batches, HBM bound) keep one s_barrier per step, placed so
