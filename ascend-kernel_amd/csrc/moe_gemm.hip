@@ -514,7 +514,7 @@ __device__ __forceinline__ uint32_t here(uint32_t v) {
 //               64 columns through the whole k range in steps of 32 k, two workgroups per CU.  The two wavefronts
 //               of a SIMD belong to different workgroups and work on different tiles: no partial sums to
 //               exchange, a barrier spans 4 wavefronts instead of 8, and while one workgroup is between two tiles
-//               (stores, tile search, first loads) the other has the SIMDs to itself.  (int4 and int8.)
+//               (stores, tile search, first loads) the other has the SIMDs to itself.  (The N-contiguous containers.)
 enum { GK_GENERAL = 0, GK_SKINNY = 1, GK_PAIR = 2, GK_PAIR_EXACT = 3, GK_PAIR_SMALL = 4, GK_PAIR_EXACT16 = 5, GK_QUAD = 6 };
 constexpr bool pair_exact(int kind) { return kind == GK_PAIR_EXACT || kind == GK_PAIR_EXACT16; }
 constexpr int pair_waves(int kind) { return kind == GK_QUAD ? 4 : 8; }
@@ -692,7 +692,8 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
     constexpr bool B8 = I8 || F8;   // one byte per weight: tiles of 64 rows x 256 bytes
     // Q4: the kind without the k split (GK_QUAD): 4 wavefronts, steps of 32 k, every wavefront in every step
     constexpr bool Q4 = KIND == GK_QUAD;
-    static_assert(!Q4 || FMT == MOE_FMT_INT4 || FMT == MOE_FMT_INT8, "the 4-wavefront kind serves int4 and int8");
+    static_assert(!Q4 || FMT == MOE_FMT_INT4 || FMT == MOE_FMT_INT8 || FMT == MOE_FMT_FP4_REF || FMT == MOE_FMT_FP8_REF,
+                  "the 4-wavefront kind serves the N-contiguous containers");
     constexpr int NW = pair_waves(KIND);
     constexpr int BK = pair_bk(KIND), S = pair_stages<FMT>(KIND), PAIR_SC_UNITS = pair_sc_units<FMT>(KIND);
     constexpr int PAIR_B_UNITS = pair_b_units<FMT>(KIND);
@@ -769,8 +770,20 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
         ja[m] = j * 64;
         ca[m] = XROWS * j * P.K * 2;
     }
-    const int cb = KC ? n0 * (P.K >> 1) : B8 ? 8 * wv * P.N + n0 : 8 * wv * (P.N >> 1) + (n0 >> 1);
+    // (Q4 on the reference's fp4 container: the 32 k of a step are the rows [16 hp, +16) and [32 + 16 hp, +16) of the
+    // container's 64-row tile, hp = step & 1: wavefront wv brings the 8 rows from 32 (wv >> 1) + 16 hp + 8 (wv & 1) on)
+    const int cb = KC            ? n0 * (P.K >> 1)
+                   : B8          ? 8 * wv * P.N + n0
+                   : (Q4 && FP4) ? (32 * (wv >> 1) + 8 * (wv & 1)) * (P.N >> 1) + (n0 >> 1)
+                                 : 8 * wv * (P.N >> 1) + (n0 >> 1);
     const int kb_step = KC ? BK / 2 : B8 ? BK * P.N : BK * (P.N >> 1);
+    // byte offset of step kp's packed rows in the expert's slab
+    auto b_step_offset = [&](int kp) {
+        if constexpr (Q4 && FP4)
+            return ((kp >> 1) * 64 + (kp & 1) * 16) * (P.N >> 1);
+        else
+            return kp * kb_step;
+    };
     // K-contiguous fp4 scales.  Fetching the 4 or 8 bytes a weight row needs per step costs a request per
     // row and step (measured: 20 % of the kernel); instead 16 bytes of a row -- the scales of SUP steps --
     // are fetched at a time: the load slot of step kt brings, for step index kp = kt + KC_D, the rows
@@ -803,7 +816,7 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
         } else if (m < NA + NB) {
             const int e = m - NA;
             lds_load16_at(rw, here(b_at) + ST * (PAIR_B_UNITS * 16) + e * 1024, vb,
-                          cb + (B8 ? 4 * e * P.N : 0) + (kt + AHEAD) * kb_step);
+                          cb + (B8 ? 4 * e * P.N : 0) + b_step_offset(kt + AHEAD));
         } else if constexpr (KC) {
             kc_issue_scale(kt + KC_D);
         } else if constexpr (F8) {
@@ -811,9 +824,9 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
             if (lane == 0)
                 __builtin_amdgcn_raw_ptr_buffer_load_lds(
                     rs8, (__attribute__((address_space(3))) void*)(uintptr_t)(here(s_at) + ST * (PAIR_SC_UNITS * 16)), 4, 0,
-                    ((kt + AHEAD) >> 1) * (P.N >> 7) * 4 + cs8, 0, 0);
+                    ((kt + AHEAD) >> (Q4 ? 2 : 1)) * (P.N >> 7) * 4 + cs8, 0, 0);
         } else {
-            const int grow = FP4  ? (kt + AHEAD) * 4 + (wv >> 1)
+            const int grow = FP4  ? (kt + AHEAD) * (Q4 ? 2 : 4) + (wv >> 1)
                              : Q4 ? scale_row((uint32_t)(kt + AHEAD))
                                   : scale_row((uint32_t)((kt + AHEAD) * 2 + (wv >> 2)));
             if (s_lane) lds_load16_at(rs, here(s_at) + ST * (PAIR_SC_UNITS * 16), lane16, grow * (P.N * 2) + cs);
@@ -947,7 +960,9 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
             // 32 j + 8 i' + p holds, in its 32-byte run q', the 8 k rows 16 i' + 8 j + [0, 8) (one dword each)
             // of byte columns 16 p + 4 q' + [0, 4).  This lane's 8 k are 32 h + 8 q + [0, 8) and its two
             // bytes start at byte column 64 (cw >> 1) + 4 i + 2 (cw & 1): p = 4 (cw >> 1) + (i >> 2), q' = i & 3.
-            const int trow = 32 * (q & 1) + 8 * (2 * h + (q >> 1)) + 4 * (cw >> 1) + (i >> 2);
+            // (Q4: the stage holds the step's 32 rows of that tile packed together, see cb)
+            const int trow = Q4 ? 16 * (q & 1) + 8 * (q >> 1) + 4 * (cw >> 1) + (i >> 2)
+                                : 32 * (q & 1) + 8 * (2 * h + (q >> 1)) + 4 * (cw >> 1) + (i >> 2);
             const int swz = 4 * ((trow >> 3) & 1);   // the halves of the rows with odd (row >> 3) are swapped (see vb)
             const u32x4_t* tb = lds_b + st * PAIR_B_UNITS + trow * 8;
             const u32x4_t lo4 = tb[(2 * (i & 3)) ^ swz], hi4 = tb[(2 * (i & 3) + 1) ^ swz];
@@ -1616,8 +1631,11 @@ static int launch_gemm_fmt(const moe_grouped_args* a, hipStream_t stream) {
         // 531 vs 549 us and 512 vs 609 us).  The one-byte containers gain nothing from it.
         if constexpr (FMT == MOE_FMT_INT4 || FMT == MOE_FMT_FP4_REF)
             if (a->M <= 12 * a->G) return launch_gemm_kind<FMT, GK_PAIR_SMALL>(P, a, stream);
-        // int4 and int8 prefill: workgroups of 4 wavefronts without the k split, two per CU
-        if constexpr (FMT == MOE_FMT_INT4 || FMT == MOE_FMT_INT8) {
+        // prefill on the 4-bit N-contiguous containers: workgroups of 4 wavefronts without the k split, two per CU
+        // (256 experts of 128 rows, K = 7168, N = 4096: int4 1792 against 1905 us, fp4 1724 against 1867 us with the
+        // k-split kind; the one-byte containers, whose tiles move twice the bytes, are 2 % slower that way: int8 1081
+        // against 1058 us, fp8 1110 against 1081 us on 128 experts, and stay on the k-split kind)
+        if constexpr (FMT == MOE_FMT_INT4 || FMT == MOE_FMT_FP4_REF) {
             const int rc = launch_gemm_kind<FMT, GK_QUAD>(P, a, stream);
             if (rc != MOE_ERR_TOO_LARGE) return rc;   // (more experts than its half of the LDS holds a table for)
         }
