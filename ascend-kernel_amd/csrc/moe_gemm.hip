@@ -238,11 +238,13 @@ __device__ __forceinline__ int a_lds_unit(int row, int c) {
     return row * (BK / 8) + (c ^ (row & 7));
 }
 
-// The same for tile rows of 32 k (four 16-byte chunks, 64 bytes): chunk c of row r at position c ^ ((r >> 2) & 3),
-// so that the 16 rows x 1 chunk a quarter of a wavefront reads, and the 16 rows x 4 chunks an LDS-direct load
-// writes, each cover all banks once.
+// The same for tile rows of 32 k (four 16-byte chunks, 64 bytes): chunk c of row r at position c ^ ((r >> 1) & 3).
+// A 16-byte LDS read is served 8 lanes (128 bytes of banks) at a time: the 8 consecutive rows such a group reads the
+// same chunk of then lie in 8 different 16-byte slots modulo 128 bytes (two rows share a 128-byte line; the pairs
+// take the four positions in turn).  (With (r >> 2) & 3 in its place the counters showed two lanes per slot:
+// SQ_LDS_BANK_CONFLICT at 39 % of the cycles the LDS was active.)
 __device__ __forceinline__ int a_lds_unit32(int row, int c) {
-    return row * 4 + (c ^ ((row >> 2) & 3));
+    return row * 4 + (c ^ ((row >> 1) & 3));
 }
 
 // Per-tile context: lane coordinates and the buffer resources of expert g.
@@ -741,9 +743,9 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
     // zeros).  Load instruction j covers rows 8j + (lane >> 3); position lane & 7 of a row
     // holds chunk (lane & 7) ^ (row & 7), the swizzle a_lds_unit expects.
     // (Q4, rows of 64 bytes: instruction j covers rows 16j + (lane >> 2); position lane & 3 of a row holds
-    // chunk (lane & 3) ^ ((row >> 2) & 3), see a_lds_unit32)
+    // chunk (lane & 3) ^ ((row >> 1) & 3), see a_lds_unit32)
     const rsrc_t rx = make_rsrc(P.x + row0 * (int64_t)P.K, (int64_t)rows * P.K * 2);
-    const int va = Q4 ? ((lane >> 2) * P.K + (((lane & 3) ^ ((lane >> 4) & 3)) * 8)) * 2
+    const int va = Q4 ? ((lane >> 2) * P.K + (((lane & 3) ^ ((lane >> 3) & 3)) * 8)) * 2
                       : ((lane >> 3) * P.K + (((lane & 7) ^ (lane >> 3)) * 8)) * 2;
     // packed tile: instruction wv brings rows 8 wv + (lane >> 3) into the 1 KB block wv of the stage;
     // the two 64-byte halves of the rows with odd (row >> 3) are swapped, so that the four q groups
