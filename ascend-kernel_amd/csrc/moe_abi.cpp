@@ -120,7 +120,6 @@ int moe_grouped_gemm_validate(const moe_grouped_args* a) {
     // (grouped_gemm/op_host/grouped_matmul_antiquant_tiling.cpp:616-621), its last tile may be half empty
     const int rc = validate_grouped(a, fp4_k ? 128 : 64, a && a->format == MOE_FMT_FP8_REF ? 128 : 256, true);
     if (rc != MOE_OK) return rc;
-    // the GEMM kernels keep G + 1 tile counts in LDS next to their tile buffers
     return a->G > MOE_GEMM_MAX_EXPERTS ? MOE_ERR_TOO_LARGE : MOE_OK;
 }
 
@@ -131,10 +130,8 @@ int moe_grouped_gemv_validate(const moe_grouped_args* a) {
     const bool k_major = a && (a->format == MOE_FMT_BF16 || a->format == MOE_FMT_FP4_B32 || a->format == MOE_FMT_FP4_B16);
     const int rc = validate_grouped(a, k_major ? 32 : 64, k_major ? 1 : a && a->format == MOE_FMT_FP8_REF ? 128 : 256, false);
     if (rc != MOE_OK) return rc;
-    // experts are the y dimension of the GEMV grids; an fp8 N that is not a multiple of 256 needs the matrix-core
-    // kernel, which keeps G + 1 tile counts in LDS
-    if (a->G > 65535) return MOE_ERR_TOO_LARGE;
-    if (a->format == MOE_FMT_FP8_REF && a->N % 256 && a->G > MOE_GEMM_MAX_EXPERTS) return MOE_ERR_TOO_LARGE;
+    // experts are the y dimension of the GEMV grids
+    if (a->G > MOE_GEMM_MAX_EXPERTS) return MOE_ERR_TOO_LARGE;
     return MOE_OK;
 }
 

@@ -52,7 +52,10 @@ struct GemmParams {
     int epilogue;   // moe_epilogue
     int slot;       // this launch's counters in tile_queue; -1: none, every tile in the fixed order
     unsigned epoch; // stamp of this launch's counters
-    int rows_in_lds;   // the scheduler keeps the experts' clamped row bounds in LDS (they fit next to the tile table)
+    // what the scheduler keeps in LDS: 2 the first tile of every expert and the experts' clamped row bounds; 1 the
+    // first tiles only (the row bounds are read from group_list per tile); 0 neither fits: the first tile of every
+    // thread's run of experts only, and a tile is found by walking its run (any number of experts)
+    int table_mode;
     uint32_t sub_per_group;   // 32-k sub-steps per scale group of the N-contiguous 4-bit containers ...
     uint32_t sub_to_group;    // ... and the multiplier that turns a sub-step index into its scale row (0: identity)
 };
@@ -1368,7 +1371,8 @@ __global__ __launch_bounds__((64 * KernelCfg<FMT, KIND>::WAVES), (KernelCfg<FMT,
     extern __shared__ u32x4_t smem[];
     constexpr int THREADS = 64 * WAVES;
     constexpr int MTM = C::MTM;
-    int* prefix = reinterpret_cast<int*>(smem + C::lds_units());      // [G + 1] first tile of every expert
+    // [G + 1] first tile of every expert; table_mode 0: [THREADS + 1] first tile of every thread's run of experts
+    int* prefix = reinterpret_cast<int*>(smem + C::lds_units());
     // [G + 1] row bounds: rowc[g] = group_list[g - 1] clamped to [0, M] (rowc[0] = 0); expert g owns the rows
     // [rowc[g], rowc[g + 1]) if that is not empty (same result as clamping start and end separately).  Kept in
     // LDS so that the scheduler does not wait for a global load per tile (2 to 4 us under a streaming kernel).
@@ -1379,7 +1383,7 @@ __global__ __launch_bounds__((64 * KernelCfg<FMT, KIND>::WAVES), (KernelCfg<FMT,
     auto clamp_row = [&](int64_t v) { return (int)min(max(v, (int64_t)0), P.M); };
     auto expert_rows = [&](int g, int& first) {
         int hi;
-        if (P.rows_in_lds) {
+        if (P.table_mode == 2) {
             first = rowc[g];
             hi = rowc[g + 1];
         } else {
@@ -1390,10 +1394,11 @@ __global__ __launch_bounds__((64 * KernelCfg<FMT, KIND>::WAVES), (KernelCfg<FMT,
     };
 
     // exclusive scan of tiles per expert: each thread takes a contiguous run of experts
+    const int per = (P.G + THREADS - 1) / THREADS;
+    const int entries = P.table_mode ? P.G : THREADS;   // the table has entries + 1 elements
     {
-        const int per = (P.G + THREADS - 1) / THREADS;
-        const int g0 = tid * per, g1 = min(P.G, g0 + per);
-        if (P.rows_in_lds) {
+        const int g0 = min(P.G, tid * per), g1 = min(P.G, g0 + per);
+        if (P.table_mode == 2) {
             for (int g = g0; g < g1; ++g) rowc[g + 1] = clamp_row(P.gl[g]);
             if (tid == 0) rowc[0] = 0;
             __syncthreads();
@@ -1422,17 +1427,21 @@ __global__ __launch_bounds__((64 * KernelCfg<FMT, KIND>::WAVES), (KernelCfg<FMT,
             before += w < wave ? v : 0;
             all += v;
         }
-        if (tid == 0) prefix[P.G] = all;
+        if (tid == 0) prefix[entries] = all;
         int run = before + incl - sum;
-        for (int g = g0; g < g1; ++g) {
-            int first, chunks, bpc;
-            expert_chunks<MTM>(expert_rows(g, first), chunks, bpc);
-            prefix[g] = run;
-            run += chunks * ntile_n;
+        if (P.table_mode) {
+            for (int g = g0; g < g1; ++g) {
+                int first, chunks, bpc;
+                expert_chunks<MTM>(expert_rows(g, first), chunks, bpc);
+                prefix[g] = run;
+                run += chunks * ntile_n;
+            }
+        } else {
+            prefix[tid] = run;
         }
         __syncthreads();
     }
-    const int total = __builtin_amdgcn_readfirstlane(prefix[P.G]);
+    const int total = __builtin_amdgcn_readfirstlane(prefix[entries]);
 
     // XCD-aware order: workgroup b runs on XCD b % 8; give each XCD a contiguous run of
     // tiles in every sweep so that its workgroups share x rows in its own L2.
@@ -1477,24 +1486,62 @@ __global__ __launch_bounds__((64 * KernelCfg<FMT, KIND>::WAVES), (KernelCfg<FMT,
         const bool take = C::PAIR && queued && sw + 1 >= fixed_sweeps;
         const Ticket tk = {take ? q_slot + xcd : nullptr, part, part + 2};
         have_ticket = take;
-        // largest g with prefix[g] <= T (empty experts have prefix[g] == prefix[g+1]): every wavefront looks at 64
+        // largest e with prefix[e] <= T (empty experts have prefix[e] == prefix[e+1]): every wavefront looks at 64
         // evenly spaced entries at once, then at the entries between two of them -- two LDS round trips
         // instead of the ten of a binary search
         const int lane64 = tid & 63;
-        const int stride = (P.G + 63) >> 6;                      // entries per lane of the first step
-        const int probe = min(lane64 * stride, P.G);
-        const unsigned long long le1 = __ballot(prefix[probe] <= T && lane64 * stride <= P.G);
+        const int stride = (entries + 63) >> 6;                  // entries per lane of the first step
+        const int probe = min(lane64 * stride, entries);
+        const unsigned long long le1 = __ballot(prefix[probe] <= T && lane64 * stride <= entries);
         const int seg = 63 - __builtin_clzll(le1 | 1ull);        // last lane whose entry is <= T (lane 0: prefix[0] = 0)
-        const int idx2 = seg * stride + lane64;
-        const unsigned long long le2 = __ballot(lane64 < stride && idx2 < P.G && prefix[idx2] <= T);
+        // (the entries <= T of a segment are its first ones: count them, 64 at a time; one pass up to 4096 entries)
+        int upto = 0;
+        for (int o = 0; o < stride; o += 64) {
+            const int idx2 = seg * stride + o + lane64;
+            const int n_le = __popcll(__ballot(o + lane64 < stride && idx2 < entries && prefix[idx2] <= T));
+            upto += n_le;
+            if (n_le < 64) break;
+        }
         // everything below is wave-uniform; readfirstlane lets the compiler keep it in SGPRs
-        const int g = __builtin_amdgcn_readfirstlane(seg * stride + 63 - __builtin_clzll(le2 | 1ull));
+        const int found = __builtin_amdgcn_readfirstlane(seg * stride + max(upto, 1) - 1);
+        int g = found, local = __builtin_amdgcn_readfirstlane(T - prefix[found]);
+        if (P.table_mode == 0) {
+            // found is a thread's run of experts: walk it 64 experts at a time (group_list from memory, the tile
+            // counts summed across the wavefront) up to the expert that holds tile number `local` of the run
+            const int e_end = min(P.G, (found + 1) * per);
+            g = -1;
+            for (int e0 = found * per, base = 0; e0 < e_end && g < 0; e0 += 64) {
+                const int ge = e0 + lane64;
+                int tiles = 0;
+                if (ge < e_end) {
+                    int first, ch, bp;
+                    expert_chunks<MTM>(expert_rows(ge, first), ch, bp);
+                    tiles = ch * ntile_n;
+                }
+                int incl = tiles;
+#pragma unroll
+                for (int off = 1; off < 64; off <<= 1) {
+                    const int up = __shfl_up(incl, off, 64);
+                    if (lane64 >= off) incl += up;
+                }
+                const unsigned long long hit = __ballot(base + incl > local);
+                if (hit) {
+                    const int l = __ffsll(hit) - 1;
+                    g = e0 + l;
+                    local -= base + __shfl(incl - tiles, l, 64);
+                } else {
+                    base += __shfl(incl, 63, 64);
+                }
+            }
+            g = __builtin_amdgcn_readfirstlane(g);
+            local = __builtin_amdgcn_readfirstlane(local);
+            if (g < 0) break;   // cannot happen: the run holds the tile
+        }
         int gfirst;
         const int m = __builtin_amdgcn_readfirstlane(expert_rows(g, gfirst));
         const int64_t gbeg = gfirst;
         int chunks, bpc;
         expert_chunks<MTM>(m, chunks, bpc);
-        const int local = __builtin_amdgcn_readfirstlane(T - prefix[g]);
         // row chunks innermost: the tiles that share a weight column tile are neighbours in the order, run at
         // the same time on one XCD and pull that slice of the expert's weights into its L2 once
         const int nt = chunks == 1 ? local : local / chunks, chunk = chunks == 1 ? 0 : local % chunks;
@@ -1565,9 +1612,12 @@ static int launch_gemm_kind(const GemmParams& P, const moe_grouped_args* a, hipS
     using C = KernelCfg<FMT, KIND>;
     const size_t lds_max = (160 * 1024 - 2048) / C::WG_PER_CU;
     const size_t table = ((size_t)a->G + 1) * sizeof(int);
-    // tile table, and the row bounds next to it where they fit (else the scheduler reads group_list per tile)
-    const bool rows_in_lds = (size_t)C::lds_units() * 16 + 2 * table <= lds_max;
-    const size_t lds = (size_t)C::lds_units() * 16 + (rows_in_lds ? 2 : 1) * table;
+    // tile table, and the row bounds next to it where they fit; else the scheduler reads group_list per tile; else,
+    // with more experts than LDS holds a table for, it keeps one entry per thread and walks group_list (see
+    // GemmParams::table_mode)
+    const size_t units = (size_t)C::lds_units() * 16;
+    const int table_mode = units + 2 * table <= lds_max ? 2 : units + table <= lds_max ? 1 : 0;
+    const size_t lds = units + (table_mode ? table_mode * table : (size_t)(64 * C::WAVES + 1) * sizeof(int));
     if (lds > lds_max) return MOE_ERR_TOO_LARGE;
     static std::atomic<uint64_t> lds_set{0};
     if (const int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(&grouped_gemm_kernel<FMT, KIND>), (int)lds_max, lds_set))
@@ -1597,7 +1647,7 @@ static int launch_gemm_kind(const GemmParams& P, const moe_grouped_args* a, hipS
         Q.slot = -1;
         Q.epoch = 0;
     }
-    Q.rows_in_lds = rows_in_lds ? 1 : 0;
+    Q.table_mode = table_mode;
     hipLaunchKernelGGL((grouped_gemm_kernel<FMT, KIND>), dim3((unsigned)grid), dim3(64 * C::WAVES), lds, stream, Q);
     return hipGetLastError() == hipSuccess ? MOE_OK : MOE_ERR_LAUNCH;
 }
@@ -1614,7 +1664,7 @@ static GemmParams gemm_params(const moe_grouped_args* a) {
     P.epilogue = a->epilogue;
     P.slot = -1;
     P.epoch = 0;
-    P.rows_in_lds = 0;
+    P.table_mode = 0;
     const uint32_t per = a->scale_rows > 0 ? (uint32_t)((a->K / a->scale_rows) >> 5) : 1u;
     P.sub_per_group = per ? per : 1u;
     P.sub_to_group = P.sub_per_group == 1 ? 0u : 0xffffffffu / P.sub_per_group + 1u;

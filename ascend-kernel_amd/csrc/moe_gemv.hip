@@ -1,10 +1,16 @@
-// Grouped GEMV for MoE decode on gfx950 (few rows per expert).  HBM bound: every
-// weight byte of an expert that owns at least one row is read exactly once per
-// group of 4 rows; experts without rows cost one group_list read.  No MFMA: wide
-// vector loads, packed-bf16 dot products, wavefront shuffles for the reductions.
-// Replaces grouped_soft_gemv (grouped_soft_gemv/op_kernel/grouped_soft_gemv.h:235-293,
-// gemv_impl.h:201-398).  Unlike the reference, more than 4 rows per expert are
-// accepted: rows are taken 4 at a time.
+// Grouped GEMV for MoE decode on gfx950 (few rows per expert).  HBM bound: every weight byte of an expert
+// that owns at least one row is read exactly once per pass over its rows; experts without rows cost one
+// group_list read.  Replaces grouped_soft_gemv (grouped_soft_gemv/op_kernel/grouped_soft_gemv.h:235-293,
+// gemv_impl.h:201-398).  Unlike the reference, more than 4 rows per expert are accepted.
+//
+// Two kernels live here, both for the K-contiguous containers:
+//   gemv_kmajor_kernel    bf16 weights (and fp4 with K % 512 != 0): no matrix cores -- wide vector loads, packed-bf16
+//                         dot products (v_dot2c_f32_bf16), wavefront shuffles for the reductions, 4 rows per pass
+//   gemv_fp4_mfma_kernel  fp4 codes: one v_mfma_f32_16x16x32_bf16 per 32-k block and 16 weight rows (a vector kernel
+//                         needs (1 + rows) / 2 instructions per 4-bit weight, more than the chip can issue while HBM
+//                         delivers the codes at full rate), wave-private streaming, no workgroup barrier in the k loop
+// The N-contiguous containers (reference fp4 / fp8, int4) run on the k-split matrix-core kernel of moe_gemm.hip with
+// this op's arithmetic (launch_gemm_exact): measured 3 times faster than a vector kernel on that layout.
 //
 // Numerics (gemv_impl.h:147-199): weights are decode * scale in fp32, NOT rounded
 // to bf16; fp32 accumulation; one RNE to bf16 at the end (grouped_soft_gemv.h:218-233).
@@ -189,210 +195,6 @@ __global__ __launch_bounds__(256) void gemv_kmajor_kernel(const uint16_t* __rest
             case 2: gemv_kmajor_rows<FMT, 2>(wg, sg, x, y, xs, row0, n0, N, K); break;
             case 3: gemv_kmajor_rows<FMT, 3>(wg, sg, x, y, xs, row0, n0, N, K); break;
             default: gemv_kmajor_rows<FMT, 4>(wg, sg, x, y, xs, row0, n0, N, K); break;
-        }
-    }
-}
-
-// ---------------------------------------------------------------------------------
-// N-contiguous containers: the reference's "fp4" (pre-shuffled) and "fp8" layouts and
-// plain int4.  A workgroup owns 256 columns of one expert; K is split across the
-// lanes of a wavefront and across the 4 wavefronts (split-K), each thread keeping
-// fp32 accumulators for the columns its 16-byte loads cover; partial sums are
-// combined with wavefront shuffles, then across wavefronts through LDS.
-// ---------------------------------------------------------------------------------
-template <int FMT>
-struct NMajor;
-template <>
-struct NMajor<MOE_FMT_FP8_REF> {
-    static constexpr int NC = 16;      // columns per 16-byte load
-    static constexpr int KSTEP = 16;   // k rows covered by the workgroup per step
-    static constexpr int SHUF_LO = 16; // lane bits >= this select the k slice
-};
-template <>
-struct NMajor<MOE_FMT_INT4> {
-    static constexpr int NC = 32;
-    static constexpr int KSTEP = 32;
-    static constexpr int SHUF_LO = 8;
-};
-template <>
-struct NMajor<MOE_FMT_FP4_REF> {
-    static constexpr int NC = 8;       // 8 columns x 4 k per 16-byte load
-    static constexpr int KSTEP = 64;   // one 64(k) x 128(byte) tile per step
-    static constexpr int SHUF_LO = 0;  // lane bit 0 selects the k half
-};
-
-template <int FMT, int MG>
-__device__ __forceinline__ void gemv_nmajor_rows(const uint8_t* __restrict__ wg, const void* __restrict__ sgv,
-                                                 const uint16_t* __restrict__ x, uint16_t* __restrict__ y,
-                                                 uint16_t* xs, float* red, int64_t row0, int n0, int N, int K,
-                                                 int scale_rows) {
-    using T = NMajor<FMT>;
-    constexpr int NC = T::NC;
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-
-    __syncthreads();
-    for (int i = tid; i < MG * (K / 8); i += 256) {
-        const int r = i / (K / 8), k8 = i % (K / 8);
-        reinterpret_cast<u32x4_t*>(xs)[r * (K / 8) + k8] =
-            *reinterpret_cast<const u32x4_t*>(x + (row0 + r) * (int64_t)K + k8 * 8);
-    }
-    __syncthreads();
-
-    float acc[MG][NC];
-#pragma unroll
-    for (int r = 0; r < MG; ++r)
-#pragma unroll
-        for (int c = 0; c < NC; ++c) acc[r][c] = 0.f;
-
-    int ncol0;  // first column (relative to n0) of this thread's accumulators
-    if (FMT == MOE_FMT_FP8_REF) {
-        const int cn = tid & 15, kk = tid >> 4;
-        ncol0 = cn * 16;
-        const float* sg = static_cast<const float*>(sgv);
-        const int sn = N / 128;
-        for (int k = kk; k < K; k += 16) {
-            const u32x4_t wv = __builtin_nontemporal_load(
-                reinterpret_cast<const u32x4_t*>(wg + (int64_t)k * N + n0 + ncol0));
-            const float s = sg[(k >> 7) * sn + ((n0 + ncol0) >> 7)];
-            float xr[MG];
-#pragma unroll
-            for (int r = 0; r < MG; ++r) xr[r] = bf16_bits_to_f32(xs[r * K + k]);
-            // two codes at a time (see e4m3_ref_pair_over_256)
-            const float s256 = s * 256.f;
-#pragma unroll
-            for (int c = 0; c < 16; c += 2) {
-                const uint32_t sel = (uint32_t)(c & 3) | 0x0c00u | ((uint32_t)((c & 3) + 1) << 16) | 0x0c000000u;
-                const f32x2_t v = e4m3_ref_pair_over_256(__builtin_amdgcn_perm(0u, wv[c >> 2], sel));
-                const float w0 = v[0] * s256, w1 = v[1] * s256;
-#pragma unroll
-                for (int r = 0; r < MG; ++r) {
-                    acc[r][c] = fmaf(xr[r], w0, acc[r][c]);
-                    acc[r][c + 1] = fmaf(xr[r], w1, acc[r][c + 1]);
-                }
-            }
-        }
-    } else if (FMT == MOE_FMT_INT4) {
-        const int cn = tid & 7, kk = tid >> 3;
-        ncol0 = cn * 32;
-        const uint16_t* sg = static_cast<const uint16_t*>(sgv);
-        const int gs = K / scale_rows;
-        for (int k = kk; k < K; k += 32) {
-            const u32x4_t wv = __builtin_nontemporal_load(
-                reinterpret_cast<const u32x4_t*>(wg + (int64_t)k * (N / 2) + (n0 + ncol0) / 2));
-            const uint16_t* sp = sg + (int64_t)(k / gs) * N + n0 + ncol0;
-            float xr[MG];
-#pragma unroll
-            for (int r = 0; r < MG; ++r) xr[r] = bf16_bits_to_f32(xs[r * K + k]);
-#pragma unroll
-            for (int c8 = 0; c8 < 4; ++c8) {
-                const u32x4_t sv = *reinterpret_cast<const u32x4_t*>(sp + c8 * 8);
-#pragma unroll
-                for (int c = 0; c < 8; ++c) {
-                    const int q = (int)((wv[c8] >> (4 * c)) & 15u) - 8;
-                    const uint32_t sb = sv[c >> 1];
-                    const float wf = (float)q * ((c & 1) ? bf16_hi(sb) : bf16_lo(sb));
-#pragma unroll
-                    for (int r = 0; r < MG; ++r) acc[r][c8 * 8 + c] = fmaf(xr[r], wf, acc[r][c8 * 8 + c]);
-                }
-            }
-        }
-    } else {  // MOE_FMT_FP4_REF
-        // Destination row R = j<<5 | i<<3 | p of tile (a, t) holds k = 64a + 16i + 8j + [0,8)
-        // and n = 256t + 32p + [0,32); its 16-byte unit u holds k offsets 4(u&1) + [0,4)
-        // (one dword each) for the 8 columns 8(u>>1) + [0,8).
-        const int u = tid & 7, rs = tid >> 3;  // rs in [0,32): R = rs + 32*jj
-        const int p = rs & 7, i = rs >> 3, q = u >> 1, h = u & 1;
-        ncol0 = 32 * p + 8 * q;
-        const uint16_t* sg = static_cast<const uint16_t*>(sgv);
-        const int64_t nb = N / 2;
-        for (int a = 0; a < K / 64; ++a) {
-#pragma unroll
-            for (int jj = 0; jj < 2; ++jj) {
-                const int R = rs + 32 * jj;
-                const u32x4_t wv = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(
-                    wg + (int64_t)(a * 64 + R) * nb + (n0 / 2) + 16 * u));
-                const int kbase = 64 * a + 16 * i + 8 * jj + 4 * h;
-                const u32x4_t sv = *reinterpret_cast<const u32x4_t*>(sg + (int64_t)(kbase >> 4) * N + n0 + ncol0);
-#pragma unroll
-                for (int d = 0; d < 4; ++d) {
-                    float xr[MG];
-#pragma unroll
-                    for (int r = 0; r < MG; ++r) xr[r] = bf16_bits_to_f32(xs[r * K + kbase + d]);
-                    const f32x2_t v0 = e2m1_pair_to_f32<0>(wv[d]), v1 = e2m1_pair_to_f32<1>(wv[d]);
-                    const f32x2_t v2 = e2m1_pair_to_f32<2>(wv[d]), v3 = e2m1_pair_to_f32<3>(wv[d]);
-                    const float wf[8] = {v0[0] * bf16_lo(sv[0]), v0[1] * bf16_hi(sv[0]), v1[0] * bf16_lo(sv[1]),
-                                         v1[1] * bf16_hi(sv[1]), v2[0] * bf16_lo(sv[2]), v2[1] * bf16_hi(sv[2]),
-                                         v3[0] * bf16_lo(sv[3]), v3[1] * bf16_hi(sv[3])};
-#pragma unroll
-                    for (int c = 0; c < 8; ++c)
-#pragma unroll
-                        for (int r = 0; r < MG; ++r) acc[r][c] = fmaf(xr[r], wf[c], acc[r][c]);
-                }
-            }
-        }
-    }
-
-    // combine the k slices held by different lanes, then by different wavefronts
-#pragma unroll
-    for (int r = 0; r < MG; ++r)
-#pragma unroll
-        for (int c = 0; c < NC; ++c) {
-            float v = acc[r][c];
-            if (FMT == MOE_FMT_FP4_REF) {
-                v += __shfl_xor(v, 1, 64);
-            } else {
-#pragma unroll
-                for (int off = 32; off >= T::SHUF_LO; off >>= 1) v += __shfl_xor(v, off, 64);
-            }
-            acc[r][c] = v;
-        }
-    const bool writer = FMT == MOE_FMT_FP4_REF ? ((lane & 1) == 0) : (lane < T::SHUF_LO);
-    const int wcol0 = FMT == MOE_FMT_FP4_REF ? 32 * (lane >> 3) + 8 * ((lane & 7) >> 1) : ncol0;
-    if (writer) {
-#pragma unroll
-        for (int r = 0; r < MG; ++r)
-#pragma unroll
-            for (int c = 0; c < NC; ++c) red[(wave * GV_ROWS + r) * 256 + wcol0 + c] = acc[r][c];
-    }
-    __syncthreads();
-    // FP4_REF: the 4 wavefronts hold different i (k), the same columns; others: different kk
-#pragma unroll
-    for (int r = 0; r < MG; ++r) {
-        const float v = red[(0 * GV_ROWS + r) * 256 + tid] + red[(1 * GV_ROWS + r) * 256 + tid] +
-                        red[(2 * GV_ROWS + r) * 256 + tid] + red[(3 * GV_ROWS + r) * 256 + tid];
-        y[(row0 + r) * (int64_t)N + n0 + tid] = (uint16_t)(pack_bf16_rne(v, 0.f) & 0xffffu);
-    }
-}
-
-template <int FMT>
-__global__ __launch_bounds__(256) void gemv_nmajor_kernel(const uint16_t* __restrict__ x,
-                                                          const uint8_t* __restrict__ w,
-                                                          const void* __restrict__ scale,
-                                                          const int64_t* __restrict__ gl, uint16_t* __restrict__ y,
-                                                          int64_t M, int K, int N, int scale_rows) {
-    extern __shared__ u32x4_t smem[];
-    float* red = reinterpret_cast<float*>(smem);                       // [4 waves][4 rows][256]
-    uint16_t* xs = reinterpret_cast<uint16_t*>(red + 4 * GV_ROWS * 256);  // [4 rows][K]
-    const int g = blockIdx.y, n0 = blockIdx.x * 256;
-    int64_t start, end;
-    group_rows(gl, g, M, start, end);
-    if (end <= start) return;
-    const uint8_t* wg;
-    const void* sg;
-    if (FMT == MOE_FMT_FP8_REF) {
-        wg = w + (int64_t)g * K * N;
-        sg = static_cast<const float*>(scale) + (int64_t)g * (K / 128) * (N / 128);
-    } else {
-        wg = w + (int64_t)g * K * (N / 2);
-        sg = static_cast<const uint16_t*>(scale) + (int64_t)g * scale_rows * N;
-    }
-    for (int64_t row0 = start; row0 < end; row0 += GV_ROWS) {
-        const int mg = (int)min((int64_t)GV_ROWS, end - row0);
-        switch (mg) {
-            case 1: gemv_nmajor_rows<FMT, 1>(wg, sg, x, y, xs, red, row0, n0, N, K, scale_rows); break;
-            case 2: gemv_nmajor_rows<FMT, 2>(wg, sg, x, y, xs, red, row0, n0, N, K, scale_rows); break;
-            case 3: gemv_nmajor_rows<FMT, 3>(wg, sg, x, y, xs, red, row0, n0, N, K, scale_rows); break;
-            default: gemv_nmajor_rows<FMT, 4>(wg, sg, x, y, xs, red, row0, n0, N, K, scale_rows); break;
         }
     }
 }
@@ -711,20 +513,6 @@ static int launch_kmajor(const moe_grouped_args* a, hipStream_t stream) {
     return hipGetLastError() == hipSuccess ? MOE_OK : MOE_ERR_LAUNCH;
 }
 
-template <int FMT>
-static int launch_nmajor(const moe_grouped_args* a, hipStream_t stream) {
-    const size_t lds = (size_t)4 * GV_ROWS * 256 * 4 + (size_t)GV_ROWS * a->K * 2;
-    if (lds > 160 * 1024) return MOE_ERR_TOO_LARGE;
-    static std::atomic<uint64_t> lds_set{0};
-    if (const int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(&gemv_nmajor_kernel<FMT>), 160 * 1024, lds_set)) return rc;
-    dim3 grid((unsigned)(a->N / 256), (unsigned)a->G);
-    hipLaunchKernelGGL((gemv_nmajor_kernel<FMT>), grid, dim3(256), lds, stream,
-                       static_cast<const uint16_t*>(a->x), static_cast<const uint8_t*>(a->weight), a->scale,
-                       a->group_list, static_cast<uint16_t*>(a->y), a->M, (int)a->K, (int)a->N,
-                       (int)a->scale_rows);
-    return hipGetLastError() == hipSuccess ? MOE_OK : MOE_ERR_LAUNCH;
-}
-
 bool gemv_preferred(const moe_grouped_args* a) {
     // Decode-sized batches on the K-contiguous containers are pure weight streaming: these kernels
     // read every weight row as contiguous runs.  The bf16 vector kernel takes 4 rows of an expert per
@@ -751,13 +539,8 @@ int launch_grouped_gemv(const moe_grouped_args* a, hipStream_t stream, bool gemm
         case MOE_FMT_FP4_REF:
         case MOE_FMT_INT4:
         case MOE_FMT_FP8_REF: {
-            // the matrix-core GEMM kernels run with this op's arithmetic (fp32 weights); the vector kernel
-            // only where the expert count does not fit those kernels' tile table in LDS
-            const int rc = launch_gemm_exact(a, stream);
-            if (rc != MOE_ERR_TOO_LARGE) return rc;
-            return a->format == MOE_FMT_INT4      ? launch_nmajor<MOE_FMT_INT4>(a, stream)
-                   : a->format == MOE_FMT_FP4_REF ? launch_nmajor<MOE_FMT_FP4_REF>(a, stream)
-                                                  : launch_nmajor<MOE_FMT_FP8_REF>(a, stream);
+            // the matrix-core GEMM kernels run with this op's arithmetic (fp32 weights)
+            return launch_gemm_exact(a, stream);
         }
         default: return MOE_ERR_BAD_FORMAT;
     }

@@ -51,8 +51,10 @@ extern "C" {
 /* hipStream_t, passed opaquely so that this header needs no HIP include. */
 typedef void *moe_stream_t;
 
-/* moe_grouped_gemm keeps a table of G + 1 tile counts in LDS next to its tile buffers. */
-#define MOE_GEMM_MAX_EXPERTS 1024
+/* Experts per call of either grouped op.  (moe_grouped_gemm keeps a table of G + 1 tile counts in LDS next to its
+ * tile buffers while that fits -- about 1000 to 2000 experts, depending on the container -- and beyond that one
+ * entry per thread, walking group_list for the rest: any count works, small ones are faster.) */
+#define MOE_GEMM_MAX_EXPERTS 65535
 
 typedef enum moe_status {
     MOE_OK = 0,
@@ -65,8 +67,7 @@ typedef enum moe_status {
                                     grouped_matmul_antiquant_tiling.cpp:260-264); one
                                     expert's weight or scale slab of 2 GiB or more, or
                                     K or N of 4194304 or more (32-bit byte offsets);
-                                    more experts than MOE_GEMM_MAX_EXPERTS (grouped
-                                    GEMM) or 65535 (grouped GEMV)                     */
+                                    more than MOE_GEMM_MAX_EXPERTS (65535) experts    */
     MOE_ERR_LAUNCH = -6,         /* hipLaunchKernel reported an error                 */
     MOE_ERR_NO_DEVICE = -7       /* no gfx950 device / wrong architecture             */
 } moe_status;

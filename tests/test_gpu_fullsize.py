@@ -1,5 +1,6 @@
 """The benchmark configurations at their full sizes on the GPU.  The oracle checks a sample
-(whole experts, so that every tile shape of those experts is covered); size-independent
+(whole experts, so that every tile shape of those experts is covered, and a few rows of many
+more experts spread over the list, so that every part of the tile order is); size-independent
 properties cover the rest: exact linearity in x, determinism, untouched trailing rows, and
 agreement between the fused and the separate FP4 paths."""
 import numpy as np
@@ -58,6 +59,34 @@ def _oracle_subset(fmt, x, w, s, o, counts, experts, gemv=False):
     return rows, ref
 
 
+def _oracle_rows(fmt, x, w, s, o, counts, picks, gemv=False):
+    """Oracle output for a few rows of many experts: picks maps an expert to row offsets within it.  A reduced
+    problem (those experts, those rows) built from the device tensors; returns (row indices into the full
+    problem, bf16 bits [rows, N])."""
+    starts = torch.cumsum(counts, 0) - counts
+    experts = sorted(picks)
+    rows = torch.tensor([int(starts[g]) + r for g in experts for r in picks[g]])
+    gl_sub = np.cumsum([len(picks[g]) for g in experts]).astype(np.int64)
+    xb = H.bits(x[rows.cuda()])
+    cpu = lambda t: None if t is None else t[torch.tensor(experts).cuda()].cpu()
+    as_np = lambda t: None if t is None else (H.bits(t) if t.dtype == torch.bfloat16 else t.numpy())
+    ref = oracle.grouped_gemm(oracle.FMT_BY_NAME[fmt], xb, as_np(cpu(w)), as_np(cpu(s)), as_np(cpu(o)), gl_sub,
+                              round_bf16=not gemv)
+    return rows, ref
+
+
+def _spread_picks(counts, n_experts, rng):
+    """First row, last row and one row in between of n_experts experts spread evenly over the list (so that tiles
+    of every part of the tile order, fixed sweeps and work-counter tail alike, are sampled)."""
+    G = counts.shape[0]
+    picks = {}
+    for g in np.linspace(0, G - 1, n_experts).round().astype(int):
+        m = int(counts[g])
+        if m > 0:
+            picks[int(g)] = sorted({0, m - 1, int(rng.integers(0, m))})
+    return picks
+
+
 def test_dsv3_int4_prefill_gate_up_and_down():
     _say("full size: DSV3 int4 prefill")
     gen = torch.Generator().manual_seed(0)
@@ -79,6 +108,10 @@ def test_dsv3_int4_prefill_gate_up_and_down():
         assert torch.isnan(y[M:]).all() and not torch.isnan(y[:M]).any()
         rows, ref = _oracle_subset("int4", x, w, s, None, counts, experts)
         H.assert_close(H.bits(y[rows.cuda()]), ref, what=f"int4 {name}")
+        # and a few rows of 40 more experts spread over the whole list
+        picks = _spread_picks(counts, 40, np.random.default_rng(K))
+        rows, ref = _oracle_rows("int4", x, w, s, None, counts, picks)
+        H.assert_close(H.bits(y[rows.cuda()]), ref, what=f"int4 {name}, rows of {len(picks)} experts")
         # determinism and exact linearity: y(2x) == 2 y(x) bit for bit (scaling by 2 is exact)
         y2 = torch.empty_like(y)
         _launch("gemm", "int4", x, w, s, None, gl, y2, K // 128)
@@ -102,6 +135,10 @@ def test_int8_grouped_gemm_8_experts():
     _launch("gemm", "int8", x, w, s, o, gl, y)
     rows, ref = _oracle_subset("int8", x, w, s, o, counts, [int(torch.argmin(counts))])
     H.assert_close(H.bits(y[rows.cuda()]), ref, what="int8")
+    # rows of every expert: first, last, and some of every 128-row chunk in between
+    picks = {g: sorted({0, int(counts[g]) - 1, *range(5, int(counts[g]), 61)}) for g in range(G)}
+    rows, ref = _oracle_rows("int8", x, w, s, o, counts, picks)
+    H.assert_close(H.bits(y[rows.cuda()]), ref, what="int8, rows of all experts")
 
 
 def test_grouped_gemv_64_experts_bf16():

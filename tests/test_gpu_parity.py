@@ -394,18 +394,32 @@ def test_gemv_n_contiguous_row_counts_up_to_and_beyond_32(fmt, K, N, group):
     assert (got[gl[-1]:] == 0x7FC0).all()
 
 
-@pytest.mark.parametrize("fmt", ["fp4", "int4", "fp8"])
-def test_gemv_n_contiguous_more_experts_than_the_matrix_core_kernel_takes(fmt):
-    """The k-split kernel keeps a tile table of G + 1 entries in LDS; beyond its capacity the GEMV op
-    falls back to the vector kernel."""
-    _say(f"gemv {fmt} G=2100")
-    G = 2100
-    rng = np.random.default_rng(11)
-    counts = rng.integers(0, 3, G)
+@pytest.mark.parametrize("fmt,op,G,style", [
+    ("int4", "gemv", 2100, "decode"), ("fp4", "gemv", 2100, "decode"), ("fp8", "gemv", 2100, "decode"),
+    ("int4", "gemm", 2100, "decode"), ("int4", "gemm", 2100, "prefill"),
+    # beyond what LDS holds a table for (about 3000 experts next to the small stages, 2700 / 5000 next to the large)
+    ("int4", "gemv", 6000, "decode"), ("int4", "gemm", 6000, "decode"), ("fp8", "gemv", 6000, "decode"),
+    ("int4", "gemm", 6000, "prefill"), ("fp4", "gemm", 6000, "prefill"), ("int8", "gemm", 6000, "prefill"),
+    ("fp4_b32", "gemm", 6000, "prefill"), ("bf16", "gemm", 12000, "decode")])
+def test_any_number_of_experts(fmt, op, G, style):
+    """The grouped GEMM kernels keep the first tile of every expert in LDS while that fits; with more experts (the
+    reference loops over any number, grouped_gemm/op_kernel/grouped_matmul_antiquant.h:241-242) they keep one entry
+    per thread and walk group_list from there.  Empty experts, experts of several row chunks and rows past
+    group_list[-1] included."""
+    _say(f"{op} {fmt} G={G} {style}")
+    rng = np.random.default_rng(G)
+    if style == "decode":
+        counts = rng.integers(0, 3, G)
+        counts[[3, G // 2, G - 2]] = [5, 9, 4]
+    else:
+        counts = rng.integers(0, 30, G)                      # on average more than 12 rows per expert
+        counts[[3, G // 2, G - 2]] = [170, 400, 33]
     gl = list(np.cumsum(counts))
-    case = H.make_case(fmt, G, 128, 256, gl, seed=12, group=32 if fmt == "int4" else 128 if fmt == "fp8" else 16)
-    got = H.run_cabi(case, H.upload(case), "gemv")
-    H.assert_close(got, H.oracle_out(case, gemv=True), what=f"gemv {fmt} G={G}")
+    K, N = (64, 256) if fmt == "bf16" else (128, 256)
+    case = H.make_case(fmt, G, K, N, gl, seed=12, group=32 if fmt == "int4" else 128 if fmt == "fp8" else 16, extra_rows=3)
+    got = H.run_cabi(case, H.upload(case), op)
+    H.assert_close(got, H.oracle_out(case, gemv=op == "gemv"), rows=slice(0, gl[-1]), what=f"{op} {fmt} G={G}")
+    assert (got[gl[-1]:] == 0x7FC0).all()
 
 
 def test_gemv_reference_fp8_test_shape_via_module():

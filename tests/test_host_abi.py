@@ -67,9 +67,10 @@ def test_grouped_validate_accepts_good_and_rejects_bad(op):
     assert val(ctypes.byref(gargs(0, M=-1))) == mg.ERR_BAD_SHAPE
     assert val(ctypes.byref(gargs(0, G=0))) == mg.ERR_BAD_SHAPE
     assert val(ctypes.byref(gargs(0, K=1 << 31, scale_rows=(1 << 31) // 16))) == mg.ERR_TOO_LARGE  # reference limit
-    # the grouped GEMM keeps a tile table of G + 1 entries in LDS; the GEMV op falls back to a kernel without one
-    assert val(ctypes.byref(gargs(0, G=1024))) == mg.MOE_OK
-    assert val(ctypes.byref(gargs(0, G=1025))) == (mg.ERR_TOO_LARGE if op == "gemm" else mg.MOE_OK)
+    # any expert count up to 65535 (beyond what LDS holds a tile table for, the kernels walk group_list instead)
+    assert val(ctypes.byref(gargs(0, G=1025))) == mg.MOE_OK
+    assert val(ctypes.byref(gargs(0, G=65535))) == mg.MOE_OK
+    assert val(ctypes.byref(gargs(0, G=65536))) == mg.ERR_TOO_LARGE
     assert val(ctypes.byref(gargs(0, weight=None))) == mg.ERR_NULL_POINTER
     assert val(ctypes.byref(gargs(0, group_list=None))) == mg.ERR_NULL_POINTER
     assert val(ctypes.byref(gargs(0, scale=None))) == mg.ERR_NULL_POINTER
@@ -114,9 +115,7 @@ def test_fp8_accepts_n_multiple_of_128(op):
     assert val(ctypes.byref(gargs(1, N=1408))) == mg.MOE_OK
     assert val(ctypes.byref(gargs(1, N=320))) == mg.ERR_BAD_ALIGNMENT
     assert val(ctypes.byref(gargs(3, N=384))) == mg.ERR_BAD_ALIGNMENT      # the other N-contiguous containers: 256
-    if op == "gemv":   # beyond the tile table of the matrix-core kernel only whole 256-column tiles
-        assert val(ctypes.byref(gargs(1, N=384, G=1025))) == mg.ERR_TOO_LARGE
-        assert val(ctypes.byref(gargs(1, N=512, G=1025))) == mg.MOE_OK
+    assert val(ctypes.byref(gargs(1, N=384, G=1025))) == mg.MOE_OK
 
 
 def test_route_static_limit_is_checked_on_the_host():
