@@ -219,7 +219,9 @@ __global__ __launch_bounds__(256) void gemv_kmajor_kernel(const uint16_t* __rest
 // that way, each 64-byte piece of a scale row is fetched from HBM several times.  Instead the
 // 4 q lanes of a row read 128 contiguous bytes of it once per 4 loop iterations (lane q: the
 // 16 scales of iteration 4 T + q) and the iteration's scales are picked up from the lane that
-// holds them with ds_bpermute.
+// holds them through a wavefront's own 2 KB of LDS (written once per 4 iterations, read with 16-byte loads that
+// the 4 q lanes share: ds_bpermute, which this replaced, serves 4 lanes that ask for one lane's register one after
+// the other -- the counters showed it as bank conflicts in 39 % of the LDS cycles).
 //
 // x (<= 16 rows of a chunk of K) is staged in LDS; the 16-byte units of row r are XOR-swizzled
 // with r so that the fragment reads of the 16 lanes of a q group fall into different banks.
@@ -227,7 +229,8 @@ __global__ __launch_bounds__(256) void gemv_kmajor_kernel(const uint16_t* __rest
 constexpr int GF_WAVES = 8;               // wavefronts per workgroup
 constexpr int GF_NR_WG = 16 * GF_WAVES;   // weight rows per workgroup
 constexpr int GF_ROWS = 16;               // activation rows per pass
-constexpr int GF_LDS_UNITS = 4096;        // 64 KiB of x per staged chunk
+constexpr int GF_LDS_UNITS = 3584;        // 56 KiB of x per staged chunk
+constexpr int GF_SCALE_UNITS = 128;       // per wavefront: the 4 q lanes' 2 x 16 bytes of scales for 16 rows
 constexpr int GF_U = 4;                   // 128-k groups (one 16-byte load per lane each) per loop iteration
 constexpr int GF_KSTEP = 128 * GF_U;      // k per loop iteration; K must be a multiple
 constexpr int GF_GEMM_ROWS_PER_EXPERT = 12;// grouped GEMM calls with at most this many rows per expert on average come here
@@ -257,11 +260,13 @@ template <int MB, bool ROUNDW, int BLK>
 __device__ __forceinline__ void gemv_fp4_mfma_rows(const uint8_t* __restrict__ wg, const uint16_t* __restrict__ sg,
                                                    const uint16_t* __restrict__ x, uint16_t* __restrict__ y,
                                                    u32x4_t* xs, int64_t row0, int mg, int n0, int N, int K) {
-    constexpr int KC = GF_LDS_UNITS / MB * 8;   // k per staged chunk: 8192, 4096 or 2048
+    constexpr int KC = GF_LDS_UNITS / MB * 8 / GF_KSTEP * GF_KSTEP;   // k per staged chunk: 7168, 3584 or 1536
     constexpr int RS = KC / 8;                  // row stride in 16-byte units
     constexpr int U = GF_U;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int i = lane & 15, q = lane >> 4;
+    // this wavefront's scale exchange: unit (2 q' + e) * 16 + i holds register e of lane (i, q')
+    u32x4_t* ss = xs + GF_LDS_UNITS + wave * GF_SCALE_UNITS;
     const int n = n0 + wave * 16 + i;
     const int nn = min(n, N - 1);
     // 32-bit byte offsets from the expert's (wavefront-uniform) base pointers: an expert's weight
@@ -411,24 +416,25 @@ __device__ __forceinline__ void gemv_fp4_mfma_rows(const uint8_t* __restrict__ w
         auto iteration = [&](const u32x4_t (&w)[U], int it) {
             const int t = it & (PER - 1);
             if (t == 0) {
-                sc[0] = sn[0];
-                sc[1] = sn[1];
+                // (a wavefront's LDS accesses complete in order: the reads of the previous scales are done)
+                ss[(2 * q) * 16 + i] = sn[0];
+                ss[(2 * q + 1) * 16 + i] = sn[1];
                 if (it + PER < niter) fetch_s(sn, it / PER + 1);
             }
 #pragma unroll
             for (int u = 0; u < U; ++u) {
                 if constexpr (BLK == 32) {
-                    // this iteration's scales live in lane (i, t): 2 dwords per group
-                    const int src = (16 * t + i) * 4;
-                    const uint32_t sd[2] = {(uint32_t)__builtin_amdgcn_ds_bpermute(src, (int)sc[u >> 1][2 * (u & 1)]),
-                                            (uint32_t)__builtin_amdgcn_ds_bpermute(src, (int)sc[u >> 1][2 * (u & 1) + 1])};
+                    // this iteration's scales are those of lane (i, t): 2 dwords per group
+                    if (u == 0) {
+                        sc[0] = ss[(2 * t) * 16 + i];
+                        sc[1] = ss[(2 * t + 1) * 16 + i];
+                    }
+                    const uint32_t sd[2] = {sc[u >> 1][2 * (u & 1)], sc[u >> 1][2 * (u & 1) + 1]};
                     group(w[u], sd, it * U + u);
                 } else {
-                    // groups 0, 1 of the iteration live in lane (i, 2 t), groups 2, 3 in lane (i, 2 t + 1): 4 dwords each
-                    const int src = (16 * (2 * t + (u >> 1)) + i) * 4;
-                    uint32_t sd[4];
-#pragma unroll
-                    for (int d = 0; d < 4; ++d) sd[d] = (uint32_t)__builtin_amdgcn_ds_bpermute(src, (int)sc[u & 1][d]);
+                    // groups 0, 1 of the iteration are with lane (i, 2 t), groups 2, 3 with lane (i, 2 t + 1): 4 dwords each
+                    const u32x4_t sv = ss[(2 * (2 * t + (u >> 1)) + (u & 1)) * 16 + i];
+                    const uint32_t sd[4] = {sv[0], sv[1], sv[2], sv[3]};
                     group(w[u], sd, it * U + u);
                 }
             }
@@ -493,7 +499,10 @@ __global__ __launch_bounds__(64 * GF_WAVES, 4) void gemv_fp4_mfma_kernel(const u
 template <bool ROUNDW, int BLK>
 static int launch_fp4_mfma(const moe_grouped_args* a, hipStream_t stream) {
     dim3 grid((unsigned)((a->N + GF_NR_WG - 1) / GF_NR_WG), (unsigned)a->G);
-    hipLaunchKernelGGL((gemv_fp4_mfma_kernel<ROUNDW, BLK>), grid, dim3(64 * GF_WAVES), (size_t)GF_LDS_UNITS * 16, stream,
+    constexpr size_t lds = (size_t)(GF_LDS_UNITS + GF_WAVES * GF_SCALE_UNITS) * 16;   // 72 KB: two workgroups per CU
+    static std::atomic<uint64_t> lds_set{0};
+    if (const int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(&gemv_fp4_mfma_kernel<ROUNDW, BLK>), (int)lds, lds_set)) return rc;
+    hipLaunchKernelGGL((gemv_fp4_mfma_kernel<ROUNDW, BLK>), grid, dim3(64 * GF_WAVES), lds, stream,
                        static_cast<const uint16_t*>(a->x), static_cast<const uint8_t*>(a->weight),
                        static_cast<const uint16_t*>(a->scale), a->group_list, static_cast<uint16_t*>(a->y), a->M,
                        (int)a->K, (int)a->N);
