@@ -761,7 +761,6 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
     const int kc_n = 32 * wv + (lane >> 1);
     const int vb = KC   ? kc_n * (P.K >> 1) + 16 * ((lane & 1) ^ ((kc_n >> 3) & 1))
                    : B8 ? (lane >> 4) * P.N + (((lane & 15) ^ (4 * (wv & 3))) * 16)
-                   : FP4 ? (lane >> 3) * (P.N >> 1) + (((lane & 7) ^ (4 * (wv & 1)) ^ ((lane >> 3) & 1)) * 16)
                         : (lane >> 3) * (P.N >> 1) + (((lane & 7) ^ (4 * (wv & 1))) * 16);
     constexpr int XI = Q4 ? MT : 2 * MT;          // x load instructions per step (1 KB each: 16 or 8 rows)
     constexpr int XROWS = Q4 ? 16 : 8;
@@ -969,9 +968,7 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
             // (Q4: the stage holds the step's 32 rows of that tile packed together, see cb)
             const int trow = Q4 ? 16 * (q & 1) + 8 * (q >> 1) + 4 * (cw >> 1) + (i >> 2)
                                 : 32 * (q & 1) + 8 * (2 * h + (q >> 1)) + 4 * (cw >> 1) + (i >> 2);
-            // the halves of the rows with odd (row >> 3) are swapped, and neighbouring units of the odd rows (see vb):
-            // the 8 lanes a 16-byte LDS read serves at a time (2 rows x units 0, 2, 4, 6) then hit 8 different slots
-            const int swz = (4 * ((trow >> 3) & 1)) ^ (trow & 1);
+            const int swz = 4 * ((trow >> 3) & 1);   // the halves of the rows with odd (row >> 3) are swapped (see vb)
             const u32x4_t* tb = lds_b + st * PAIR_B_UNITS + trow * 8;
             const u32x4_t lo4 = tb[(2 * (i & 3)) ^ swz], hi4 = tb[(2 * (i & 3) + 1) ^ swz];
 #pragma unroll

@@ -287,7 +287,9 @@ __device__ __forceinline__ void gemv_fp4_mfma_rows(const uint8_t* __restrict__ w
         const uint8_t* wp = wg + (kc0 >> 1);                                   // group c of the chunk: + 64 c bytes
         const uint8_t* sp = reinterpret_cast<const uint8_t*>(sg) + (kc0 / BLK) * 2;  // scale b of the chunk: + 2 b bytes
         // x fragment of block 4 c + j: unit (16 c + 4 j + q) ^ r of row r = xj[j][16 c].  MFMA rows
-        // >= MB read row i % MB again: their products land in accumulator rows that are not stored.
+        // >= MB read row i % MB again: their products land in accumulator rows that are not stored
+        // (lanes that read the same unit are served together: timed alone, this pattern reads as fast as
+        // 64 consecutive units, and sending the repeated rows to other units was slower).
         const int r = i % MB;
         const u32x4_t* xj[4];
 #pragma unroll
