@@ -224,4 +224,6 @@ int moe_grouped_gemv(const moe_grouped_args* a, moe_stream_t stream) {
     return moe::launch_grouped_gemv(a, static_cast<hipStream_t>(stream));
 }
 
+int64_t moe_test_shift_launch_number(int64_t delta) { return moe::gemm_shift_launch_number(delta); }
+
 }  // extern "C"

@@ -50,8 +50,8 @@ struct GemmParams {
     int64_t M;
     int K, N, G, scale_rows;
     int epilogue;   // moe_epilogue
-    int slot;       // this launch's counters in tile_queue; -1: none, every tile in the fixed order
-    unsigned epoch; // stamp of this launch's counters
+    int slot;       // this launch's counter in tile_queue; -1: none, every tile in the fixed order
+    unsigned long long stamp;   // what this launch raises its counter to before it draws from it
     // what the scheduler keeps in LDS: 2 the first tile of every expert and the experts' clamped row bounds; 1 the
     // first tiles only (the row bounds are read from group_list per tile); 0 neither fits: the first tile of every
     // thread's run of experts only, and a tile is found by walking its run (any number of experts)
@@ -64,71 +64,60 @@ struct GemmParams {
 // placed first runs about 1.5 times as fast as the other while both are resident, and the XCDs differ by a few
 // per cent), so an even split of the tiles leaves most of the chip waiting for the slowest workgroup.  All but
 // the last two or three tiles of a workgroup's share are handed out in a fixed, XCD-aware order; the rest
-// (the tail) are taken one at a time from counters in the library's device memory.
+// (the tail) are taken one at a time, front to back, from a counter in the library's device memory.  (One
+// counter per XCD, each for a run of its own or for every eighth chunk of the tail, and stealing between them
+// at the end, kept more of the tail's reads in the XCDs' L2s but was 1.5 - 2 % slower on the prefill shapes and
+// 5 % on the weight-streaming decode shapes.)
 //
-// The tail is cut into 8 contiguous runs, one per XCD, each with a counter of its own: the workgroups of an
-// XCD keep drawing neighbouring tiles (the same experts' x rows and weight slices in that XCD's L2) and only
-// when their run is used up take tiles from the XCD that has most left.
-//
-// A launch owns one slot of 8 counters.  The host numbers the launches; launch L uses slot L % GM_QUEUE_SLOTS
-// and stamps every counter it touches with its epoch (L / GM_QUEUE_SLOTS, never 0) in the upper bits: a counter
-// that carries another epoch is left over from an earlier launch and counts as zero, so nothing has to be
-// cleared at the end of a kernel and no state a kernel leaves behind can mislead a later one.  Two launches
-// share a slot only if GM_QUEUE_SLOTS launches after the first one it is still running.  A launch that is
-// being captured into a HIP graph gets no slot at all (slot -1): its kernel node would keep the slot for every
-// replay while the ring moves on, so it walks all of its tiles in the fixed order instead.
-constexpr int GM_QUEUE_SLOTS = 1024;
-constexpr int GM_QUEUE_TAIL_SWEEPS = 2;   // tiles per workgroup that are left to the counters (plus the remainder)
-constexpr unsigned GM_QUEUE_COUNT_BITS = 20, GM_QUEUE_COUNT_MASK = (1u << GM_QUEUE_COUNT_BITS) - 1u;
-constexpr unsigned GM_QUEUE_EPOCHS = (1u << (32 - GM_QUEUE_COUNT_BITS)) - 1u;   // epochs 1 .. GM_QUEUE_EPOCHS
-__device__ unsigned int tile_queue[GM_QUEUE_SLOTS * 8];
-static std::atomic<unsigned> queue_launches{0};   // launches of every kind of kernel in this file, for slot and epoch
+// A launch owns one slot = one 64-bit counter.  The host numbers the launches (64 bits, never reused); launch L
+// uses slot L % GM_QUEUE_SLOTS and the stamp (L / GM_QUEUE_SLOTS + 1) << GM_QUEUE_COUNT_BITS, which grows with
+// every use of the slot.  Every workgroup raises the counter to the stamp when it starts (atomic max, fire and
+// forget, long before its first draw); a draw is a fetch-and-add, and the value it returns minus the stamp is
+// the ticket.  Whatever an earlier launch left in the slot is smaller than the stamp and simply disappears, so
+// nothing has to be cleared at the end of a kernel and no state a kernel leaves behind can mislead a later one.
+// A launch that only starts after a later launch has taken its slot (its stream was held back for
+// GM_QUEUE_SLOTS launches) sees that from the counter, which it reads once behind its stamp, and never draws:
+// it walks all of its tiles in the fixed order and disturbs nobody.  A draw that returns a value outside
+// [stamp, stamp + 2^GM_QUEUE_COUNT_BITS) means that the slot was taken over while this launch was running: the
+// workgroup then walks its share of the tail in the fixed order -- tiles that were already handed out get
+// computed twice, which only rewrites the same values -- but its stray draws have cost the later launch
+// tickets, i.e. tiles: a launch that is still running when the GM_QUEUE_SLOTS-th launch after it starts is
+// the one thing callers must not arrange.  A launch that is being captured into a HIP graph gets no slot at
+// all (slot -1): its kernel node would keep slot and stamp for every replay while the ring moves on, so it
+// walks all of its tiles in the fixed order.
+constexpr int GM_QUEUE_SLOTS = 4096;
+constexpr int GM_QUEUE_STRIDE = 8;        // 64-bit words per slot: a cache line of its own
+constexpr int GM_QUEUE_TAIL_SWEEPS = 2;   // tiles per workgroup that are left to the counter (plus the remainder)
+constexpr unsigned GM_QUEUE_COUNT_BITS = 24;
+typedef unsigned long long queue_word_t;
+__device__ queue_word_t tile_queue[GM_QUEUE_SLOTS * GM_QUEUE_STRIDE];
+static std::atomic<uint64_t> queue_launches{0};   // launches of every kind of kernel in this file, for slot and stamp
 
-// The ticket a fetch-and-add on counter q returned (raw), for a launch of the given epoch: the count
-// before the add if the counter was this launch's already, else the counter is stamped first (compare-and-
-// swap, so that exactly one workgroup gets ticket 0 of a stale counter).  Every path ends after at most as
-// many rounds as there are workgroups.
-__device__ __forceinline__ unsigned queue_ticket(unsigned int* q, unsigned raw, unsigned epoch) {
-    if ((raw >> GM_QUEUE_COUNT_BITS) == epoch) return raw & GM_QUEUE_COUNT_MASK;
-    for (;;) {
-        const unsigned v = __hip_atomic_load(q, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        if ((v >> GM_QUEUE_COUNT_BITS) == epoch) return atomicAdd(q, 1u) & GM_QUEUE_COUNT_MASK;
-        if (atomicCAS(q, v, (epoch << GM_QUEUE_COUNT_BITS) | 1u) == v) return 0u;
-    }
+// Raises the counter to the launch's stamp and tells whether the slot is (still) this launch's.  The read is an
+// ordinary load behind the atomic, not the atomic's own return value: that came back 2.5 us later than the
+// group_list loads the caller waits for anyway.
+__device__ __forceinline__ bool queue_stamp(queue_word_t* q, queue_word_t stamp) {
+    (void)__hip_atomic_fetch_max(q, stamp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const queue_word_t now = __hip_atomic_load(q, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return now - stamp < (1ull << GM_QUEUE_COUNT_BITS);
 }
-// The tail [lo, lo + n) of a launch as the 8 runs of its XCDs
-struct TailRuns {
-    int lo, n;
-    __device__ __forceinline__ int first(int x) const { return lo + (int)(((int64_t)n * x) >> 3); }
-    __device__ __forceinline__ int size(int x) const { return first(x + 1) - first(x); }
-};
-// One thread resolves the workgroup's next tail tile from the raw value its fetch-and-add on the own XCD's
-// counter returned; -1 when the tail is used up.
-__device__ __forceinline__ int queue_resolve(unsigned int* slot, int xcd, unsigned raw, unsigned epoch, const TailRuns& tr) {
-    unsigned t = queue_ticket(slot + xcd, raw, epoch);
-    if ((int)t < tr.size(xcd)) return tr.first(xcd) + (int)t;
-    for (;;) {
-        // the XCD with most tiles left (the 8 loads are independent: one round trip)
-        unsigned v[8];
-#pragma unroll
-        for (int x = 0; x < 8; ++x) v[x] = __hip_atomic_load(slot + x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        int best = -1, left = 0;
-#pragma unroll
-        for (int x = 0; x < 8; ++x) {
-            const int used = (v[x] >> GM_QUEUE_COUNT_BITS) == epoch ? (int)(v[x] & GM_QUEUE_COUNT_MASK) : 0;
-            const int l = tr.size(x) - used;
-            if (l > left) { left = l; best = x; }
-        }
-        if (best < 0) return -1;
-        t = queue_ticket(slot + best, atomicAdd(slot + best, 1u), epoch);
-        if ((int)t < tr.size(best)) return tr.first(best) + (int)t;
-    }
+// A draw adds 1 to the counter's low word only (the count never carries out of it) and gets that word back: one
+// register in flight instead of two in the tile routines, which have none to spare.  The word still shows the
+// low 32 - GM_QUEUE_COUNT_BITS bits of the launch's use of the slot, enough to tell a slot that was taken over.
+__device__ __forceinline__ unsigned queue_draw_raw(queue_word_t* q) {
+    return __hip_atomic_fetch_add(reinterpret_cast<unsigned*>(q), 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
+// The ticket in a counter's low word raw, for a launch with the given stamp; -1: the slot is not this launch's
+__device__ __forceinline__ int queue_ticket_of_draw(unsigned raw, queue_word_t stamp) {
+    const unsigned d = raw - (unsigned)stamp;
+    return d < (1u << GM_QUEUE_COUNT_BITS) ? (int)d : -1;
+}
+__device__ __forceinline__ int queue_draw(queue_word_t* q, queue_word_t stamp) { return queue_ticket_of_draw(queue_draw_raw(q), stamp); }
 // A tile routine that is handed a counter draws the workgroup's next ticket from it while it finishes its own
 // tile (the counter's round trip, about 3 us under load, overlaps the tile's reduction and stores) and leaves
-// the raw value in *out behind its last barrier.
+// the ticket in *out behind its last barrier.
 struct Ticket {
-    unsigned int* counter;   // null: the caller draws the ticket itself
+    queue_word_t* counter;   // null: the caller draws the ticket itself
     int* out;
     int* arrivals;           // a word of LDS for the tile routine's arrival counter (see gemm_tile_pair)
 };
@@ -578,8 +567,8 @@ __device__ __forceinline__ void pair_finish(const GemmParams& P, u32x4_t* smem, 
                                             int col0, int64_t row0, int rows, int n0, const Ticket& tk) {
     const int i = lane & 15, q = lane >> 4;
     const bool takes = tk.counter != nullptr && threadIdx.x == 0;
-    unsigned int next_tile = 0;
-    if (takes) next_tile = atomicAdd(tk.counter, 1u);
+    unsigned next_tile = 0;
+    if (takes) next_tile = queue_draw_raw(tk.counter);
     constexpr int MH = (MT + 1) / 2, RR = MH < 4 ? MH : 4, ROUNDS = (MH + RR - 1) / RR;
     // the last tile of an N that is not a multiple of 256 (the reference's fp8 container: multiples of 128)
     // computes columns past N from whatever follows in the slab: they are not stored
@@ -665,7 +654,7 @@ __device__ __forceinline__ void pair_finish(const GemmParams& P, u32x4_t* smem, 
     } else {
         finish(std::integral_constant<int, 1>{});
     }
-    if (takes) *tk.out = (int)next_tile;
+    if (takes) *tk.out = queue_ticket_of_draw(next_tile, P.stamp);
     lds_barrier();   // the slots are read: the next tile may load into the ring (the stores are still in flight)
 }
 
@@ -1379,7 +1368,10 @@ __global__ __launch_bounds__((64 * KernelCfg<FMT, KIND>::WAVES), (KernelCfg<FMT,
     int* rowc = prefix + (P.G + 1);
     const int tid = threadIdx.x;
     const int ntile_n = (P.N + C::BN - 1) / C::BN;
-    __shared__ int part[THREADS];   // scan partials; part[0] later carries the tile taken from the queue
+    // scan partials (one per wavefront); later part[0] carries the ticket drawn from the queue, part[1] the tile
+    // resolved from it, part[2] the tile routine's arrival counter
+    __shared__ int part[THREADS];
+    constexpr int PART_FIXED = 16;   // first whether this workgroup uses the launch's counter, then its number of fixed sweeps
     auto clamp_row = [&](int64_t v) { return (int)min(max(v, (int64_t)0), P.M); };
     auto expert_rows = [&](int g, int& first) {
         int hi;
@@ -1392,6 +1384,9 @@ __global__ __launch_bounds__((64 * KernelCfg<FMT, KIND>::WAVES), (KernelCfg<FMT,
         }
         return max(hi - first, 0);
     };
+
+    // the launch's counter is raised to its stamp now, long before the first draw from it
+    if (tid == 0) part[PART_FIXED] = P.slot >= 0 && queue_stamp(tile_queue + GM_QUEUE_STRIDE * max(P.slot, 0), P.stamp);
 
     // exclusive scan of tiles per expert: each thread takes a contiguous run of experts
     const int per = (P.G + THREADS - 1) / THREADS;
@@ -1449,42 +1444,44 @@ __global__ __launch_bounds__((64 * KernelCfg<FMT, KIND>::WAVES), (KernelCfg<FMT,
     const int per_xcd = (nwg + 7) / 8;
     const int vid = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
     const int sweep = per_xcd * 8;   // == nwg: the grid is a multiple of 8
-    // a launch without counters (captured into a HIP graph) walks every tile in the fixed order
-    const bool queued = P.slot >= 0;
-    const int fixed_sweeps = queued ? max(0, total / sweep - GM_QUEUE_TAIL_SWEEPS) : (total + sweep - 1) / sweep;
-    const int xcd = blockIdx.x % 8;
-    unsigned int* q_slot = tile_queue + 8 * max(P.slot, 0);
-    const TailRuns tail = {fixed_sweeps * sweep, max(total - fixed_sweeps * sweep, 0)};
+    // The number of sweeps in the fixed order lives in LDS, not in a register that would stay live across the tile
+    // routines; GM_NO_QUEUE: a launch without counters (captured into a HIP graph, or one whose slot a later launch
+    // holds by now) walks every tile in the fixed order, sweep after sweep until the tile number passes the last.
+    constexpr int GM_NO_QUEUE = 0x7fffffff;
+    if (tid == 0) part[PART_FIXED] = part[PART_FIXED] ? max(0, total / sweep - GM_QUEUE_TAIL_SWEEPS) : GM_NO_QUEUE;
+    __syncthreads();
 
-    bool have_ticket = false;   // the previous tile routine left the raw ticket in part[0]
+    bool have_ticket = false;   // the previous tile routine left its ticket in part[0]
+    queue_word_t* const q_own = tile_queue + GM_QUEUE_STRIDE * max(P.slot, 0);
     for (int sw = 0;; ++sw) {
         int T;
-        if (sw < fixed_sweeps) {
-            T = sw * sweep + vid;
-            if (T >= total) break;
-        } else {
-            if (!queued) break;
+        int fixed = __builtin_amdgcn_readfirstlane(part[PART_FIXED]);
+        if (sw >= fixed) {
+            if (fixed == GM_NO_QUEUE) break;
             if (!have_ticket) {
-                __syncthreads();   // part[] of the previous round is read (the scan's part[], the first time)
-                if (tid == 0) part[0] = (int)atomicAdd(q_slot + xcd, 1u);
+                __syncthreads();   // part[] of the previous round is read
+                if (tid == 0) part[0] = queue_draw(q_own, P.stamp);
                 __syncthreads();
             }
-            // the usual case needs no second exchange: a ticket of this launch inside the XCD's own run
-            const unsigned raw = (unsigned)__builtin_amdgcn_readfirstlane(part[0]);
-            const int own = (int)(raw & GM_QUEUE_COUNT_MASK);
-            if ((raw >> GM_QUEUE_COUNT_BITS) == P.epoch && own < tail.size(xcd)) {
-                T = tail.first(xcd) + own;
+            const int own = __builtin_amdgcn_readfirstlane(part[0]);
+            if (own >= 0) {
+                T = fixed * sweep + own;
+                if (T >= total) break;
             } else {
-                __syncthreads();
-                if (tid == 0) part[1] = queue_resolve(q_slot, xcd, raw, P.epoch, tail);
-                __syncthreads();
-                T = __builtin_amdgcn_readfirstlane(part[1]);
-                if (T < 0) break;
+                // the slot belongs to a later launch: this workgroup's share of the tail in the fixed order
+                __syncthreads();   // everyone has read this round's part[PART_FIXED]
+                if (tid == 0) part[PART_FIXED] = GM_NO_QUEUE;
+                sw = fixed;
+                fixed = GM_NO_QUEUE;
             }
         }
+        if (sw < fixed) {
+            T = sw * sweep + vid;
+            if (T >= total) break;
+        }
         // from the last tile of the fixed order on, the k-split tile routines draw the next ticket themselves
-        const bool take = C::PAIR && queued && sw + 1 >= fixed_sweeps;
-        const Ticket tk = {take ? q_slot + xcd : nullptr, part, part + 2};
+        const bool take = C::PAIR && fixed != GM_NO_QUEUE && sw + 1 >= fixed;
+        const Ticket tk = {take ? q_own : nullptr, part, part + 2};
         have_ticket = take;
         // largest e with prefix[e] <= T (empty experts have prefix[e] == prefix[e+1]): every wavefront looks at 64
         // evenly spaced entries at once, then at the entries between two of them -- two LDS round trips
@@ -1594,6 +1591,10 @@ __global__ __launch_bounds__((64 * KernelCfg<FMT, KIND>::WAVES), (KernelCfg<FMT,
     }
 }
 
+int64_t gemm_shift_launch_number(int64_t delta) {
+    return (int64_t)(queue_launches.fetch_add((uint64_t)delta, std::memory_order_relaxed) + (uint64_t)delta);
+}
+
 // Compute units of the current device, looked up once per device.
 static int device_cu_count() {
     static std::atomic<int> cached[64];
@@ -1640,12 +1641,12 @@ static int launch_gemm_kind(const GemmParams& P, const moe_grouped_args* a, hipS
         capture = hipStreamCaptureStatusActive;
     }
     if (capture == hipStreamCaptureStatusNone) {
-        const unsigned launch = queue_launches.fetch_add(1, std::memory_order_relaxed);
+        const uint64_t launch = queue_launches.fetch_add(1, std::memory_order_relaxed);
         Q.slot = (int)(launch % GM_QUEUE_SLOTS);
-        Q.epoch = (launch / GM_QUEUE_SLOTS) % GM_QUEUE_EPOCHS + 1u;
+        Q.stamp = (launch / GM_QUEUE_SLOTS + 1) << GM_QUEUE_COUNT_BITS;
     } else {
         Q.slot = -1;
-        Q.epoch = 0;
+        Q.stamp = 0;
     }
     Q.table_mode = table_mode;
     hipLaunchKernelGGL((grouped_gemm_kernel<FMT, KIND>), dim3((unsigned)grid), dim3(64 * C::WAVES), lds, stream, Q);
@@ -1663,7 +1664,7 @@ static GemmParams gemm_params(const moe_grouped_args* a) {
     P.M = a->M; P.K = (int)a->K; P.N = (int)a->N; P.G = (int)a->G; P.scale_rows = (int)a->scale_rows;
     P.epilogue = a->epilogue;
     P.slot = -1;
-    P.epoch = 0;
+    P.stamp = 0;
     P.table_mode = 0;
     const uint32_t per = a->scale_rows > 0 ? (uint32_t)((a->K / a->scale_rows) >> 5) : 1u;
     P.sub_per_group = per ? per : 1u;

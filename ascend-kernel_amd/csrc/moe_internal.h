@@ -30,6 +30,8 @@ bool gemv_preferred(const moe_grouped_args* a);
 // op's arithmetic; MOE_ERR_TOO_LARGE when the expert count does not fit its LDS
 int launch_gemm_exact(const moe_grouped_args* a, hipStream_t stream);
 int launch_grouped_gemm(const moe_grouped_args* a, hipStream_t stream);
+// moves the grouped GEMM's launch number (which picks a launch's tile counter and stamp) by delta; returns the new number
+int64_t gemm_shift_launch_number(int64_t delta);
 int launch_prepack_fp4_ref(const moe_prepack_fp4_args* a, hipStream_t stream);
 int launch_route(const moe_route_args* a, hipStream_t stream);
 // the same with the workspace in the library's own static device array (a->workspace is ignored)

@@ -26,7 +26,7 @@ SYMBOLS = (
     "moe_dequant_fp4_bf16_workspace_bytes", "moe_grouped_gemm_workspace_bytes", "moe_grouped_gemv_workspace_bytes",
     "moe_dequant_fp4_bf16", "moe_grouped_gemm", "moe_grouped_gemv",
     "moe_prepack_fp4_ref_validate", "moe_prepack_fp4_ref_workspace_bytes", "moe_prepack_fp4_ref",
-    "moe_route_validate", "moe_route_workspace_bytes", "moe_route", "moe_route_static",
+    "moe_route_validate", "moe_route_workspace_bytes", "moe_route", "moe_route_static", "moe_test_shift_launch_number",
 )
 
 
@@ -79,6 +79,8 @@ for _n, _t in (("dequant_fp4_bf16", DequantArgs), ("grouped_gemm", GroupedArgs),
 
 
 lib.moe_route_static.restype = ctypes.c_int
+lib.moe_test_shift_launch_number.restype = ctypes.c_int64
+lib.moe_test_shift_launch_number.argtypes = [ctypes.c_int64]
 lib.moe_route_static.argtypes = [ctypes.POINTER(RouteArgs), ctypes.c_void_p]
 ROUTE_STATIC_SCRATCH_BYTES = 2 << 20
 

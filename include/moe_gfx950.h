@@ -7,13 +7,15 @@
  * device, never copies group_list to the host and allocates nothing.  The only
  * state between calls is set-up done once per process or GPU (a kernel attribute,
  * the CU count, the address of moe_route_static's scratch array) and the tile counters
- * of the grouped GEMM kernels: 32 KB of the library's own device memory, 1024 slots.
- * An eager launch takes the next slot and stamps it with its own epoch, so nothing a
- * kernel leaves in a slot can mislead a later one; launches may overlap on different
- * streams (two eager launches would share a slot only if one were still running 1024
- * launches after it was issued).  A launch made while its stream is being captured
- * into a HIP graph takes no slot and walks its tiles in a fixed order, so graphs may
- * be replayed any number of times, beside each other and beside eager launches.
+ * of the grouped GEMM kernels: 256 KB of the library's own device memory, 4096 slots of
+ * one counter.  An eager launch takes the next slot and raises its counter to a stamp
+ * that grows with every use of the slot, so nothing a kernel leaves in a slot can mislead
+ * a later one; launches may overlap on different streams.  The one arrangement to avoid:
+ * a launch that is still running when the 4096th grouped launch after it starts (that
+ * later launch may then miss tiles; a launch that merely starts that late notices and
+ * disturbs nobody).  A launch made while its stream is being captured into a HIP graph
+ * takes no slot and walks its tiles in a fixed order, so graphs may be replayed any
+ * number of times, beside each other and beside eager launches.
  * Calls are re-entrant except where moe_route_static says otherwise.  All functions
  * return MOE_OK (0) or a negative moe_status; nothing throws across this boundary.
  *
@@ -251,6 +253,11 @@ int moe_route(const moe_route_args *args, moe_stream_t stream);
  * time on the same GPU race on it -- keep them on one stream or otherwise ordered. */
 #define MOE_ROUTE_STATIC_SCRATCH_BYTES (2u << 20)
 int moe_route_static(const moe_route_args *args, moe_stream_t stream);
+
+/* Test support, no counterpart in the reference and no use in production: moves the library's count of
+ * grouped launches (which picks a launch's tile counter and stamp) by delta and returns the new count, so
+ * that a test can make a launch find its counter taken over by a later one. */
+int64_t moe_test_shift_launch_number(int64_t delta);
 
 #ifdef __cplusplus
 }

@@ -199,13 +199,16 @@ def test_decode_batches_on_the_small_tile_kinds(fmt, shape, op):
     assert (got[gl[-1]:] == 0x7FC0).all()
 
 
-def test_gemm_tile_queue_slots_are_reused_safely():
-    """The persistent grid takes its last tiles from counters in device memory; every launch uses one of 1024
-    slots and stamps it with its epoch, so whatever an earlier launch left in a slot counts as zero.  More
-    launches than slots, on two streams, with more tiles than workgroups: a launch misled by a slot's old
-    content would skip tiles (rows left unwritten)."""
+def test_gemm_tile_counters_are_reused_and_taken_over_safely():
+    """The persistent grid takes its last tiles from a counter in device memory; every launch uses one of 4096
+    slots and raises the counter to a stamp that grows with every use of the slot, so whatever an earlier launch
+    left there counts as nothing.  A launch misled by a slot's content would skip tiles (rows left unwritten).
+    The library's launch number is moved (test hook) so that (1) slots are used again with the next stamp,
+    (2) launches find their slot already stamped by a later launch and fall back to the fixed order, and (3) a
+    launch has its slot taken over while it runs: its own result must still be right."""
     import moe_gfx950 as mg
-    _say("gemm tile queue: 2300 launches")
+    slots = 4096
+    _say("gemm tile counters: reuse, late start, take-over")
     rng = np.random.default_rng(5)
     counts = rng.choice([0, 1, 3, 16, 17, 33], 40)
     gl = list(np.cumsum(counts))
@@ -219,17 +222,52 @@ def test_gemm_tile_queue_slots_are_reused_safely():
         ys.append(y)
         argss.append(mg.grouped_args(mg.format_from_compute_type(c["fmt"]), p(d["x"]), p(d["weight"]), p(d["scale"]),
                                      p(d["offset"]), p(d["group_list"]), p(y), c["M"], c["K"], c["N"], c["G"], c["scale_rows"]))
+
+    def check(what):
+        torch.cuda.synchronize()
+        for c, y in zip(cases, ys):
+            got = y.cpu().numpy().view(np.uint16)
+            H.assert_close(got, H.oracle_out(c), rows=slice(0, gl[-1]), what=f"{what} {c['fmt']}")
+            y.fill_(0x7FC0)
+        torch.cuda.synchronize()
+
+    def run(iters, what):
+        for it in range(iters):
+            for st, args in zip(streams, argss):
+                mg.grouped_gemm(args, st.cuda_stream)
+            if it in (0, iters - 1):
+                check(f"{what}, launch {it}")
+
     torch.cuda.synchronize()
-    for it in range(1150):
-        for st, args in zip(streams, argss):
-            mg.grouped_gemm(args, st.cuda_stream)
-        if it in (0, 600, 1149):
+    try:
+        run(300, "fresh slots")
+        mg.lib.moe_test_shift_launch_number(slots - 600)
+        run(300, "the same slots, next stamp")
+        mg.lib.moe_test_shift_launch_number(-slots)
+        run(20, "slots that a later launch has stamped")
+        mg.lib.moe_test_shift_launch_number(2 * slots)
+        run(2, "back to normal")
+        # (3): A runs on one stream; the launch number is moved so that B, on another stream, gets A's slot with
+        # the next stamp and starts as soon as A's first workgroups leave.  A's last draws then fail and its
+        # workgroups finish their share in the fixed order.  Only A's result is defined.
+        big = H.make_case("int4", 48, 1024, 2048, [128 * (g + 1) for g in range(48)], seed=3, group=128)
+        dev = H.upload(big)
+        ya = torch.full((big["M"], big["N"]), 0x7FC0, dtype=torch.int16, device="cuda")
+        yb = torch.empty_like(ya)
+        mk = lambda y: mg.grouped_args(mg.format_from_compute_type("int4"), p(dev["x"]), p(dev["weight"]), p(dev["scale"]), p(dev["offset"]),
+                                       p(dev["group_list"]), p(y), big["M"], big["K"], big["N"], big["G"], big["scale_rows"])
+        a_args, b_args = mk(ya), mk(yb)
+        torch.cuda.synchronize()
+        for rep in range(3):
+            mg.grouped_gemm(a_args, streams[0].cuda_stream)
+            mg.lib.moe_test_shift_launch_number(slots - 1)
+            mg.grouped_gemm(b_args, streams[1].cuda_stream)
             torch.cuda.synchronize()
-            for c, y in zip(cases, ys):
-                got = y.cpu().numpy().view(np.uint16)
-                H.assert_close(got, H.oracle_out(c), rows=slice(0, gl[-1]), what=f"launch {it} {c['fmt']}")
-                y.fill_(0x7FC0)
+            H.assert_close(ya.cpu().numpy().view(np.uint16), H.oracle_out(big), what=f"launch whose slot is taken over, rep {rep}")
+            ya.fill_(0x7FC0)
             torch.cuda.synchronize()
+    finally:
+        mg.lib.moe_test_shift_launch_number(2 * slots)   # past every stamp written above
 
 
 def test_gemm_int4_group_size_32_and_64():
