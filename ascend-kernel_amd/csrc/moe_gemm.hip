@@ -1476,7 +1476,10 @@ __global__ __launch_bounds__((64 * KernelCfg<FMT, KIND>::WAVES), (KernelCfg<FMT,
             }
         }
         if (sw < fixed) {
-            T = sw * sweep + vid;
+            // (the last, partial sweep of a launch without a counter goes to the workgroups in launch order, i.e.
+            // round-robin over the XCDs and to different CUs first, not to the first XCDs' workgroups only: where two
+            // workgroups share a CU the tiles per CU, which is what its time follows, then differ by at most one)
+            T = sw * sweep + ((sw + 1) * sweep > total ? (int)blockIdx.x : vid);
             if (T >= total) break;
         }
         // from the last tile of the fixed order on, the k-split tile routines draw the next ticket themselves
