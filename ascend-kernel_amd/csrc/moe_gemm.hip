@@ -14,8 +14,10 @@
 // workgroup from a work counter (see tile_queue).  Every wavefront owns its columns for ALL
 // rows of the tile, so each weight element is dequantized exactly once per tile.  Two tile routines:
 //   gemm_tile_pair  every quantized container (int4, int8, the K-contiguous fp4 containers, the
-//                   reference's fp4 and fp8): 8 wavefronts, the two of a SIMD split the k range;
-//                   x, packed weights and scales arrive by LDS-direct loads into a ring of stages;
+//                   reference's fp4 and fp8); x, packed weights and scales arrive by LDS-direct loads into a
+//                   ring of stages walked by an unrolled k loop.  Either 8 wavefronts, the two of a SIMD
+//                   splitting the k range (int8, fp8, K-contiguous fp4), or 4 wavefronts that each take their
+//                   64 columns through all of k, two such workgroups per CU (int4 and fp4 prefill);
 //                   tiles of up to 160 rows, or of up to 32 / 16 rows with small stages (decode batches,
 //                   and the GEMV op's arithmetic on the N-contiguous containers)
 //   gemm_tile       the bf16 container: 4 wavefronts of 64 columns, x through a double-buffered,
