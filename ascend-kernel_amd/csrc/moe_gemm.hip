@@ -73,12 +73,12 @@ struct GemmParams {
 //
 // A launch owns one slot = one 64-bit counter.  The host numbers the launches (64 bits, never reused); launch L
 // uses slot L % GM_QUEUE_SLOTS and the stamp (L / GM_QUEUE_SLOTS + 1) << GM_QUEUE_COUNT_BITS, which grows with
-// every use of the slot.  Every workgroup raises the counter to the stamp when it starts (atomic max, fire and
-// forget, long before its first draw); a draw is a fetch-and-add, and the value it returns minus the stamp is
-// the ticket.  Whatever an earlier launch left in the slot is smaller than the stamp and simply disappears, so
+// every use of the slot.  The first workgroups raise the counter to the stamp when they start (atomic max, fire and
+// forget, one tile's time before anybody's first draw); a draw is a fetch-and-add, and the value it returns minus
+// the stamp is the ticket.  Whatever an earlier launch left in the slot is smaller than the stamp and simply disappears, so
 // nothing has to be cleared at the end of a kernel and no state a kernel leaves behind can mislead a later one.
 // A launch that only starts after a later launch has taken its slot (its stream was held back for
-// GM_QUEUE_SLOTS launches) sees that from the counter, which it reads once behind its stamp, and never draws:
+// GM_QUEUE_SLOTS launches) sees that from the counter, which every workgroup reads once when it starts, and never draws:
 // it walks all of its tiles in the fixed order and disturbs nobody.  A draw that returns a value outside
 // [stamp, stamp + 2^GM_QUEUE_COUNT_BITS) means that the slot was taken over while this launch was running: the
 // workgroup then walks its share of the tail in the fixed order -- tiles that were already handed out get
@@ -95,13 +95,17 @@ typedef unsigned long long queue_word_t;
 __device__ queue_word_t tile_queue[GM_QUEUE_SLOTS * GM_QUEUE_STRIDE];
 static std::atomic<uint64_t> queue_launches{0};   // launches of every kind of kernel in this file, for slot and stamp
 
-// Raises the counter to the launch's stamp and tells whether the slot is (still) this launch's.  The read is an
-// ordinary load behind the atomic, not the atomic's own return value: that came back 2.5 us later than the
-// group_list loads the caller waits for anyway.
-__device__ __forceinline__ bool queue_stamp(queue_word_t* q, queue_word_t stamp) {
-    (void)__hip_atomic_fetch_max(q, stamp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+// What a workgroup does with the launch's counter when it starts: it reads it (an ordinary load, issued ahead of the
+// group_list loads and back with them) to see whether the slot is still this launch's, and the first 8 workgroups,
+// one per XCD, raise it to the launch's stamp.  Not every workgroup: 512 atomics on one address at the start of a
+// kernel held everybody's first loads up (tile table ready after 8 us instead of 2), and an atomic's own return
+// value came back 2.5 us behind the loads.  A workgroup that draws before any of those stamps has arrived (it
+// cannot be the usual case: draws start one tile into the kernel) gets a value below the stamp, takes it for a lost
+// slot and does its share in the fixed order.
+__device__ __forceinline__ bool queue_open(queue_word_t* q, queue_word_t stamp, bool stamps) {
     const queue_word_t now = __hip_atomic_load(q, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    return now - stamp < (1ull << GM_QUEUE_COUNT_BITS);
+    if (stamps) (void)__hip_atomic_fetch_max(q, stamp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return now < stamp + (1ull << GM_QUEUE_COUNT_BITS);   // else: a later launch holds the slot
 }
 // A draw adds 1 to the counter's low word only (the count never carries out of it) and gets that word back: one
 // register in flight instead of two in the tile routines, which have none to spare.  The word still shows the
@@ -1387,8 +1391,8 @@ __global__ __launch_bounds__((64 * KernelCfg<FMT, KIND>::WAVES), (KernelCfg<FMT,
         return max(hi - first, 0);
     };
 
-    // the launch's counter is raised to its stamp now, long before the first draw from it
-    if (tid == 0) part[PART_FIXED] = P.slot >= 0 && queue_stamp(tile_queue + GM_QUEUE_STRIDE * max(P.slot, 0), P.stamp);
+    // the launch's counter is looked at, and raised to the launch's stamp, now: long before the first draw from it
+    if (tid == 0) part[PART_FIXED] = P.slot >= 0 && queue_open(tile_queue + GM_QUEUE_STRIDE * max(P.slot, 0), P.stamp, blockIdx.x < 8);
 
     // exclusive scan of tiles per expert: each thread takes a contiguous run of experts
     const int per = (P.G + THREADS - 1) / THREADS;
@@ -1450,7 +1454,9 @@ __global__ __launch_bounds__((64 * KernelCfg<FMT, KIND>::WAVES), (KernelCfg<FMT,
     // routines; GM_NO_QUEUE: a launch without counters (captured into a HIP graph, or one whose slot a later launch
     // holds by now) walks every tile in the fixed order, sweep after sweep until the tile number passes the last.
     constexpr int GM_NO_QUEUE = 0x7fffffff;
-    if (tid == 0) part[PART_FIXED] = part[PART_FIXED] ? max(0, total / sweep - GM_QUEUE_TAIL_SWEEPS) : GM_NO_QUEUE;
+    // (at least one sweep in the fixed order before the first draw, so that the stamp is there by then; launches of
+    // at most one tile per workgroup have nothing to balance)
+    if (tid == 0) part[PART_FIXED] = part[PART_FIXED] && total > sweep ? max(1, total / sweep - GM_QUEUE_TAIL_SWEEPS) : GM_NO_QUEUE;
     __syncthreads();
 
     bool have_ticket = false;   // the previous tile routine left its ticket in part[0]
