@@ -733,8 +733,7 @@ __device__ __forceinline__ void gemm_tile_pair(const GemmParams& P, u32x4_t* sme
     const rsrc_t rs8 = make_rsrc(static_cast<const float*>(P.scale) + (int64_t)g * (P.K >> 7) * (P.N >> 7),
                                  (int64_t)(P.K >> 7) * (P.N >> 7) * 4);
     const int cs8 = ((n0 + 64 * cw) >> 7) * 4;
-    // 32-k sub-steps per scale group, and sub-step -> scale row as a multiply (both worked out on the host)
-    const uint32_t per = (B8 || KC) ? 1u : P.sub_per_group;
+    // sub-step -> scale row as a multiply (worked out on the host from the 32-k sub-steps per scale group)
     const uint32_t gmul = (B8 || KC) ? 0u : P.sub_to_group;
     auto scale_row = [&](uint32_t sub) { return gmul ? (int)__umulhi(sub, gmul) : (int)sub; };
     // x rows through a buffer resource that ends after the last valid row (padded rows read as
