@@ -58,8 +58,9 @@ struct GemmParams {
     // first tiles only (the row bounds are read from group_list per tile); 0 neither fits: the first tile of every
     // thread's run of experts only, and a tile is found by walking its run (any number of experts)
     int table_mode;
-    uint32_t sub_per_group;   // 32-k sub-steps per scale group of the N-contiguous 4-bit containers ...
-    uint32_t sub_to_group;    // ... and the multiplier that turns a sub-step index into its scale row (0: identity)
+    // N-contiguous 4-bit containers: the multiplier that turns a 32-k sub-step index into its scale row, i.e.
+    // divides by the sub-steps per scale group (0: identity)
+    uint32_t sub_to_group;
 };
 
 // Work queue of the persistent grid.  Workgroups do not run at one speed (of two that share a CU the one
@@ -1677,8 +1678,7 @@ static GemmParams gemm_params(const moe_grouped_args* a) {
     P.stamp = 0;
     P.table_mode = 0;
     const uint32_t per = a->scale_rows > 0 ? (uint32_t)((a->K / a->scale_rows) >> 5) : 1u;
-    P.sub_per_group = per ? per : 1u;
-    P.sub_to_group = P.sub_per_group == 1 ? 0u : 0xffffffffu / P.sub_per_group + 1u;
+    P.sub_to_group = per <= 1 ? 0u : 0xffffffffu / per + 1u;
     return P;
 }
 
