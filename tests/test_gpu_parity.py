@@ -460,6 +460,44 @@ def test_any_number_of_experts(fmt, op, G, style):
     assert (got[gl[-1]:] == 0x7FC0).all()
 
 
+@pytest.mark.parametrize("fmt,tiles", [("int4", 511), ("int4", 512), ("int4", 513), ("int4", 1023), ("int4", 1025), ("int4", 1537),
+                                       ("int8", 255), ("int8", 257), ("int8", 513), ("int8", 769)])
+def test_tile_counts_around_the_grid_size(fmt, tiles):
+    """The persistent grid is 512 workgroups for the 4-wavefront kind (int4 prefill) and 256 for the 8-wavefront kind
+    (int8) on a 256-CU part.  Launches of at most one tile per workgroup use no tile counter, larger ones run at least
+    one sweep in the fixed order before the first draw, and a launch without a counter deals its last, partial sweep out
+    in launch order: tile counts on either side of one, two and three sweeps, eagerly and replayed from a graph."""
+    _say(f"tile counts around the grid size: {fmt} {tiles} tiles")
+    G = tiles                                            # one 16-row chunk x one 256-column tile per expert
+    gl = list(16 * np.arange(1, G + 1))                  # 16 rows per expert: more than 12 on average, so the prefill kinds run
+    case = H.make_case(fmt, G, 128, 256, gl, seed=tiles, group=32, extra_rows=2)
+    dev = H.upload(case)
+    ref = H.oracle_out(case)
+    got = H.run_cabi(case, dev, "gemm")
+    H.assert_close(got, ref, rows=slice(0, gl[-1]), what=f"{fmt} {tiles} tiles, eager")
+    assert (got[gl[-1]:] == 0x7FC0).all()
+    # the same launch captured (no counter: every tile in the fixed order) and replayed twice
+    import moe_gfx950 as mg
+    p = lambda t: 0 if t is None else t.data_ptr()
+    y = torch.full((case["M"], case["N"]), 0x7FC0, dtype=torch.int16, device="cuda")
+    args = mg.grouped_args(mg.format_from_compute_type(fmt), p(dev["x"]), p(dev["weight"]), p(dev["scale"]), p(dev["offset"]),
+                           p(dev["group_list"]), p(y), case["M"], case["K"], case["N"], case["G"], case["scale_rows"])
+    st = torch.cuda.Stream()
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(st):
+        with torch.cuda.graph(g, stream=st):
+            mg.grouped_gemm(args, st.cuda_stream)
+    for rep in range(2):
+        y.fill_(0x7FC0)
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        got = y.cpu().numpy().view(np.uint16)
+        H.assert_close(got, ref, rows=slice(0, gl[-1]), what=f"{fmt} {tiles} tiles, replay {rep}")
+        assert (got[gl[-1]:] == 0x7FC0).all()
+
+
 def test_gemv_reference_fp8_test_shape_via_module():
     """test_group_soft_gemv_fp8.py:37-88: G=4, M=4, K=512, N=1536, x = ones, expected value
     from fp32 (un-rounded) weights, rtol 0.02."""
