@@ -45,6 +45,24 @@ def _launch(op, fmt, x, w, s, o, gl, y, scale_rows=1):
     torch.cuda.synchronize()
 
 
+def _replayed(op, fmt, x, w, s, o, gl, y, scale_rows=1):
+    """The same call captured into a HIP graph (no tile counter: every tile in the fixed order) and replayed into y."""
+    import moe_gfx950 as mg
+
+    p = lambda t: 0 if t is None else t.data_ptr()
+    K, N = x.shape[1], y.shape[1]
+    args = mg.grouped_args(mg.format_from_compute_type(fmt), p(x), p(w), p(s), p(o), p(gl), p(y), x.shape[0], K, N,
+                           gl.shape[0], scale_rows)
+    st = torch.cuda.Stream()
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(st):
+        with torch.cuda.graph(g, stream=st):
+            (mg.grouped_gemm if op == "gemm" else mg.grouped_gemv)(args, st.cuda_stream)
+    g.replay()
+    torch.cuda.synchronize()
+
+
 def _oracle_subset(fmt, x, w, s, o, counts, experts, gemv=False):
     """Oracle output for the rows of the chosen experts only (a reduced problem built from the
     device tensors): returns (row indices into the full problem, bf16 bits [rows, N])."""
@@ -116,6 +134,10 @@ def test_dsv3_int4_prefill_gate_up_and_down():
         y2 = torch.empty_like(y)
         _launch("gemm", "int4", x, w, s, None, gl, y2, K // 128)
         assert torch.equal(y[:M].view(torch.int16), y2[:M].view(torch.int16))
+        # the order of the tiles does not enter the results: replayed from a graph (fixed order, no work counter)
+        y2.fill_(float("nan"))
+        _replayed("gemm", "int4", x, w, s, None, gl, y2, K // 128)
+        assert torch.equal(y[:M].view(torch.int16), y2[:M].view(torch.int16)) and torch.isnan(y2[M:]).all()
         _launch("gemm", "int4", (x.float() * 2).to(torch.bfloat16), w, s, None, gl, y2, K // 128)
         assert torch.equal((y[:M].float() * 2), y2[:M].float())
         del x, w, s, y, y2
@@ -232,6 +254,10 @@ def test_decode_batch_on_the_n_contiguous_containers(fmt):
         assert torch.isfinite(y[:M].float()).all()
         rows, ref = _oracle_subset(fmt, x, w, s, None, counts, experts, gemv=op == "gemv")
         H.assert_close(H.bits(y[rows.cuda()]), ref, what=f"{fmt} {op} vs oracle")
+        y2 = torch.full_like(y, float("nan"))
+        _replayed(op, fmt, x, w, s, None, gl, y2, scale_rows=srows)
+        assert torch.equal(y[:M].view(torch.int16), y2[:M].view(torch.int16)) and torch.isnan(y2[M:]).all(), "graph replay differs"
+        del y2
         ys[op] = y[:M]
     # the ops differ by the rounding of the weights to bf16 (2^-9 per weight, summed over K = 7168): small against
     # the largest outputs, not against every single one
