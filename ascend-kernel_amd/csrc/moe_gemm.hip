@@ -1694,13 +1694,20 @@ static int launch_gemm_fmt(const moe_grouped_args* a, hipStream_t stream) {
         // 531 vs 549 us and 512 vs 609 us).  The one-byte containers gain nothing from it.
         if constexpr (FMT == MOE_FMT_INT4 || FMT == MOE_FMT_FP4_REF)
             if (a->M <= 12 * a->G) return launch_gemm_kind<FMT, GK_PAIR_SMALL>(P, a, stream);
-        // prefill on the 4-bit N-contiguous containers: workgroups of 4 wavefronts without the k split, two per CU
-        // (256 experts of 128 rows, K = 7168, N = 4096: int4 1792 against 1905 us, fp4 1724 against 1867 us with the
-        // k-split kind; the one-byte containers, whose tiles move twice the bytes, are 2 % slower that way: int8 1081
-        // against 1058 us, fp8 1110 against 1081 us on 128 experts, and stay on the k-split kind)
-        if constexpr (FMT == MOE_FMT_INT4 || FMT == MOE_FMT_FP4_REF) {
-            const int rc = launch_gemm_kind<FMT, GK_QUAD>(P, a, stream);
-            if (rc != MOE_ERR_TOO_LARGE) return rc;   // (more experts than its half of the LDS holds a table for)
+        // prefill on the N-contiguous containers: workgroups of 4 wavefronts without the k split, two per CU.  The 4-bit
+        // ones always (256 experts of 128 rows, K = 7168, N = 4096: int4 1792 against 1905 us, fp4 1724 against 1867 us
+        // with the k-split kind).  The one-byte ones, whose tiles move twice the bytes, when an expert has more rows than
+        // one tile takes on average, so that its row chunks share a weight slice in L2: 8 experts of 512 rows, K = 4096,
+        // N = 14336: int8 454 against 476 us, fp8 480 against 495 us; 64 experts of 512 rows at K = 7168, N = 4096: 1755
+        // against 1870 us and 1872 against 1929 us; but with 128 rows per expert, every weight tile read once from HBM,
+        // 1090 - 1110 against 1063 - 1098 us (int8) and 1125 - 1152 against 1088 - 1136 us (fp8) on 128 experts
+        constexpr bool four_bit = FMT == MOE_FMT_INT4 || FMT == MOE_FMT_FP4_REF;
+        constexpr bool one_byte = FMT == MOE_FMT_INT8 || FMT == MOE_FMT_FP8_REF;
+        if constexpr (four_bit || one_byte) {
+            if (four_bit || a->M > (int64_t)(16 * PAIR_CAPB) * a->G) {
+                const int rc = launch_gemm_kind<FMT, GK_QUAD>(P, a, stream);
+                if (rc != MOE_ERR_TOO_LARGE) return rc;
+            }
         }
         return launch_gemm_kind<FMT, GK_PAIR>(P, a, stream);
     } else {

@@ -181,7 +181,20 @@ def build_dsv3_int4_prefill(torch, mg, gen):
 EXTRA = ("dequant", "prepack", "route", "gemv_bf16", "gemm_int8", "fused_fp4", "reference_containers")
 
 
-def run_extra(torch, mg, gen, iters, warmup, only=None):
+def settle(torch, fn, ms):
+    """Runs fn untimed for about ms milliseconds of queued launches: a matrix-bound kernel that follows a light
+    phase is measured at the clocks the board settles to under it, not while they are still moving (measured on
+    the int8 workload: 565 us per launch in the first 20 launches after a pause, 475 us from the 40th on)."""
+    if ms <= 0:
+        return
+    t0 = time.perf_counter()
+    while (time.perf_counter() - t0) * 1e3 < ms:
+        for _ in range(20):
+            fn()
+        torch.cuda.synchronize()
+
+
+def run_extra(torch, mg, gen, iters, warmup, only=None, settle_ms=0.0):
     """The other benchmark configurations; `only` names one of EXTRA to run just that one (for profiles that
     must hold a single workload's kernels)."""
     out = {}
@@ -195,9 +208,9 @@ def run_extra(torch, mg, gen, iters, warmup, only=None):
     if want("gemv_bf16"):
         out.update(extra_gemv_bf16(torch, mg, gen, iters, warmup))
     if want("gemm_int8"):
-        out.update(extra_gemm_int8(torch, mg, iters, warmup))
+        out.update(extra_gemm_int8(torch, mg, iters, warmup, settle_ms))
     if want("fused_fp4") or want("reference_containers"):
-        out.update(extra_decode_256e(torch, mg, gen, iters, warmup, fused=want("fused_fp4"), ref=want("reference_containers")))
+        out.update(extra_decode_256e(torch, mg, gen, iters, warmup, fused=want("fused_fp4"), ref=want("reference_containers"), settle_ms=settle_ms))
     return out
 
 
@@ -309,7 +322,7 @@ def extra_gemv_bf16(torch, mg, gen, iters, warmup):
     return out
 
 
-def extra_gemm_int8(torch, mg, iters, warmup):
+def extra_gemm_int8(torch, mg, iters, warmup, settle_ms=0.0):
     out = {}
     # c3: int8 antiquant grouped GEMM, 8 experts, multinomial 4096 rows, K=4096, N=14336
     G, M, K, N = 8, 4096, 4096, 14336
@@ -321,6 +334,7 @@ def extra_gemm_int8(torch, mg, iters, warmup):
     o = bf16_uniform(torch, (G, N), -2.0, 2.0)
     y = torch.empty(M, N, dtype=torch.bfloat16, device="cuda")
     op = Op(mg, torch, "gemm", "int8", x, w, s, o, gl, y)
+    settle(torch, op, settle_ms / 2)
     t, = time_launches(torch, [op], iters, warmup)
     fl = 2.0 * M * K * N
     out["grouped_gemm_int8_8e"] = dict(flops=fl, us=t * 1e6, TFLOPs=fl / t / 1e12,
@@ -329,7 +343,7 @@ def extra_gemm_int8(torch, mg, iters, warmup):
     return out
 
 
-def extra_decode_256e(torch, mg, gen, iters, warmup, fused=True, ref=True):
+def extra_decode_256e(torch, mg, gen, iters, warmup, fused=True, ref=True, settle_ms=0.0):
     out = {}
     stream = lambda: torch.cuda.current_stream().cuda_stream
     run_fused, run_ref = fused, ref
@@ -342,13 +356,13 @@ def extra_decode_256e(torch, mg, gen, iters, warmup, fused=True, ref=True):
     x = bf16_normal(torch, (M, K))
     y = torch.empty(M, N, dtype=torch.bfloat16, device="cuda")
     if run_fused:
-        out.update(decode_fused_fp4(torch, mg, iters, warmup, G, K, N, M, A, x, gl, y))
+        out.update(decode_fused_fp4(torch, mg, iters, warmup, G, K, N, M, A, x, gl, y, settle_ms))
     if run_ref:
-        out.update(decode_reference_containers(torch, mg, iters, warmup, G, K, N, M, A, x, gl, y))
+        out.update(decode_reference_containers(torch, mg, iters, warmup, G, K, N, M, A, x, gl, y, settle_ms))
     return out
 
 
-def decode_fused_fp4(torch, mg, iters, warmup, G, K, N, M, A, x, gl, y):
+def decode_fused_fp4(torch, mg, iters, warmup, G, K, N, M, A, x, gl, y, settle_ms=0.0):
     out = {}
     stream = lambda: torch.cuda.current_stream().cuda_stream
     w = torch.randint(0, 256, (G, N, K // 2), dtype=torch.uint8, device="cuda")
@@ -363,6 +377,7 @@ def decode_fused_fp4(torch, mg, iters, warmup, G, K, N, M, A, x, gl, y):
     sep = Op(mg, torch, "gemm", "bf16", x, wd, None, None, gl, y2)
     y3 = torch.empty(M, N, dtype=torch.bfloat16, device="cuda")
     gemv = Op(mg, torch, "gemv", "fp4_b32", x, w, s, None, gl, y3)   # same kernel with the GEMV op's fp32 weights
+    settle(torch, lambda: (fused(), gemv()), settle_ms / 4)
     t_f, t_d, t_s, t_v = time_launches(torch, [fused, dq_all, sep, gemv], max(iters // 2, 5), warmup)
     nbytes = A * (N * K // 2 + N * (K // 32) * 2) + M * K * 2 + M * N * 2
     diff = float((y.float() - y2.float()).abs().max())
@@ -376,7 +391,7 @@ def decode_fused_fp4(torch, mg, iters, warmup, G, K, N, M, A, x, gl, y):
     return out
 
 
-def decode_reference_containers(torch, mg, iters, warmup, G, K, N, M, A, x, gl, y):
+def decode_reference_containers(torch, mg, iters, warmup, G, K, N, M, A, x, gl, y, settle_ms=0.0):
     out = {}
     # the same decode batch on the reference's own containers (N-contiguous: pre-shuffled fp4 with per-16
     # scales, fp8 with 128 x 128 block scales) and on int4 group-128, through both ops
@@ -392,6 +407,7 @@ def decode_reference_containers(torch, mg, iters, warmup, G, K, N, M, A, x, gl, 
             s = bf16_uniform(torch, sshape, 2.0 ** -8, 2.0 ** -2)
         w = w.view(torch.int8) if fmt == "fp4" else w
         ops = [Op(mg, torch, kind, fmt, x, w, s, None, gl, y, scale_rows=srows) for kind in ("gemv", "gemm")]
+        settle(torch, lambda: (ops[0](), ops[1]()), settle_ms / 4)
         t_v, t_m = time_launches(torch, ops, max(iters // 2, 5), warmup)
         nbytes = A * wbytes + M * K * 2 + M * N * 2
         ref[fmt] = dict(bytes=nbytes, gemv_op_us=t_v * 1e6, gemv_op_frac_hbm=nbytes / t_v / 1e9 / PEAK_HBM_GBS,
@@ -589,7 +605,7 @@ def main():
         del src, dst
 
     if args.only in EXTRA:
-        print(json.dumps({"only": args.only, "workloads": run_extra(torch, mg, gen, max(args.steps, 20), args.warmup, only=args.only)}),
+        print(json.dumps({"only": args.only, "workloads": run_extra(torch, mg, gen, max(args.steps, 20), args.warmup, only=args.only, settle_ms=args.settle_ms)}),
               flush=True)
         return
     if args.only == "headline":
@@ -676,7 +692,7 @@ def main():
         "board": board,
     }
     if not args.no_extra:
-        result["workloads"] = run_extra(torch, mg, gen, max(args.steps, 20), args.warmup)
+        result["workloads"] = run_extra(torch, mg, gen, max(args.steps, 20), args.warmup, settle_ms=args.settle_ms)
         result["workloads"]["gate_up_swiglu_fused"] = fused
         torch.cuda.empty_cache()
     if not args.no_cpu:

@@ -498,6 +498,21 @@ def test_tile_counts_around_the_grid_size(fmt, tiles):
         assert (got[gl[-1]:] == 0x7FC0).all()
 
 
+@pytest.mark.parametrize("fmt,N", [("int8", 512), ("fp8", 512), ("fp8", 384)])
+def test_one_byte_containers_with_many_rows_per_expert(fmt, N):
+    """int8 and the reference's fp8 run on the 4-wavefront kind (two workgroups per CU, no k split) once an expert has
+    more rows than one tile takes on average: every row-block count of its tiles, several row chunks per expert, empty
+    experts, ragged last blocks, and for fp8 a half-empty last column tile."""
+    _say(f"{fmt} N={N} on the 4-wavefront kind")
+    counts = [400, 0, 333, 161, 170, 529, 16, 1, 320, 200, 0, 145, 159, 160, 97]
+    gl = list(np.cumsum(counts))
+    assert gl[-1] > 160 * len(gl)
+    case = H.make_case(fmt, len(gl), 512, N, gl, seed=31 + N, extra_rows=3)
+    got = H.run_cabi(case, H.upload(case), "gemm")
+    H.assert_close(got, H.oracle_out(case), rows=slice(0, gl[-1]), what=f"{fmt} N={N}, many rows per expert")
+    assert (got[gl[-1]:] == 0x7FC0).all()
+
+
 def test_gemv_reference_fp8_test_shape_via_module():
     """test_group_soft_gemv_fp8.py:37-88: G=4, M=4, K=512, N=1536, x = ones, expected value
     from fp32 (un-rounded) weights, rtol 0.02."""

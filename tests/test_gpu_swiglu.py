@@ -79,6 +79,21 @@ def test_swiglu_fp8_half_empty_last_tile():
     assert (got[gl[-1]:] == 0x7FC0).all(), "rows beyond group_list[-1] were written"
 
 
+@pytest.mark.parametrize("fmt,N", [("int8", 512), ("fp8", 512), ("fp8", 384)])
+def test_swiglu_one_byte_containers_with_many_rows_per_expert(fmt, N):
+    """The fused activation on the 4-wavefront kind as the one-byte containers use it (more than 160 rows per expert on
+    average)."""
+    _say(f"swiglu {fmt} N={N}, many rows per expert")
+    counts = [400, 0, 333, 161, 170, 529, 16, 1, 320, 200]
+    gl = list(np.cumsum(counts))
+    case = H.make_case(fmt, len(gl), 256, N, gl, seed=9 + N, extra_rows=2)
+    if fmt == "int8":
+        case["x"] = oracle.f32_to_bf16_bits(oracle.bf16_bits_to_f32(case["x"]) * 4.0)
+    got = _run(case)
+    H.assert_close(got, _expected(case), rows=slice(0, gl[-1]), what=f"swiglu {fmt} N={N}")
+    assert (got[gl[-1]:] == 0x7FC0).all(), "rows beyond group_list[-1] were written"
+
+
 def test_swiglu_int4_prefill_tile_sizes():
     """Every row-block count of the int4 prefill kernel (1..10 blocks of 16 rows) and ragged last blocks."""
     _say("swiglu int4 tile sizes")
