@@ -54,7 +54,7 @@ extern "C" {
 typedef void *moe_stream_t;
 
 /* Experts per call of either grouped op.  (moe_grouped_gemm keeps a table of G + 1 tile counts in LDS next to its
- * tile buffers while that fits -- about 1000 to 2000 experts, depending on the container -- and beyond that one
+ * tile buffers while that fits -- about 2500 to 5300 experts, depending on the kernel -- and beyond that one
  * entry per thread, walking group_list for the rest: any count works, small ones are faster.) */
 #define MOE_GEMM_MAX_EXPERTS 65535
 
